@@ -1,0 +1,161 @@
+/*
+ * gs355 -- C ABI of the MI355X (gfx950) forward rasterizer for 3D Gaussian
+ * splatting.
+ *
+ * This library replaces the native extension behind the reference's Python
+ * package `opt_gaussian_rasterization` (third-party CUDA submodule, empty in
+ * the reference tree: .gitmodules:1-4).  The reference binds it through a
+ * torch C++ extension; the entry points below are what that binding calls for
+ * this path, restated as plain C:
+ *
+ *   GaussianRasterizer.forward(...)         -> gs355_render / gs355_run
+ *       call sites: benchmarks/nerf/origin_gs/gs_model.py:211-220,
+ *                   benchmarks/nerf/scaffold_gs/gs_model.py:218-227,
+ *                   benchmarks/nerf/octree_gs/gs_model.py:306-315
+ *   GaussianRasterizer.visible_filter(...)  -> gs355_visible_filter
+ *       call sites: origin_gs/gs_model.py:327-329, scaffold_gs/gs_model.py:
+ *                   432-434, octree_gs/gs_model.py:491-493
+ *   GaussianRasterizationSettings(...)      -> gs355_frame
+ *       built at:   origin_gs/gs_model.py:148-161 (and the two siblings)
+ *
+ * Rules of the boundary
+ *   - extern "C", plain pointers and sizes; no torch, pybind or C++ types.
+ *   - Every device buffer (inputs, outputs, workspace) is owned by the caller;
+ *     the library allocates no device memory and keeps no pointer after return.
+ *   - Work is enqueued on the stream passed in (a hipStream_t cast to void*;
+ *     NULL = the default stream).  No call synchronises the device.
+ *   - Return 0 on success, a negative gs355_status otherwise;
+ *     gs355_last_error() gives the message of the calling thread's last error.
+ *     Argument validation happens before any HIP call, so every GS355_EINVAL /
+ *     GS355_ENOSPC is reachable on a machine without a GPU.
+ *   - All tensors are contiguous fp32 (int32 for radii) in device memory.
+ */
+#ifndef GS355_H
+#define GS355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GS355_VERSION 1
+#define GS355_API __attribute__((visibility("default")))
+#define GS355_TILE 16 /* tile edge in pixels */
+
+typedef enum gs355_status {
+    GS355_OK = 0,
+    GS355_EINVAL = -1,    /* bad argument (null pointer, bad size, exclusive inputs violated) */
+    GS355_ENOSPC = -2,    /* workspace smaller than gs355_workspace_layout() requires */
+    GS355_EOVERFLOW = -3, /* P, the image or the key capacity exceed the 32-bit ranges the kernels index with */
+    GS355_EHIP = -4       /* a HIP runtime call failed */
+} gs355_status;
+
+/* Per-frame record: the fields of GaussianRasterizationSettings.  The four
+ * tensors stay where the reference keeps them (device memory, after
+ * `camera.cuda()`), so no host read-back is needed per frame.  `prefiltered`
+ * and `debug` of the reference's record have no effect on results and are not
+ * part of the ABI. */
+typedef struct gs355_frame {
+    int32_t image_width, image_height;
+    float tanfovx, tanfovy;
+    float scale_modifier;
+    int32_t sh_degree;       /* active SH degree, 0..3 */
+    int32_t sh_coeffs;       /* coefficient rows M of `shs` ([P,M,3]); >= (sh_degree+1)^2 */
+    const float *viewmatrix; /* device f32[16]: torch [4,4] row-major, p_view = [p,1] @ viewmatrix */
+    const float *projmatrix; /* device f32[16]: p_hom = [p,1] @ projmatrix */
+    const float *campos;     /* device f32[3] */
+    const float *bg;         /* device f32[3] */
+} gs355_frame;
+
+/* Inputs of forward(): exactly one of shs / colors_precomp, exactly one of
+ * (scales, rotations) / cov3D_precomp. */
+typedef struct gs355_gaussians {
+    int32_t P;
+    const float *means3D;        /* [P,3] */
+    const float *shs;            /* [P,M,3] or NULL */
+    const float *colors_precomp; /* [P,3] or NULL */
+    const float *opacities;      /* [P] ([P,1] contiguous) */
+    const float *scales;         /* [P,3] or NULL */
+    const float *rotations;      /* [P,4] (r,x,y,z) or NULL */
+    const float *cov3D_precomp;  /* [P,6] (xx,xy,xz,yy,yz,zz) or NULL */
+} gs355_gaussians;
+
+/* Outputs of forward().  image and radii are required for a full render;
+ * depth and alpha may be NULL. */
+typedef struct gs355_outputs {
+    float *image;   /* [3,H,W] */
+    float *depth;   /* [H,W]  sum of depth * alpha * T, or NULL */
+    float *alpha;   /* [H,W]  1 - T_final, or NULL */
+    int32_t *radii; /* [P] */
+} gs355_outputs;
+
+/* Words of the workspace header (u32 unless noted), written by the scan stage. */
+typedef struct gs355_header {
+    uint64_t num_keys_total; /* exact number of (tile, Gaussian) keys the frame needs */
+    uint32_t num_keys;       /* min(num_keys_total, key capacity): what later stages process */
+    uint32_t overflow;       /* 1 if num_keys_total > key capacity (the frame must be redone with more) */
+    uint32_t num_visible;    /* Gaussians with radius > 0 */
+    uint32_t reserved[11];
+} gs355_header;
+
+/* Byte offsets of every array inside the caller's workspace (each 256-byte
+ * aligned).  Tests read intermediates through these. */
+typedef struct gs355_layout {
+    size_t header;        /* gs355_header */
+    size_t records;       /* f32[P][12]: px, py, conic_x, conic_y, conic_z, opacity, r, g, b, depth, 0, 0 */
+    size_t tiles_touched; /* u32[P] */
+    size_t offsets;       /* u32[P]   inclusive prefix sum of tiles_touched */
+    size_t scan_tmp;      /* u32[...] block sums of the scans */
+    size_t keys[2];       /* u64[n_cap] x 2 (ping-pong) */
+    size_t values[2];     /* u32[n_cap] x 2 */
+    size_t sort_hist;     /* u32[...] per-block digit histograms of the radix sort */
+    size_t ranges;        /* u32[tiles][2] */
+    size_t total_bytes;
+    int32_t unsorted_buffer; /* which keys/values buffer the duplicate stage writes (0) */
+    int32_t sorted_buffer;   /* which buffer holds the sorted pairs after the sort stage */
+    int32_t sort_passes;     /* radix passes the sort stage runs for this image size */
+    int32_t sort_bits;       /* significant key bits: 32 + ceil(log2(tiles)) */
+} gs355_layout;
+
+/* Stages of gs355_run, in pipeline order. */
+enum {
+    GS355_STAGE_PREPROCESS = 1, /* per-Gaussian cull / EWA / conic / radius / colour -> records, tiles_touched, radii */
+    GS355_STAGE_SCAN = 2,       /* inclusive scan of tiles_touched -> offsets, header */
+    GS355_STAGE_DUPLICATE = 4,  /* (tile << 32 | depth bits, index) for each tile of each survivor */
+    GS355_STAGE_SORT = 8,       /* stable LSD radix sort of the pairs by key */
+    GS355_STAGE_RANGES = 16,    /* per-tile [first, last) in the sorted keys */
+    GS355_STAGE_BLEND = 32,     /* front-to-back alpha blending per 16x16 tile */
+    GS355_STAGE_ALL = 63
+};
+
+GS355_API int gs355_version(void);
+GS355_API const char *gs355_last_error(void);
+
+/* Workspace the caller must provide for P Gaussians, a key capacity of n_cap
+ * (tile, Gaussian) pairs and a width x height image. */
+GS355_API int gs355_workspace_layout(int32_t P, int64_t n_cap, int32_t width, int32_t height, gs355_layout *out);
+
+/* Run the stages selected in stage_mask (they must be run in pipeline order
+ * over the same workspace; a later call may continue where an earlier one
+ * stopped).  Stages after the scan read the key count from the workspace
+ * header on the device, so no host synchronisation is needed between stages;
+ * if header.overflow is set the results of those stages are to be discarded
+ * and the frame redone with a larger n_cap. */
+GS355_API int gs355_run(const gs355_frame *frame, const gs355_gaussians *g, void *workspace, size_t workspace_bytes,
+              int64_t n_cap, const gs355_outputs *out, uint32_t stage_mask, void *stream);
+
+/* All stages: the body of GaussianRasterizer.forward. */
+GS355_API int gs355_render(const gs355_frame *frame, const gs355_gaussians *g, void *workspace, size_t workspace_bytes,
+                 int64_t n_cap, const gs355_outputs *out, void *stream);
+
+/* GaussianRasterizer.visible_filter: radii only (cull, covariance, radius,
+ * non-empty tile rectangle); needs no workspace.  shs/colors/opacities of
+ * `g` are ignored and may be NULL. */
+GS355_API int gs355_visible_filter(const gs355_frame *frame, const gs355_gaussians *g, int32_t *radii, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GS355_H */

@@ -1,0 +1,127 @@
+"""ctypes binding of libgs355.so (the C ABI declared in include/gs355.h).
+
+The library is built in-tree by `python -m landmarksystem_amd.csrc.build`.
+There is no fallback: if the shared object is missing, loading raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libgs355.so")
+
+GS355_OK, GS355_EINVAL, GS355_ENOSPC, GS355_EOVERFLOW, GS355_EHIP = 0, -1, -2, -3, -4
+
+STAGE_PREPROCESS, STAGE_SCAN, STAGE_DUPLICATE, STAGE_SORT, STAGE_RANGES, STAGE_BLEND = 1, 2, 4, 8, 16, 32
+STAGE_ALL = 63
+
+EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
+           "gs355_visible_filter")
+
+
+class Frame(C.Structure):
+    _fields_ = [
+        ("image_width", C.c_int32),
+        ("image_height", C.c_int32),
+        ("tanfovx", C.c_float),
+        ("tanfovy", C.c_float),
+        ("scale_modifier", C.c_float),
+        ("sh_degree", C.c_int32),
+        ("sh_coeffs", C.c_int32),
+        ("viewmatrix", C.c_void_p),
+        ("projmatrix", C.c_void_p),
+        ("campos", C.c_void_p),
+        ("bg", C.c_void_p),
+    ]
+
+
+class Gaussians(C.Structure):
+    _fields_ = [
+        ("P", C.c_int32),
+        ("means3D", C.c_void_p),
+        ("shs", C.c_void_p),
+        ("colors_precomp", C.c_void_p),
+        ("opacities", C.c_void_p),
+        ("scales", C.c_void_p),
+        ("rotations", C.c_void_p),
+        ("cov3D_precomp", C.c_void_p),
+    ]
+
+
+class Outputs(C.Structure):
+    _fields_ = [("image", C.c_void_p), ("depth", C.c_void_p), ("alpha", C.c_void_p), ("radii", C.c_void_p)]
+
+
+class Header(C.Structure):
+    _fields_ = [
+        ("num_keys_total", C.c_uint64),
+        ("num_keys", C.c_uint32),
+        ("overflow", C.c_uint32),
+        ("num_visible", C.c_uint32),
+        ("reserved", C.c_uint32 * 11),
+    ]
+
+
+class Layout(C.Structure):
+    _fields_ = [
+        ("header", C.c_size_t),
+        ("records", C.c_size_t),
+        ("tiles_touched", C.c_size_t),
+        ("offsets", C.c_size_t),
+        ("scan_tmp", C.c_size_t),
+        ("keys", C.c_size_t * 2),
+        ("values", C.c_size_t * 2),
+        ("sort_hist", C.c_size_t),
+        ("ranges", C.c_size_t),
+        ("total_bytes", C.c_size_t),
+        ("unsorted_buffer", C.c_int32),
+        ("sorted_buffer", C.c_int32),
+        ("sort_passes", C.c_int32),
+        ("sort_bits", C.c_int32),
+    ]
+
+
+class Gs355Error(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__("gs355 error %d: %s" % (code, message))
+        self.code = code
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load libgs355.so once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s is missing: build it with `python -m landmarksystem_amd.csrc.build` "
+            "(there is no non-HIP fallback)" % LIB_PATH
+        )
+    lib = C.CDLL(LIB_PATH)
+    lib.gs355_version.restype = C.c_int
+    lib.gs355_last_error.restype = C.c_char_p
+    lib.gs355_workspace_layout.argtypes = [C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.POINTER(Layout)]
+    lib.gs355_workspace_layout.restype = C.c_int
+    lib.gs355_run.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_void_p, C.c_size_t, C.c_int64,
+                              C.POINTER(Outputs), C.c_uint32, C.c_void_p]
+    lib.gs355_run.restype = C.c_int
+    lib.gs355_render.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_void_p, C.c_size_t, C.c_int64,
+                                 C.POINTER(Outputs), C.c_void_p]
+    lib.gs355_render.restype = C.c_int
+    lib.gs355_visible_filter.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_void_p, C.c_void_p]
+    lib.gs355_visible_filter.restype = C.c_int
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    if rc != GS355_OK:
+        raise Gs355Error(rc, load().gs355_last_error().decode("utf-8", "replace"))
+
+
+def workspace_layout(P: int, n_cap: int, width: int, height: int) -> Layout:
+    L = Layout()
+    check(load().gs355_workspace_layout(int(P), int(n_cap), int(width), int(height), C.byref(L)))
+    return L

@@ -1,0 +1,245 @@
+// Host side of the gs355 C ABI: argument validation, workspace layout and the
+// stage sequence of GaussianRasterizer.forward / .visible_filter (reference
+// call sites: benchmarks/nerf/origin_gs/gs_model.py:211-220, 327-329).
+// Validation runs before any HIP call so that error paths are testable on a
+// machine without a GPU.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "gs355_internal.h"
+
+namespace gs355 {
+
+static thread_local char g_error[512] = "";
+
+int set_error(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+namespace {
+
+constexpr size_t kAlign = 256;
+constexpr int64_t kMaxKeys = (1ll << 32) - 1 - kSortTile;  // key slots are indexed with u32
+
+size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+
+int ceil_log2(uint32_t v)
+{
+    int b = 0;
+    while ((1ull << b) < v) ++b;
+    return b;
+}
+
+int check_dims(int32_t P, int64_t n_cap, int32_t W, int32_t H)
+{
+    if (P < 0) return set_error(GS355_EINVAL, "P must be >= 0 (got %d)", P);
+    if (W <= 0 || H <= 0) return set_error(GS355_EINVAL, "image size must be positive (got %dx%d)", W, H);
+    if (n_cap < 0) return set_error(GS355_EINVAL, "n_cap must be >= 0 (got %lld)", (long long)n_cap);
+    if (n_cap > kMaxKeys)
+        return set_error(GS355_EOVERFLOW, "n_cap %lld exceeds the 32-bit key index range (%lld)", (long long)n_cap,
+                         (long long)kMaxKeys);
+    const int64_t gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+    if (gx * gy > (1ll << 24))
+        return set_error(GS355_EOVERFLOW, "image %dx%d has more than 2^24 tiles", W, H);
+    return GS355_OK;
+}
+
+int make_layout(int32_t P, int64_t n_cap, int32_t W, int32_t H, gs355_layout* L)
+{
+    const int rc = check_dims(P, n_cap, W, H);
+    if (rc) return rc;
+    const size_t tiles = (size_t)((W + kTile - 1) / kTile) * (size_t)((H + kTile - 1) / kTile);
+    const size_t p = (size_t)P, n = (size_t)n_cap;
+    const size_t sort_blocks = (n + kSortTile - 1) / kSortTile;
+    const size_t hist_words = (size_t)kRadix * sort_blocks;
+    size_t tmp_words = scan_tmp_words(p);
+    if (scan_tmp_words(hist_words) > tmp_words) tmp_words = scan_tmp_words(hist_words);
+
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = off;
+        off = align_up(off + (bytes ? bytes : 1));
+        return at;
+    };
+    std::memset(L, 0, sizeof *L);
+    L->header = take(sizeof(gs355_header));
+    L->records = take(p * kRecordFloats * sizeof(float));
+    L->tiles_touched = take(p * sizeof(uint32_t));
+    L->offsets = take(p * sizeof(uint32_t));
+    L->scan_tmp = take(tmp_words * sizeof(uint32_t));
+    L->keys[0] = take(n * sizeof(uint64_t));
+    L->keys[1] = take(n * sizeof(uint64_t));
+    L->values[0] = take(n * sizeof(uint32_t));
+    L->values[1] = take(n * sizeof(uint32_t));
+    L->sort_hist = take(hist_words * sizeof(uint32_t));
+    L->ranges = take(tiles * 2 * sizeof(uint32_t));
+    L->total_bytes = off;
+    L->sort_bits = 32 + ceil_log2((uint32_t)tiles);
+    L->sort_passes = (L->sort_bits + kRadixBits - 1) / kRadixBits;
+    L->unsorted_buffer = 0;
+    L->sorted_buffer = L->sort_passes & 1;
+    return GS355_OK;
+}
+
+int check_frame(const gs355_frame* f, bool need_colour)
+{
+    if (!f) return set_error(GS355_EINVAL, "frame is NULL");
+    if (f->image_width <= 0 || f->image_height <= 0)
+        return set_error(GS355_EINVAL, "image size must be positive (got %dx%d)", f->image_width, f->image_height);
+    if (!f->viewmatrix || !f->projmatrix)
+        return set_error(GS355_EINVAL, "viewmatrix / projmatrix must be device pointers to 16 floats");
+    if (!(f->tanfovx > 0.0f) || !(f->tanfovy > 0.0f))
+        return set_error(GS355_EINVAL, "tanfovx / tanfovy must be positive");
+    if (need_colour) {
+        if (!f->bg) return set_error(GS355_EINVAL, "bg must be a device pointer to 3 floats");
+    }
+    return GS355_OK;
+}
+
+int check_geometry_inputs(const gs355_gaussians* g)
+{
+    if (!g) return set_error(GS355_EINVAL, "gaussians is NULL");
+    if (g->P < 0) return set_error(GS355_EINVAL, "P must be >= 0 (got %d)", g->P);
+    if (g->P == 0) return GS355_OK;
+    if (!g->means3D) return set_error(GS355_EINVAL, "means3D is NULL");
+    const bool has_sr = g->scales != nullptr && g->rotations != nullptr;
+    const bool any_sr = g->scales != nullptr || g->rotations != nullptr;
+    const bool has_cov = g->cov3D_precomp != nullptr;
+    if ((has_sr && has_cov) || (!has_sr && !has_cov) || (any_sr && !has_sr))
+        return set_error(GS355_EINVAL, "Please provide exactly one of either scale/rotation pair or precomputed 3D covariance!");
+    return GS355_OK;
+}
+
+int check_colour_inputs(const gs355_frame* f, const gs355_gaussians* g)
+{
+    if (g->P == 0) return GS355_OK;
+    if ((g->shs != nullptr) == (g->colors_precomp != nullptr))
+        return set_error(GS355_EINVAL, "Please provide excatly one of either SHs or precomputed colors!");
+    if (!g->opacities) return set_error(GS355_EINVAL, "opacities is NULL");
+    if (g->shs) {
+        if (f->sh_degree < 0 || f->sh_degree > 3)
+            return set_error(GS355_EINVAL, "sh_degree must be in [0,3] (got %d)", f->sh_degree);
+        const int need = (f->sh_degree + 1) * (f->sh_degree + 1);
+        if (f->sh_coeffs < need)
+            return set_error(GS355_EINVAL, "shs holds %d coefficients per Gaussian, sh_degree %d needs %d", f->sh_coeffs,
+                             f->sh_degree, need);
+        if (!f->campos) return set_error(GS355_EINVAL, "campos must be a device pointer to 3 floats");
+    }
+    return GS355_OK;
+}
+
+FrameArgs make_args(const gs355_frame* f)
+{
+    FrameArgs a;
+    a.W = f->image_width;
+    a.H = f->image_height;
+    a.grid_x = (a.W + kTile - 1) / kTile;
+    a.grid_y = (a.H + kTile - 1) / kTile;
+    a.tanfovx = f->tanfovx;
+    a.tanfovy = f->tanfovy;
+    a.focal_x = (float)a.W / (2.0f * f->tanfovx);
+    a.focal_y = (float)a.H / (2.0f * f->tanfovy);
+    a.scale_modifier = f->scale_modifier;
+    a.sh_degree = f->sh_degree;
+    a.sh_coeffs = f->sh_coeffs;
+    a.viewmatrix = f->viewmatrix;
+    a.projmatrix = f->projmatrix;
+    a.campos = f->campos;
+    a.bg = f->bg;
+    return a;
+}
+
+}  // namespace
+}  // namespace gs355
+
+using namespace gs355;
+
+extern "C" {
+
+int gs355_version(void) { return GS355_VERSION; }
+
+const char* gs355_last_error(void) { return g_error; }
+
+int gs355_workspace_layout(int32_t P, int64_t n_cap, int32_t width, int32_t height, gs355_layout* out)
+{
+    if (!out) return set_error(GS355_EINVAL, "layout output is NULL");
+    return make_layout(P, n_cap, width, height, out);
+}
+
+int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspace, size_t workspace_bytes,
+              int64_t n_cap, const gs355_outputs* out, uint32_t stage_mask, void* stream)
+{
+    int rc;
+    if ((stage_mask & ~(uint32_t)GS355_STAGE_ALL) != 0 || stage_mask == 0)
+        return set_error(GS355_EINVAL, "stage_mask 0x%x selects no known stage", stage_mask);
+    if ((rc = check_frame(frame, true))) return rc;
+    if ((rc = check_geometry_inputs(g))) return rc;
+    if ((rc = check_colour_inputs(frame, g))) return rc;
+    if (!out) return set_error(GS355_EINVAL, "outputs is NULL");
+    if ((stage_mask & GS355_STAGE_PREPROCESS) && g->P > 0 && !out->radii)
+        return set_error(GS355_EINVAL, "outputs.radii is NULL");
+    if ((stage_mask & GS355_STAGE_BLEND) && !out->image) return set_error(GS355_EINVAL, "outputs.image is NULL");
+    gs355_layout L;
+    if ((rc = make_layout(g->P, n_cap, frame->image_width, frame->image_height, &L))) return rc;
+    if (!workspace) return set_error(GS355_EINVAL, "workspace is NULL");
+    if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
+        return set_error(GS355_EINVAL, "workspace must be 256-byte aligned");
+    if (workspace_bytes < L.total_bytes)
+        return set_error(GS355_ENOSPC, "workspace has %zu bytes, %zu needed (P=%d, n_cap=%lld, %dx%d)", workspace_bytes,
+                         L.total_bytes, g->P, (long long)n_cap, frame->image_width, frame->image_height);
+
+    char* ws = static_cast<char*>(workspace);
+    auto* header = reinterpret_cast<gs355_header*>(ws + L.header);
+    auto* records = reinterpret_cast<float*>(ws + L.records);
+    auto* touched = reinterpret_cast<uint32_t*>(ws + L.tiles_touched);
+    auto* offsets = reinterpret_cast<uint32_t*>(ws + L.offsets);
+    auto* scan_tmp = reinterpret_cast<uint32_t*>(ws + L.scan_tmp);
+    uint64_t* keys[2] = {reinterpret_cast<uint64_t*>(ws + L.keys[0]), reinterpret_cast<uint64_t*>(ws + L.keys[1])};
+    uint32_t* vals[2] = {reinterpret_cast<uint32_t*>(ws + L.values[0]), reinterpret_cast<uint32_t*>(ws + L.values[1])};
+    auto* hist = reinterpret_cast<uint32_t*>(ws + L.sort_hist);
+    auto* ranges = reinterpret_cast<uint32_t*>(ws + L.ranges);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const FrameArgs fa = make_args(frame);
+    const uint32_t cap = (uint32_t)n_cap;
+
+    if (stage_mask & GS355_STAGE_PREPROCESS)
+        if ((rc = launch_preprocess(fa, *g, false, records, touched, out->radii, s))) return rc;
+    if (stage_mask & GS355_STAGE_SCAN)
+        if ((rc = launch_scan_offsets(touched, out->radii, g->P, offsets, scan_tmp, header, cap, s))) return rc;
+    if (stage_mask & GS355_STAGE_DUPLICATE)
+        if ((rc = launch_duplicate(fa, g->P, records, out->radii, offsets, header, keys[0], vals[0], s))) return rc;
+    if (stage_mask & GS355_STAGE_SORT)
+        if ((rc = launch_sort(header, cap, L.sort_passes, keys[0], keys[1], vals[0], vals[1], hist, scan_tmp, s)))
+            return rc;
+    if (stage_mask & GS355_STAGE_RANGES)
+        if ((rc = launch_ranges(header, cap, keys[L.sorted_buffer], ranges, fa.grid_x * fa.grid_y, s))) return rc;
+    if (stage_mask & GS355_STAGE_BLEND)
+        if ((rc = launch_blend(fa, header, ranges, vals[L.sorted_buffer], records, out->image, out->depth, out->alpha,
+                               s)))
+            return rc;
+    return GS355_OK;
+}
+
+int gs355_render(const gs355_frame* frame, const gs355_gaussians* g, void* workspace, size_t workspace_bytes,
+                 int64_t n_cap, const gs355_outputs* out, void* stream)
+{
+    return gs355_run(frame, g, workspace, workspace_bytes, n_cap, out, GS355_STAGE_ALL, stream);
+}
+
+int gs355_visible_filter(const gs355_frame* frame, const gs355_gaussians* g, int32_t* radii, void* stream)
+{
+    int rc;
+    if ((rc = check_frame(frame, false))) return rc;
+    if ((rc = check_geometry_inputs(g))) return rc;
+    if (g->P > 0 && !radii) return set_error(GS355_EINVAL, "radii is NULL");
+    const FrameArgs fa = make_args(frame);
+    return launch_preprocess(fa, *g, true, nullptr, nullptr, radii, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

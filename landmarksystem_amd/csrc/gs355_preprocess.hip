@@ -1,0 +1,284 @@
+// Per-Gaussian preprocess and key duplication for gfx950.
+//
+// Replaces the per-Gaussian stage of the rasterizer behind the reference's
+// GaussianRasterizer.forward / .visible_filter (call sites:
+// benchmarks/nerf/origin_gs/gs_model.py:211-220, 327-329).  The in-tree Python
+// statements of two sub-steps are followed for layout and constants:
+//   SH -> RGB            landmark/nerf_components/utils/sh_utils.py:24-94
+//   scale/quat -> cov3D  landmark/nerf_components/utils/general_utils.py:64-102
+//
+// This translation unit is compiled with -ffp-contract=off: depth bits,
+// radius and the tile rectangle feed the integer pipeline (keys, sort order,
+// ranges), so every expression here is evaluated as unfused IEEE fp32 in the
+// written order, with correctly rounded division and square root.
+#include "gs355_internal.h"
+
+namespace gs355 {
+
+namespace {
+
+constexpr float kShC0 = 0.28209479177387814f;
+constexpr float kShC1 = 0.4886025119029199f;
+constexpr float kShC2[5] = {1.0925484305920792f, -1.0925484305920792f, 0.31539156525252005f,
+                            -1.0925484305920792f, 0.5462742152960396f};
+constexpr float kShC3[7] = {-0.5900435899266435f, 2.890611442640554f, -0.4570457994644658f,
+                            0.3731763325901154f, -0.4570457994644658f, 1.445305721320277f,
+                            -0.5900435899266435f};
+
+struct Rect {
+    int x0, y0, x1, y1;
+};
+
+// min(grid, max(0, (int)v)) with truncation toward zero, defined for any v.
+__device__ __forceinline__ int tile_clamp(float v, int grid)
+{
+    if (!(v > 0.0f)) return 0;
+    if (v >= (float)grid) return grid;
+    return (int)v;
+}
+
+__device__ __forceinline__ Rect tile_rect(float px, float py, int radius, int grid_x, int grid_y)
+{
+    const float r = (float)radius;
+    Rect q;
+    q.x0 = tile_clamp((px - r) / 16.0f, grid_x);
+    q.y0 = tile_clamp((py - r) / 16.0f, grid_y);
+    q.x1 = tile_clamp((px + r + 15.0f) / 16.0f, grid_x);
+    q.y1 = tile_clamp((py + r + 15.0f) / 16.0f, grid_y);
+    return q;
+}
+
+// 3D covariance, packed upper triangle, from scale and (r,x,y,z) quaternion.
+__device__ __forceinline__ void covariance3d(const float* __restrict__ scale, float mod,
+                                             const float* __restrict__ quat, float cov[6])
+{
+    const float sx = mod * scale[0], sy = mod * scale[1], sz = mod * scale[2];
+    const float r = quat[0], x = quat[1], y = quat[2], z = quat[3];
+    // rows of the rotation, each column scaled by its axis length
+    const float l00 = (1.f - 2.f * (y * y + z * z)) * sx, l01 = (2.f * (x * y - r * z)) * sy,
+                l02 = (2.f * (x * z + r * y)) * sz;
+    const float l10 = (2.f * (x * y + r * z)) * sx, l11 = (1.f - 2.f * (x * x + z * z)) * sy,
+                l12 = (2.f * (y * z - r * x)) * sz;
+    const float l20 = (2.f * (x * z - r * y)) * sx, l21 = (2.f * (y * z + r * x)) * sy,
+                l22 = (1.f - 2.f * (x * x + y * y)) * sz;
+    cov[0] = (l00 * l00 + l01 * l01) + l02 * l02;
+    cov[1] = (l00 * l10 + l01 * l11) + l02 * l12;
+    cov[2] = (l00 * l20 + l01 * l21) + l02 * l22;
+    cov[3] = (l10 * l10 + l11 * l11) + l12 * l12;
+    cov[4] = (l10 * l20 + l11 * l21) + l12 * l22;
+    cov[5] = (l20 * l20 + l21 * l21) + l22 * l22;
+}
+
+template <bool kRadiiOnly>
+__global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaussians g,
+                                                         float* __restrict__ records,
+                                                         uint32_t* __restrict__ tiles_touched,
+                                                         int32_t* __restrict__ radii)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= g.P) return;
+
+    const float* __restrict__ V = f.viewmatrix;
+    const float* __restrict__ M = f.projmatrix;
+
+    int radius = 0;
+    uint32_t touched = 0;
+    do {
+        const float x = g.means3D[3 * (size_t)i], y = g.means3D[3 * (size_t)i + 1], z = g.means3D[3 * (size_t)i + 2];
+        const float vx = ((V[0] * x + V[4] * y) + V[8] * z) + V[12];
+        const float vy = ((V[1] * x + V[5] * y) + V[9] * z) + V[13];
+        const float vz = ((V[2] * x + V[6] * y) + V[10] * z) + V[14];
+        if (vz <= 0.2f) break;  // behind or too close to the camera plane
+
+        const float hx = ((M[0] * x + M[4] * y) + M[8] * z) + M[12];
+        const float hy = ((M[1] * x + M[5] * y) + M[9] * z) + M[13];
+        const float hw = ((M[3] * x + M[7] * y) + M[11] * z) + M[15];
+        const float inv_w = 1.0f / (hw + 0.0000001f);
+        const float ndc_x = hx * inv_w, ndc_y = hy * inv_w;
+
+        float cov[6];
+        if (g.cov3D_precomp) {
+#pragma unroll
+            for (int k = 0; k < 6; ++k) cov[k] = g.cov3D_precomp[6 * (size_t)i + k];
+        } else {
+            covariance3d(g.scales + 3 * (size_t)i, f.scale_modifier, g.rotations + 4 * (size_t)i, cov);
+        }
+
+        // EWA splatting: Jacobian of the perspective projection at the
+        // (frustum-clamped) view-space mean, times the world->view rotation.
+        const float lim_x = 1.3f * f.tanfovx, lim_y = 1.3f * f.tanfovy;
+        const float tz = vz;
+        const float tx = fminf(lim_x, fmaxf(-lim_x, vx / tz)) * tz;
+        const float ty = fminf(lim_y, fmaxf(-lim_y, vy / tz)) * tz;
+        const float j00 = f.focal_x / tz, j02 = -(f.focal_x * tx) / (tz * tz);
+        const float j11 = f.focal_y / tz, j12 = -(f.focal_y * ty) / (tz * tz);
+        // a[r][k] = sum_i J[r][i] * Rwv[i][k], Rwv[i][k] = V[4k+i]
+        const float a00 = j00 * V[0] + j02 * V[2], a01 = j00 * V[4] + j02 * V[6], a02 = j00 * V[8] + j02 * V[10];
+        const float a10 = j11 * V[1] + j12 * V[2], a11 = j11 * V[5] + j12 * V[6], a12 = j11 * V[9] + j12 * V[10];
+        // b = a * Sigma
+        const float b00 = (a00 * cov[0] + a01 * cov[1]) + a02 * cov[2];
+        const float b01 = (a00 * cov[1] + a01 * cov[3]) + a02 * cov[4];
+        const float b02 = (a00 * cov[2] + a01 * cov[4]) + a02 * cov[5];
+        const float b10 = (a10 * cov[0] + a11 * cov[1]) + a12 * cov[2];
+        const float b11 = (a10 * cov[1] + a11 * cov[3]) + a12 * cov[4];
+        const float b12 = (a10 * cov[2] + a11 * cov[4]) + a12 * cov[5];
+        // 2D covariance b * a^T with the 0.3 px low-pass on the diagonal
+        const float ca = ((b00 * a00 + b01 * a01) + b02 * a02) + 0.3f;
+        const float cb = (b00 * a10 + b01 * a11) + b02 * a12;
+        const float cc = ((b10 * a10 + b11 * a11) + b12 * a12) + 0.3f;
+
+        const float det = ca * cc - cb * cb;
+        if (det == 0.0f) break;
+        const float det_inv = 1.0f / det;
+        const float mid = 0.5f * (ca + cc);
+        const float disc = sqrtf(fmaxf(0.1f, mid * mid - det));
+        const float lambda1 = mid + disc, lambda2 = mid - disc;
+        const float rf = ceilf(3.0f * sqrtf(fmaxf(lambda1, lambda2)));
+        if (!(rf < 1073741824.0f)) break;  // non-finite or absurd footprint
+        const int rad = (int)rf;
+
+        const float px = ((ndc_x + 1.0f) * (float)f.W - 1.0f) * 0.5f;
+        const float py = ((ndc_y + 1.0f) * (float)f.H - 1.0f) * 0.5f;
+        const Rect q = tile_rect(px, py, rad, f.grid_x, f.grid_y);
+        const int area = (q.x1 - q.x0) * (q.y1 - q.y0);
+        if (area == 0) break;
+
+        radius = rad;
+        touched = (uint32_t)area;
+        if (kRadiiOnly) break;
+
+        float cr, cg, cbl;
+        if (g.colors_precomp) {
+            cr = g.colors_precomp[3 * (size_t)i];
+            cg = g.colors_precomp[3 * (size_t)i + 1];
+            cbl = g.colors_precomp[3 * (size_t)i + 2];
+        } else {
+            const float* __restrict__ sh = g.shs + (size_t)i * f.sh_coeffs * 3;
+            float dx = x - f.campos[0], dy = y - f.campos[1], dz = z - f.campos[2];
+            const float len = sqrtf((dx * dx + dy * dy) + dz * dz);
+            dx = dx / len;
+            dy = dy / len;
+            dz = dz / len;
+            float out[3];
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                float res = kShC0 * sh[c];
+                if (f.sh_degree > 0) {
+                    res = res - kShC1 * dy * sh[3 + c] + kShC1 * dz * sh[6 + c] - kShC1 * dx * sh[9 + c];
+                    if (f.sh_degree > 1) {
+                        const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
+                        const float xy = dx * dy, yz = dy * dz, xz = dx * dz;
+                        res = res + kShC2[0] * xy * sh[12 + c] + kShC2[1] * yz * sh[15 + c] +
+                              kShC2[2] * (2.0f * zz - xx - yy) * sh[18 + c] + kShC2[3] * xz * sh[21 + c] +
+                              kShC2[4] * (xx - yy) * sh[24 + c];
+                        if (f.sh_degree > 2) {
+                            res = res + kShC3[0] * dy * (3.0f * xx - yy) * sh[27 + c] +
+                                  kShC3[1] * xy * dz * sh[30 + c] +
+                                  kShC3[2] * dy * (4.0f * zz - xx - yy) * sh[33 + c] +
+                                  kShC3[3] * dz * (2.0f * zz - 3.0f * xx - 3.0f * yy) * sh[36 + c] +
+                                  kShC3[4] * dx * (4.0f * zz - xx - yy) * sh[39 + c] +
+                                  kShC3[5] * dz * (xx - yy) * sh[42 + c] +
+                                  kShC3[6] * dx * (xx - 3.0f * yy) * sh[45 + c];
+                        }
+                    }
+                }
+                res += 0.5f;
+                out[c] = res < 0.0f ? 0.0f : res;
+            }
+            cr = out[0];
+            cg = out[1];
+            cbl = out[2];
+        }
+
+        float4* __restrict__ rec = reinterpret_cast<float4*>(records + (size_t)i * kRecordFloats);
+        rec[0] = make_float4(px, py, cc * det_inv, -cb * det_inv);
+        rec[1] = make_float4(ca * det_inv, g.opacities[i], cr, cg);
+        rec[2] = make_float4(cbl, vz, 0.0f, 0.0f);
+    } while (false);
+
+    radii[i] = radius;
+    if (!kRadiiOnly) tiles_touched[i] = touched;
+}
+
+// One workgroup expands the keys of 256 consecutive Gaussians.  Output slots
+// are walked by consecutive lanes (coalesced stores); each slot finds its
+// source Gaussian by binary search over the group's offsets held in LDS.
+__global__ __launch_bounds__(256) void duplicate_kernel(FrameArgs f, int32_t P, const float* __restrict__ records,
+                                                        const int32_t* __restrict__ radii,
+                                                        const uint32_t* __restrict__ offsets,
+                                                        const gs355_header* __restrict__ header,
+                                                        uint64_t* __restrict__ keys, uint32_t* __restrict__ values)
+{
+    __shared__ uint32_t s_end[256];    // inclusive offset of each Gaussian of the group
+    __shared__ uint32_t s_depth[256];  // depth bits
+    __shared__ int s_x0[256], s_y0[256], s_w[256];
+
+    if (header->overflow) return;  // capacity too small: the caller redoes the frame
+    const int t = threadIdx.x;
+    const int g0 = blockIdx.x * 256;
+    const int i = g0 + t;
+    const uint32_t begin = g0 == 0 ? 0u : offsets[g0 - 1];
+    uint32_t end_i = begin;
+    if (i < P) {
+        end_i = offsets[i];
+        const int rad = radii[i];
+        if (rad > 0) {
+            const float* rec = records + (size_t)i * kRecordFloats;
+            const Rect q = tile_rect(rec[0], rec[1], rad, f.grid_x, f.grid_y);
+            s_x0[t] = q.x0;
+            s_y0[t] = q.y0;
+            s_w[t] = q.x1 - q.x0;
+            s_depth[t] = __float_as_uint(rec[9]);
+        }
+    }
+    s_end[t] = end_i;  // threads past P repeat `begin`, harmless: never selected
+    __syncthreads();
+    const int last = min(255, P - 1 - g0);
+    const uint32_t end = s_end[last];
+
+    for (uint32_t j = begin + t; j < end; j += 256) {
+        // smallest k with s_end[k] > j
+        int lo = 0, hi = last;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (s_end[mid] > j) hi = mid;
+            else lo = mid + 1;
+        }
+        const uint32_t first = lo == 0 ? begin : s_end[lo - 1];
+        const uint32_t local = j - first;
+        const int w = s_w[lo];
+        const int ty = s_y0[lo] + (int)(local / (uint32_t)w);
+        const int tx = s_x0[lo] + (int)(local % (uint32_t)w);
+        const uint64_t key = ((uint64_t)(uint32_t)(ty * f.grid_x + tx) << 32) | (uint64_t)s_depth[lo];
+        keys[j] = key;
+        values[j] = (uint32_t)(g0 + lo);
+    }
+}
+
+}  // namespace
+
+int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_only, float* records,
+                      uint32_t* tiles_touched, int32_t* radii, hipStream_t s)
+{
+    if (g.P == 0) return GS355_OK;
+    const dim3 block(256), grid((g.P + 255) / 256);
+    if (radii_only)
+        hipLaunchKernelGGL(preprocess_kernel<true>, grid, block, 0, s, f, g, records, tiles_touched, radii);
+    else
+        hipLaunchKernelGGL(preprocess_kernel<false>, grid, block, 0, s, f, g, records, tiles_touched, radii);
+    GS355_CHECK_LAUNCH("preprocess");
+    return GS355_OK;
+}
+
+int launch_duplicate(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
+                     const uint32_t* offsets, const gs355_header* header, uint64_t* keys, uint32_t* values,
+                     hipStream_t s)
+{
+    if (P == 0) return GS355_OK;
+    hipLaunchKernelGGL(duplicate_kernel, dim3((P + 255) / 256), dim3(256), 0, s, f, P, records, radii, offsets,
+                       header, keys, values);
+    GS355_CHECK_LAUNCH("duplicate");
+    return GS355_OK;
+}
+
+}  // namespace gs355

@@ -1,0 +1,227 @@
+"""Host driver of the rasterizer stages: marshals torch tensors into the C ABI
+(include/gs355.h), owns the grow-only device workspace and handles the one
+data-dependent size of a frame, the number of (tile, Gaussian) keys.
+
+PyTorch is used for device memory and streams only; every computation is a
+HIP kernel behind `gs355_run` / `gs355_visible_filter`.
+"""
+import ctypes as C
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_KEY_HEADROOM = 1.25  # capacity = keys needed by the last frame that overflowed x this
+
+
+def _dev_f32(t: Optional[torch.Tensor], device: torch.device, name: str, shape=None) -> Optional[torch.Tensor]:
+    """Contiguous fp32 tensor on `device` (callers pass slices such as
+    `scales[:, :3]`, and per-frame matrices may still live on the host)."""
+    if t is None:
+        return None
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a torch.Tensor, got %r" % (name, type(t)))
+    t = t.detach()
+    if t.device != device:
+        t = t.to(device)
+    if t.dtype != torch.float32:
+        t = t.float()
+    if shape is not None:
+        if t.numel() != math.prod(shape):
+            raise ValueError("%s has %d elements, expected shape %s" % (name, t.numel(), tuple(shape)))
+    return t.contiguous()
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+class Workspace:
+    """Grow-only device buffer plus the key-capacity estimate for one device.
+
+    The library never allocates device memory: this is the caller-owned
+    workspace of the C ABI.  Work using one Workspace must stay on one stream
+    at a time."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self.buffer: Optional[torch.Tensor] = None
+        self.key_capacity = 0
+        self.header_host = torch.zeros(8, dtype=torch.int64, pin_memory=True)
+        self.header_event = torch.cuda.Event()
+        self.frames = 0
+        self.overflows = 0
+
+    def ensure(self, P: int, n_cap: int, width: int, height: int) -> "_lib.Layout":
+        layout = _lib.workspace_layout(P, n_cap, width, height)
+        if self.buffer is None or self.buffer.numel() < layout.total_bytes:
+            self.buffer = None  # release before growing
+            self.buffer = torch.empty(int(layout.total_bytes * 1.1) + 4096, dtype=torch.uint8, device=self.device)
+        return layout
+
+    def view(self, layout: "_lib.Layout", name: str, P: int, n_keys: int, tiles: int) -> torch.Tensor:
+        """Typed view of one workspace array (for tests and diagnostics)."""
+        buf = self.buffer
+
+        def take(off, nbytes, dtype):
+            return buf[off:off + nbytes].view(dtype)
+
+        if name == "header":
+            return take(layout.header, 64, torch.int64)
+        if name == "records":
+            return take(layout.records, P * 48, torch.float32).view(P, 12)
+        if name == "tiles_touched":
+            return take(layout.tiles_touched, P * 4, torch.int32)
+        if name == "offsets":
+            return take(layout.offsets, P * 4, torch.int32)
+        if name in ("keys", "sorted_keys"):
+            which = layout.unsorted_buffer if name == "keys" else layout.sorted_buffer
+            return take(layout.keys[which], n_keys * 8, torch.int64)
+        if name in ("values", "sorted_values"):
+            which = layout.unsorted_buffer if name == "values" else layout.sorted_buffer
+            return take(layout.values[which], n_keys * 4, torch.int32)
+        if name == "ranges":
+            return take(layout.ranges, tiles * 8, torch.int32).view(tiles, 2)
+        raise KeyError(name)
+
+
+_workspaces: Dict[Tuple[int, int], Workspace] = {}
+
+
+def default_workspace(device: torch.device) -> Workspace:
+    stream = torch.cuda.current_stream(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = _workspaces[key] = Workspace(device)
+    return ws
+
+
+class FrameInputs:
+    """The tensors of one rasterizer call, validated and marshalled."""
+
+    def __init__(self, settings, means3D, opacities=None, shs=None, colors_precomp=None, scales=None, rotations=None,
+                 cov3D_precomp=None, need_colour: bool = True):
+        if not isinstance(means3D, torch.Tensor) or not means3D.is_cuda:
+            raise ValueError("means3D must be a tensor on the GPU (the rasterizer has no CPU path)")
+        dev = means3D.device
+        self.device = dev
+        P = means3D.shape[0]
+        self.P = P
+        if need_colour:
+            if (shs is None and colors_precomp is None) or (shs is not None and colors_precomp is not None):
+                raise Exception("Please provide excatly one of either SHs or precomputed colors!")
+        if ((scales is None or rotations is None) and cov3D_precomp is None) or (
+            (scales is not None or rotations is not None) and cov3D_precomp is not None
+        ):
+            raise Exception("Please provide exactly one of either scale/rotation pair or precomputed 3D covariance!")
+
+        self.means3D = _dev_f32(means3D, dev, "means3D", (P, 3))
+        self.opacities = _dev_f32(opacities, dev, "opacities", (P,)) if need_colour else None
+        self.shs = _dev_f32(shs, dev, "shs") if need_colour else None
+        self.colors_precomp = _dev_f32(colors_precomp, dev, "colors_precomp", (P, 3)) if need_colour else None
+        self.scales = _dev_f32(scales, dev, "scales", (P, 3))
+        self.rotations = _dev_f32(rotations, dev, "rotations", (P, 4))
+        self.cov3D_precomp = _dev_f32(cov3D_precomp, dev, "cov3D_precomp", (P, 6))
+        sh_coeffs = 0
+        if self.shs is not None:
+            if self.shs.dim() != 3 or self.shs.shape[0] != P or self.shs.shape[2] != 3:
+                raise ValueError("shs must have shape [P, M, 3], got %s" % (tuple(self.shs.shape),))
+            sh_coeffs = int(self.shs.shape[1])
+
+        s = settings
+        self.width, self.height = int(s.image_width), int(s.image_height)
+        self.viewmatrix = _dev_f32(s.viewmatrix, dev, "viewmatrix", (16,))
+        self.projmatrix = _dev_f32(s.projmatrix, dev, "projmatrix", (16,))
+        self.campos = _dev_f32(s.campos, dev, "campos", (3,))
+        self.bg = _dev_f32(s.bg, dev, "bg", (3,))
+
+        f = _lib.Frame()
+        f.image_width, f.image_height = self.width, self.height
+        f.tanfovx, f.tanfovy = float(s.tanfovx), float(s.tanfovy)
+        f.scale_modifier = float(s.scale_modifier)
+        f.sh_degree, f.sh_coeffs = int(s.sh_degree), sh_coeffs
+        f.viewmatrix, f.projmatrix = _ptr(self.viewmatrix), _ptr(self.projmatrix)
+        f.campos, f.bg = _ptr(self.campos), _ptr(self.bg)
+        self.frame = f
+
+        g = _lib.Gaussians()
+        g.P = P
+        g.means3D, g.shs, g.colors_precomp = _ptr(self.means3D), _ptr(self.shs), _ptr(self.colors_precomp)
+        g.opacities, g.scales, g.rotations = _ptr(self.opacities), _ptr(self.scales), _ptr(self.rotations)
+        g.cov3D_precomp = _ptr(self.cov3D_precomp)
+        self.gaussians = g
+
+    @property
+    def tiles(self) -> int:
+        return ((self.width + 15) // 16) * ((self.height + 15) // 16)
+
+
+def visible_filter(inputs: FrameInputs) -> torch.Tensor:
+    """radii int32[P] of the cull / covariance / radius / tile-rectangle test."""
+    radii = torch.empty(inputs.P, dtype=torch.int32, device=inputs.device)
+    stream = torch.cuda.current_stream(inputs.device).cuda_stream
+    _lib.check(_lib.load().gs355_visible_filter(C.byref(inputs.frame), C.byref(inputs.gaussians), _ptr(radii), stream))
+    return radii
+
+
+class FrameOutputs:
+    def __init__(self, inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True):
+        dev, H, W = inputs.device, inputs.height, inputs.width
+        self.image = torch.empty((3, H, W), dtype=torch.float32, device=dev)
+        self.depth = torch.empty((1, H, W), dtype=torch.float32, device=dev) if want_depth else None
+        self.alpha = torch.empty((1, H, W), dtype=torch.float32, device=dev) if want_alpha else None
+        self.radii = torch.empty(inputs.P, dtype=torch.int32, device=dev)
+        o = _lib.Outputs()
+        o.image, o.depth, o.alpha, o.radii = _ptr(self.image), _ptr(self.depth), _ptr(self.alpha), _ptr(self.radii)
+        self.c = o
+        self.num_keys = 0
+        self.num_visible = 0
+
+
+def run_stages(inputs: FrameInputs, outputs: FrameOutputs, ws: Workspace, n_cap: int, stage_mask: int):
+    """Enqueue the selected stages over `ws`; returns the layout used."""
+    layout = ws.ensure(inputs.P, n_cap, inputs.width, inputs.height)
+    stream = torch.cuda.current_stream(inputs.device).cuda_stream
+    rc = _lib.load().gs355_run(C.byref(inputs.frame), C.byref(inputs.gaussians), ws.buffer.data_ptr(),
+                               ws.buffer.numel(), int(n_cap), C.byref(outputs.c), int(stage_mask), stream)
+    _lib.check(rc)
+    return layout
+
+
+def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True,
+           ws: Optional[Workspace] = None) -> FrameOutputs:
+    """All stages of one frame.
+
+    The key count is only known on the device after the scan.  The header is
+    copied to pinned host memory right after the scan and the remaining stages
+    are enqueued against the current capacity without waiting; the host then
+    waits for that small copy only (the GPU keeps working on sort and blend).
+    If the frame needed more keys than the capacity, it is redone once with
+    the exact requirement plus headroom; capacity never shrinks."""
+    ws = ws or default_workspace(inputs.device)
+    out = FrameOutputs(inputs, want_depth, want_alpha)
+    if ws.key_capacity == 0:
+        ws.key_capacity = max(1 << 20, 4 * inputs.P)
+    front = _lib.STAGE_PREPROCESS | _lib.STAGE_SCAN
+    back = _lib.STAGE_DUPLICATE | _lib.STAGE_SORT | _lib.STAGE_RANGES | _lib.STAGE_BLEND
+    for attempt in range(3):
+        n_cap = ws.key_capacity
+        layout = run_stages(inputs, out, ws, n_cap, front)
+        ws.header_host.copy_(ws.buffer[layout.header:layout.header + 64].view(torch.int64), non_blocking=True)
+        ws.header_event.record(torch.cuda.current_stream(inputs.device))
+        run_stages(inputs, out, ws, n_cap, back)
+        ws.header_event.synchronize()
+        total = int(ws.header_host[0])
+        word1 = int(ws.header_host[1])
+        overflow = (word1 >> 32) & 0xFFFFFFFF
+        out.num_keys = total
+        out.num_visible = int(ws.header_host[2]) & 0xFFFFFFFF
+        ws.frames += 1
+        if not overflow:
+            return out
+        ws.overflows += 1
+        ws.key_capacity = int(total * _KEY_HEADROOM) + 4096
+    raise RuntimeError("key capacity still insufficient after regrowing (needed %d keys)" % out.num_keys)

@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Headline benchmark: 1080p frames/s of the 3DGS forward render at 6M Gaussians
+on one MI355X (synthetic city-block scene, SH degree 3, RGB + depth + alpha).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--gaussians P]
+
+A step is one full frame through GaussianRasterizer.forward (the product path:
+preprocess -> scan -> duplicate -> sort -> ranges -> blend) with every input
+already resident in HBM.  Prints ONE JSON line with the frame rate, a
+per-stage breakdown timed with HIP events on the launch stream, the roofline
+figure of the dominant stage and a CPU baseline (the PyTorch-CPU rasterizer of
+the same semantics on the host cores, on a bounded sample of the workload).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+FP32_PEAK_TFLOPS = 157.3  # MI355X fp32 vector peak (packed FMA); this build issues unpacked FP32 only
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=3, choices=[1, 2, 3])
+    ap.add_argument("--gaussians", type=int, default=None, help="override the Gaussian count (not the headline workload)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--stage-steps", type=int, default=20)
+    return ap.parse_args()
+
+
+def settings_for(scene, device):
+    from landmarksystem_amd import GaussianRasterizationSettings
+
+    cam = scene.camera.to(device)
+    return GaussianRasterizationSettings(
+        image_height=cam.height, image_width=cam.width, tanfovx=math.tan(cam.FovX * 0.5),
+        tanfovy=math.tan(cam.FovY * 0.5), bg=scene.bg.to(device), scale_modifier=1.0,
+        viewmatrix=cam.world_view_transform, projmatrix=cam.full_proj_transform, sh_degree=scene.sh_degree,
+        campos=cam.camera_center, prefiltered=False, debug=False,
+    )
+
+
+def stage_breakdown(torch, pipeline, _lib, inp, n_cap, steps):
+    """Average milliseconds per stage, HIP events on the launch stream."""
+    stages = [("preprocess", _lib.STAGE_PREPROCESS), ("scan", _lib.STAGE_SCAN), ("duplicate", _lib.STAGE_DUPLICATE),
+              ("sort", _lib.STAGE_SORT), ("ranges", _lib.STAGE_RANGES), ("blend", _lib.STAGE_BLEND)]
+    ws = pipeline.Workspace(inp.device)
+    out = pipeline.FrameOutputs(inp)
+    for _, m in stages:  # warm
+        pipeline.run_stages(inp, out, ws, n_cap, m)
+    torch.cuda.synchronize()
+    acc = {n: 0.0 for n, _ in stages}
+    for _ in range(steps):
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(stages) + 1)]
+        evs[0].record()
+        for k, (_, m) in enumerate(stages):
+            pipeline.run_stages(inp, out, ws, n_cap, m)
+            evs[k + 1].record()
+        torch.cuda.synchronize()
+        for k, (n, _) in enumerate(stages):
+            acc[n] += evs[k].elapsed_time(evs[k + 1])
+    lay = _lib.workspace_layout(inp.P, n_cap, inp.width, inp.height)
+    hdr = ws.view(lay, "header", inp.P, 0, inp.tiles).cpu()
+    ranges = ws.view(lay, "ranges", inp.P, 0, inp.tiles).cpu().numpy().view("uint32")
+    stats = {"num_keys": int(hdr[0]), "num_visible": int(hdr[2]) & 0xFFFFFFFF,
+             "range_sum": int((ranges[:, 1].astype("int64") - ranges[:, 0]).sum()), "sort_passes": int(lay.sort_passes)}
+    return {n: acc[n] / steps for n in acc}, stats
+
+
+def algorithmic_work(P, V, N, tiles, npix, sh_coeffs, passes, blend_pairs):
+    """Algorithmic bytes / flops per frame and stage."""
+    b_in = 12 + 12 + 16 + 4 + 12 * sh_coeffs  # mean, scale, quat, opacity, SH
+    return {
+        "preprocess": 12 * P + 8 * P + V * (b_in - 12) + V * 40,
+        "scan": 8 * P,
+        "duplicate": V * 20 + 12 * N,
+        "sort": N * (8 + passes * 24),
+        "ranges": 8 * N + 8 * tiles,
+        "blend_bytes": 40 * N + 20 * npix,
+        "blend_flops": 25 * blend_pairs,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build renders on one GPU; --gpus %d is not supported (run with --gpus 1)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from landmarksystem_amd import GaussianRasterizer, _lib, pipeline, scenes
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    _lib.load()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    t0 = time.time()
+    make = scenes.BY_INDEX[args.config]
+    scene = make(args.gaussians) if args.gaussians else make()
+    gen_s = time.time() - t0
+    d = scene.to(dev)
+    rast = GaussianRasterizer(settings_for(scene, dev))
+    kwargs = dict(means3D=d.means3D, means2D=None, shs=d.shs, colors_precomp=None, opacities=d.opacities,
+                  scales=d.scales, rotations=d.rotations, cov3D_precomp=None)
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            rast(**kwargs)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            image, radii, depth = rast(**kwargs)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    fps = args.steps / elapsed
+
+    # per-stage breakdown on the same inputs
+    inp = pipeline.FrameInputs(rast.raster_settings, d.means3D, opacities=d.opacities, shs=d.shs, scales=d.scales,
+                               rotations=d.rotations)
+    n_cap = pipeline.default_workspace(dev).key_capacity
+    stage_ms, stats = stage_breakdown(torch, pipeline, _lib, inp, n_cap, args.stage_steps)
+    P, V, N = scene.P, stats["num_visible"], stats["num_keys"]
+    tiles, npix = inp.tiles, inp.width * inp.height
+
+    # blend work: exact pair count from the CPU oracle would need minutes at this size; use the
+    # kernel-independent upper bound 256 * (sum of tile range lengths), as defined for the blend stage
+    blend_pairs_upper = 256 * stats["range_sum"]
+    work = algorithmic_work(P, V, N, tiles, npix, scene.shs.shape[1], stats["sort_passes"], blend_pairs_upper)
+    stages = {}
+    for name in ("preprocess", "scan", "duplicate", "sort", "ranges"):
+        ms = stage_ms[name]
+        stages[name] = {"ms": round(ms, 4), "bytes": work[name], "GBps": round(work[name] / ms / 1e6, 1),
+                        "frac_hbm": round(work[name] / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    ms = stage_ms["blend"]
+    stages["blend"] = {"ms": round(ms, 4), "flops_upper": work["blend_flops"],
+                       "TFLOPs_upper": round(work["blend_flops"] / ms / 1e9, 2),
+                       "frac_fp32_upper": round(work["blend_flops"] / ms / 1e9 / FP32_PEAK_TFLOPS, 4)}
+    stages["rates"] = {"gaussians_per_s_preprocess": round(P / stage_ms["preprocess"] * 1e3),
+                       "sorted_keys_per_s": round(N / stage_ms["sort"] * 1e3) if N else 0,
+                       "blend_frames_per_s": round(1e3 / stage_ms["blend"], 1)}
+
+    dominant = max(("preprocess", "scan", "duplicate", "sort", "ranges", "blend"), key=lambda n: stage_ms[n])
+    if dominant == "blend":
+        roofline = {"bound": "mfma", "kernel": "blend_kernel", "achieved": stages["blend"]["TFLOPs_upper"],
+                    "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": stages["blend"]["frac_fp32_upper"],
+                    "traffic": None,
+                    "note": "FP32 VALU kernel (no MFMA); peak is the MI355X fp32 figure; flops = 25 x 256 x sum of "
+                            "tile range lengths (upper bound on evaluated pixel-Gaussian pairs)"}
+    else:
+        roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": None}
+
+    result = {
+        "metric": "1080p frames/sec at 6M Gaussians (1 GPU)",
+        "value": round(fps, 2),
+        "unit": "frames/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[%d]: %s, %d Gaussians, SH degree %d, %dx%d, RGB+depth+alpha" %
+                               (args.config - 1, scene.name, P, scene.sh_degree, inp.width, inp.height),
+                   "visible": V, "keys": N, "tiles": tiles, "scene_gen_s": round(gen_s, 1)},
+        "roofline": roofline,
+        "stages": stages,
+    }
+    if not args.no_cpu_baseline:
+        try:
+            from oracle import torch_oracle
+
+            result["cpu_baseline"] = torch_oracle.timed_baseline(scene)
+        except Exception as exc:  # the baseline is a reported figure, never a reason to lose the GPU numbers
+            result["cpu_baseline"] = {"error": repr(exc)}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -104,12 +104,6 @@ class FrameInputs:
 
     def __init__(self, settings, means3D, opacities=None, shs=None, colors_precomp=None, scales=None, rotations=None,
                  cov3D_precomp=None, need_colour: bool = True):
-        if not isinstance(means3D, torch.Tensor) or not means3D.is_cuda:
-            raise ValueError("means3D must be a tensor on the GPU (the rasterizer has no CPU path)")
-        dev = means3D.device
-        self.device = dev
-        P = means3D.shape[0]
-        self.P = P
         if need_colour:
             if (shs is None and colors_precomp is None) or (shs is not None and colors_precomp is not None):
                 raise Exception("Please provide excatly one of either SHs or precomputed colors!")
@@ -117,6 +111,12 @@ class FrameInputs:
             (scales is not None or rotations is not None) and cov3D_precomp is not None
         ):
             raise Exception("Please provide exactly one of either scale/rotation pair or precomputed 3D covariance!")
+        if not isinstance(means3D, torch.Tensor) or not means3D.is_cuda:
+            raise ValueError("means3D must be a tensor on the GPU (the rasterizer has no CPU path)")
+        dev = means3D.device
+        self.device = dev
+        P = means3D.shape[0]
+        self.P = P
 
         self.means3D = _dev_f32(means3D, dev, "means3D", (P, 3))
         self.opacities = _dev_f32(opacities, dev, "opacities", (P,)) if need_colour else None

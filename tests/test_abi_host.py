@@ -1,0 +1,149 @@
+"""Host side of the C ABI, no GPU needed: the library loads, exports exactly the
+symbols include/gs355.h declares, lays the workspace out sanely and rejects bad
+arguments before touching HIP."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from landmarksystem_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "gs355.h")).read()
+    return sorted(set(re.findall(r"GS355_API\s+[\w\s\*]+?\b(gs355_\w+)\s*\(", text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_functions()
+    assert names == sorted(_lib.EXPORTS)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.gs355_version() == 1
+
+
+def test_struct_sizes_match_the_header():
+    # 64-byte header; pointers are 8 bytes; the layout struct mirrors include/gs355.h field by field
+    assert C.sizeof(_lib.Header) == 64
+    assert C.sizeof(_lib.Frame) == 7 * 4 + 4 + 4 * 8  # 7 scalars, padding to 8, 4 pointers
+    assert C.sizeof(_lib.Gaussians) == 8 + 7 * 8
+    assert C.sizeof(_lib.Outputs) == 4 * 8
+    assert C.sizeof(_lib.Layout) == 12 * 8 + 4 * 4
+
+
+def test_workspace_layout_is_aligned_ordered_and_sized():
+    P, n_cap, W, H = 100_000, 1_500_000, 1920, 1080
+    L = _lib.workspace_layout(P, n_cap, W, H)
+    offs = [L.header, L.records, L.tiles_touched, L.offsets, L.scan_tmp, L.keys[0], L.keys[1], L.values[0],
+            L.values[1], L.sort_hist, L.ranges, L.total_bytes]
+    assert all(o % 256 == 0 for o in offs)
+    assert offs == sorted(offs) and len(set(offs)) == len(offs)
+    assert L.records - L.header >= 64
+    assert L.tiles_touched - L.records >= P * 48
+    assert L.keys[1] - L.keys[0] >= n_cap * 8
+    assert L.values[1] - L.values[0] >= n_cap * 4
+    tiles = 120 * 68
+    assert L.total_bytes - L.ranges >= tiles * 8
+    assert L.sort_bits == 32 + 13 and L.sort_passes == 6 and L.sorted_buffer == 0
+    L4k = _lib.workspace_layout(10, 10, 3840, 2160)
+    assert L4k.sort_bits == 47 and L4k.sort_passes == 6
+    Ls = _lib.workspace_layout(10, 10, 256, 256)  # 256 tiles -> 40 bits -> 5 passes -> result in buffer 1
+    assert Ls.sort_bits == 40 and Ls.sort_passes == 5 and Ls.sorted_buffer == 1
+    L0 = _lib.workspace_layout(0, 0, 16, 16)
+    assert L0.total_bytes > 0
+
+
+def _err(code_expected, fn, *args):
+    rc = fn(*args)
+    assert rc == code_expected, (rc, _lib.load().gs355_last_error())
+    return _lib.load().gs355_last_error().decode()
+
+
+def test_layout_rejects_bad_dimensions():
+    lib = _lib.load()
+    L = _lib.Layout()
+    assert "P must be" in _err(_lib.GS355_EINVAL, lib.gs355_workspace_layout, -1, 10, 64, 64, C.byref(L))
+    assert "image size" in _err(_lib.GS355_EINVAL, lib.gs355_workspace_layout, 1, 10, 0, 64, C.byref(L))
+    assert "n_cap" in _err(_lib.GS355_EINVAL, lib.gs355_workspace_layout, 1, -5, 64, 64, C.byref(L))
+    assert "32-bit" in _err(_lib.GS355_EOVERFLOW, lib.gs355_workspace_layout, 1, 1 << 32, 64, 64, C.byref(L))
+    assert "tiles" in _err(_lib.GS355_EOVERFLOW, lib.gs355_workspace_layout, 1, 10, 1 << 20, 1 << 20, C.byref(L))
+    assert _err(_lib.GS355_EINVAL, lib.gs355_workspace_layout, 1, 10, 64, 64, None)
+    with pytest.raises(_lib.Gs355Error) as e:
+        _lib.workspace_layout(-3, 0, 8, 8)
+    assert e.value.code == _lib.GS355_EINVAL
+
+
+def _frame(W=64, H=64, deg=0, coeffs=1, ptr=0x1000):
+    f = _lib.Frame()
+    f.image_width, f.image_height, f.tanfovx, f.tanfovy, f.scale_modifier = W, H, 0.5, 0.5, 1.0
+    f.sh_degree, f.sh_coeffs = deg, coeffs
+    f.viewmatrix = f.projmatrix = f.campos = f.bg = ptr
+    return f
+
+
+def _gauss(P=10, shs=True, colors=False, sr=True, cov=False, ptr=0x1000):
+    g = _lib.Gaussians()
+    g.P = P
+    g.means3D = g.opacities = ptr
+    g.shs = ptr if shs else None
+    g.colors_precomp = ptr if colors else None
+    g.scales = g.rotations = (ptr if sr else None)
+    g.cov3D_precomp = ptr if cov else None
+    return g
+
+
+def test_run_validates_before_any_hip_call():
+    """All of these return before a kernel could be launched: the fake
+    pointers are never dereferenced and no GPU is needed."""
+    lib = _lib.load()
+    out = _lib.Outputs()
+    out.image = out.radii = 0x1000
+    run = lambda f, g, ws, nbytes, cap, o, mask: lib.gs355_run(  # noqa: E731
+        C.byref(f) if f else None, C.byref(g) if g else None, ws, nbytes, cap, C.byref(o) if o else None, mask, None)
+    f, g = _frame(), _gauss()
+    assert "frame is NULL" in _err(_lib.GS355_EINVAL, run, None, g, 0x1000, 1 << 30, 100, out, _lib.STAGE_ALL)
+    assert "gaussians is NULL" in _err(_lib.GS355_EINVAL, run, f, None, 0x1000, 1 << 30, 100, out, _lib.STAGE_ALL)
+    assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 0)
+    assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 128)
+    assert "SHs or precomputed colors" in _err(_lib.GS355_EINVAL, run, f, _gauss(shs=True, colors=True), 0x1000,
+                                                1 << 30, 100, out, _lib.STAGE_ALL)
+    assert "SHs or precomputed colors" in _err(_lib.GS355_EINVAL, run, f, _gauss(shs=False, colors=False), 0x1000,
+                                                1 << 30, 100, out, _lib.STAGE_ALL)
+    assert "scale/rotation" in _err(_lib.GS355_EINVAL, run, f, _gauss(sr=True, cov=True), 0x1000, 1 << 30, 100, out,
+                                     _lib.STAGE_ALL)
+    assert "scale/rotation" in _err(_lib.GS355_EINVAL, run, f, _gauss(sr=False, cov=False), 0x1000, 1 << 30, 100,
+                                     out, _lib.STAGE_ALL)
+    assert "sh_degree" in _err(_lib.GS355_EINVAL, run, _frame(deg=4, coeffs=25), g, 0x1000, 1 << 30, 100, out,
+                               _lib.STAGE_ALL)
+    assert "coefficients" in _err(_lib.GS355_EINVAL, run, _frame(deg=3, coeffs=4), g, 0x1000, 1 << 30, 100, out,
+                                  _lib.STAGE_ALL)
+    bad = _frame()
+    bad.tanfovx = 0.0
+    assert "tanfov" in _err(_lib.GS355_EINVAL, run, bad, g, 0x1000, 1 << 30, 100, out, _lib.STAGE_ALL)
+    assert "workspace is NULL" in _err(_lib.GS355_EINVAL, run, f, g, None, 1 << 30, 100, out, _lib.STAGE_ALL)
+    assert "aligned" in _err(_lib.GS355_EINVAL, run, f, g, 0x1001, 1 << 30, 100, out, _lib.STAGE_ALL)
+    msg = _err(_lib.GS355_ENOSPC, run, f, g, 0x1000, 1024, 100, out, _lib.STAGE_ALL)
+    assert "needed" in msg
+    assert "32-bit" in _err(_lib.GS355_EOVERFLOW, run, f, g, 0x1000, 1 << 30, 1 << 33, out, _lib.STAGE_ALL)
+    no_img = _lib.Outputs()
+    no_img.radii = 0x1000
+    assert "image is NULL" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, no_img, _lib.STAGE_BLEND)
+    no_radii = _lib.Outputs()
+    no_radii.image = 0x1000
+    assert "radii is NULL" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, no_radii, _lib.STAGE_ALL)
+
+
+def test_visible_filter_validates():
+    lib = _lib.load()
+    f, g = _frame(), _gauss(shs=False)
+    vf = lambda f, g, r: lib.gs355_visible_filter(C.byref(f) if f else None, C.byref(g) if g else None, r, None)  # noqa: E731
+    assert "frame is NULL" in _err(_lib.GS355_EINVAL, vf, None, g, 0x1000)
+    assert "radii is NULL" in _err(_lib.GS355_EINVAL, vf, f, g, None)
+    assert "scale/rotation" in _err(_lib.GS355_EINVAL, vf, f, _gauss(sr=False), 0x1000)
+    half = _gauss()
+    half.rotations = None
+    assert "scale/rotation" in _err(_lib.GS355_EINVAL, vf, f, half, 0x1000)

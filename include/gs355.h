@@ -104,7 +104,7 @@ typedef struct gs355_header {
  * aligned).  Tests read intermediates through these. */
 typedef struct gs355_layout {
     size_t header;        /* gs355_header */
-    size_t records;       /* f32[P][12]: px, py, conic_x, conic_y, conic_z, opacity, r, g, b, depth, 0, 0 */
+    size_t records;       /* f32[P][12]: px, py, conic_x, conic_y, conic_z, opacity, r, g, b, depth, reach_x, reach_y */
     size_t tiles_touched; /* u32[P] */
     size_t offsets;       /* u32[P]   inclusive prefix sum of tiles_touched */
     size_t scan_tmp;      /* u32[...] block sums of the scans */
@@ -127,7 +127,10 @@ enum {
     GS355_STAGE_SORT = 8,       /* stable LSD radix sort of the pairs by key */
     GS355_STAGE_RANGES = 16,    /* per-tile [first, last) in the sorted keys */
     GS355_STAGE_BLEND = 32,     /* front-to-back alpha blending per 16x16 tile */
-    GS355_STAGE_ALL = 63
+    GS355_STAGE_ALL = 63,
+    /* Verification variant of the blend stage: every staged Gaussian is evaluated on every pixel of the tile
+     * (no per-quadrant culling).  Produces the same image as GS355_STAGE_BLEND; not part of GS355_STAGE_ALL. */
+    GS355_STAGE_BLEND_PLAIN = 64
 };
 
 GS355_API int gs355_version(void);

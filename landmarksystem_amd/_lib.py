@@ -13,6 +13,7 @@ GS355_OK, GS355_EINVAL, GS355_ENOSPC, GS355_EOVERFLOW, GS355_EHIP = 0, -1, -2, -
 
 STAGE_PREPROCESS, STAGE_SCAN, STAGE_DUPLICATE, STAGE_SORT, STAGE_RANGES, STAGE_BLEND = 1, 2, 4, 8, 16, 32
 STAGE_ALL = 63
+STAGE_BLEND_PLAIN = 64
 
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
            "gs355_visible_filter")

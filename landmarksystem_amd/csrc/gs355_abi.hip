@@ -176,7 +176,7 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
               int64_t n_cap, const gs355_outputs* out, uint32_t stage_mask, void* stream)
 {
     int rc;
-    if ((stage_mask & ~(uint32_t)GS355_STAGE_ALL) != 0 || stage_mask == 0)
+    if ((stage_mask & ~(uint32_t)(GS355_STAGE_ALL | GS355_STAGE_BLEND_PLAIN)) != 0 || stage_mask == 0)
         return set_error(GS355_EINVAL, "stage_mask 0x%x selects no known stage", stage_mask);
     if ((rc = check_frame(frame, true))) return rc;
     if ((rc = check_geometry_inputs(g))) return rc;
@@ -184,7 +184,7 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     if (!out) return set_error(GS355_EINVAL, "outputs is NULL");
     if ((stage_mask & GS355_STAGE_PREPROCESS) && g->P > 0 && !out->radii)
         return set_error(GS355_EINVAL, "outputs.radii is NULL");
-    if ((stage_mask & GS355_STAGE_BLEND) && !out->image) return set_error(GS355_EINVAL, "outputs.image is NULL");
+    if ((stage_mask & (GS355_STAGE_BLEND | GS355_STAGE_BLEND_PLAIN)) && !out->image) return set_error(GS355_EINVAL, "outputs.image is NULL");
     gs355_layout L;
     if ((rc = make_layout(g->P, n_cap, frame->image_width, frame->image_height, &L))) return rc;
     if (!workspace) return set_error(GS355_EINVAL, "workspace is NULL");
@@ -219,9 +219,9 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
             return rc;
     if (stage_mask & GS355_STAGE_RANGES)
         if ((rc = launch_ranges(header, cap, keys[L.sorted_buffer], ranges, fa.grid_x * fa.grid_y, s))) return rc;
-    if (stage_mask & GS355_STAGE_BLEND)
+    if (stage_mask & (GS355_STAGE_BLEND | GS355_STAGE_BLEND_PLAIN))
         if ((rc = launch_blend(fa, header, ranges, vals[L.sorted_buffer], records, out->image, out->depth, out->alpha,
-                               s)))
+                               (stage_mask & GS355_STAGE_BLEND) != 0, s)))
             return rc;
     return GS355_OK;
 }

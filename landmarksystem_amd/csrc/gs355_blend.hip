@@ -42,6 +42,45 @@ __global__ __launch_bounds__(256) void ranges_kernel(const gs355_header* __restr
     if (j == n - 1) ranges[2 * t + 1] = n;
 }
 
+// exp(power) -> alpha, the three discrete tests and the accumulation for one
+// (pixel, Gaussian) pair.  `power` is evaluated with unfused multiplies and
+// adds in a fixed order so that the sign test and the alpha threshold see the
+// same exponent as a scalar evaluation of the same formula.
+struct PixelState {
+    float T, c0, c1, c2, depth;
+    bool done;
+};
+
+__device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, const float4 a, const float4 b,
+                                          const float4 c)
+{
+    const float dx = a.x - pxf, dy = a.y - pyf;
+    const float t1 = __fmul_rn(__fmul_rn(a.z, dx), dx);
+    const float t2 = __fmul_rn(__fmul_rn(b.x, dy), dy);
+    const float t3 = __fmul_rn(__fmul_rn(a.w, dx), dy);
+    const float power = __fsub_rn(__fmul_rn(-0.5f, __fadd_rn(t1, t2)), t3);
+    if (power > 0.0f) return;
+    const float alpha = fminf(0.99f, b.y * __expf(power));
+    if (alpha < 1.0f / 255.0f) return;
+    const float test_T = p.T * (1.0f - alpha);
+    if (test_T < 0.0001f) {
+        p.done = true;
+        return;
+    }
+    const float w = alpha * p.T;
+    p.c0 += b.z * w;
+    p.c1 += b.w * w;
+    p.c2 += c.x * w;
+    p.depth += c.y * w;
+    p.T = test_T;
+}
+
+// kCull: each wavefront first tests the staged Gaussians against its own 8x8
+// quadrant (one Gaussian per lane, bounding box of the alpha >= 1/255 region
+// from the record) and then visits only the ballot's set bits.  A skipped
+// (quadrant, Gaussian) pair is one whose 64 pixels would all have taken the
+// `alpha < 1/255` branch, so both variants produce identical images.
+template <bool kCull>
 __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_header* __restrict__ header,
                                                     const uint32_t* __restrict__ ranges,
                                                     const uint32_t* __restrict__ values,
@@ -50,61 +89,65 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
 {
     __shared__ float4 s_a[256];  // px, py, conic_x, conic_y
     __shared__ float4 s_b[256];  // conic_z, opacity, r, g
-    __shared__ float2 s_c[256];  // b, depth
+    __shared__ float4 s_c[256];  // b, depth, reach_x, reach_y
     __shared__ uint32_t s_wave_done[4];
 
     if (header->overflow) return;
     const int tile = blockIdx.x;
     const int tile_x = tile % f.grid_x, tile_y = tile / f.grid_x;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int px = tile_x * kTile + (wave & 1) * 8 + (lane & 7);
-    const int py = tile_y * kTile + (wave >> 1) * 8 + (lane >> 3);
+    const int qx0 = tile_x * kTile + (wave & 1) * 8, qy0 = tile_y * kTile + (wave >> 1) * 8;
+    const int px = qx0 + (lane & 7), py = qy0 + (lane >> 3);
     const bool inside = px < f.W && py < f.H;
     const float pxf = (float)px, pyf = (float)py;
+    // pixel-centre bounds of this wavefront's quadrant
+    const float qx_lo = (float)qx0, qx_hi = (float)(qx0 + 7), qy_lo = (float)qy0, qy_hi = (float)(qy0 + 7);
 
     const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
-    float T = 1.0f, c0 = 0.0f, c1 = 0.0f, c2 = 0.0f, dsum = 0.0f;
-    bool done = !inside;
+    PixelState p = {1.0f, 0.0f, 0.0f, 0.0f, 0.0f, !inside};
 
     for (uint32_t base = lo; base < hi; base += 256) {
-        const bool wave_done = __ballot(!done) == 0ull;
+        const bool wave_done = __ballot(!p.done) == 0ull;
         if (lane == 0) s_wave_done[wave] = wave_done ? 1u : 0u;
         const uint32_t j = base + tid;
         if (j < hi) {
             const uint32_t g = values[j];
             const float4* __restrict__ rec = reinterpret_cast<const float4*>(records + (size_t)g * kRecordFloats);
-            const float4 r0 = rec[0], r1 = rec[1];
-            const float2 r2 = *reinterpret_cast<const float2*>(rec + 2);
-            s_a[tid] = r0;
-            s_b[tid] = r1;
-            s_c[tid] = r2;
+            s_a[tid] = rec[0];
+            s_b[tid] = rec[1];
+            s_c[tid] = rec[2];
         }
         __syncthreads();
         if ((s_wave_done[0] & s_wave_done[1] & s_wave_done[2] & s_wave_done[3]) != 0u) break;
         const int count = (int)min(256u, hi - base);
         if (!wave_done) {
-            for (int k = 0; k < count; ++k) {
-                if (__ballot(!done) == 0ull) break;
-                if (done) continue;
-                const float4 a = s_a[k];
-                const float4 b = s_b[k];
-                const float dx = a.x - pxf, dy = a.y - pyf;
-                const float power = -0.5f * (a.z * dx * dx + b.x * dy * dy) - a.w * dx * dy;
-                if (power > 0.0f) continue;
-                const float alpha = fminf(0.99f, b.y * __expf(power));
-                if (alpha < 1.0f / 255.0f) continue;
-                const float test_T = T * (1.0f - alpha);
-                if (test_T < 0.0001f) {
-                    done = true;
-                    continue;
+            if (kCull) {
+                bool finished = false;
+                for (int chunk = 0; chunk < count && !finished; chunk += 64) {
+                    const int k = chunk + lane;
+                    bool hit = false;
+                    if (k < count) {
+                        const float4 a = s_a[k];
+                        const float4 c = s_c[k];
+                        hit = (a.x + c.z >= qx_lo) && (a.x - c.z <= qx_hi) && (a.y + c.w >= qy_lo) &&
+                              (a.y - c.w <= qy_hi);
+                    }
+                    uint64_t todo = __ballot(hit);
+                    while (todo != 0ull) {
+                        const int kk = chunk + (int)__builtin_ctzll(todo);
+                        todo &= todo - 1ull;
+                        if (!p.done) blend_one(p, pxf, pyf, s_a[kk], s_b[kk], s_c[kk]);
+                        if (__ballot(!p.done) == 0ull) {
+                            finished = true;
+                            break;
+                        }
+                    }
                 }
-                const float2 c = s_c[k];
-                const float w = alpha * T;
-                c0 += b.z * w;
-                c1 += b.w * w;
-                c2 += c.x * w;
-                dsum += c.y * w;
-                T = test_T;
+            } else {
+                for (int k = 0; k < count; ++k) {
+                    if (__ballot(!p.done) == 0ull) break;
+                    if (!p.done) blend_one(p, pxf, pyf, s_a[k], s_b[k], s_c[k]);
+                }
             }
         }
         __syncthreads();
@@ -113,11 +156,11 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
     if (inside) {
         const size_t plane = (size_t)f.W * f.H;
         const size_t o = (size_t)py * f.W + px;
-        image[o] = c0 + T * f.bg[0];
-        image[plane + o] = c1 + T * f.bg[1];
-        image[2 * plane + o] = c2 + T * f.bg[2];
-        if (out_depth) out_depth[o] = dsum;
-        if (out_alpha) out_alpha[o] = 1.0f - T;
+        image[o] = p.c0 + p.T * f.bg[0];
+        image[plane + o] = p.c1 + p.T * f.bg[1];
+        image[2 * plane + o] = p.c2 + p.T * f.bg[2];
+        if (out_depth) out_depth[o] = p.depth;
+        if (out_alpha) out_alpha[o] = 1.0f - p.T;
     }
 }
 
@@ -137,11 +180,15 @@ int launch_ranges(const gs355_header* header, uint32_t n_cap, const uint64_t* ke
 }
 
 int launch_blend(const FrameArgs& f, const gs355_header* header, const uint32_t* ranges, const uint32_t* values,
-                 const float* records, float* image, float* depth, float* alpha, hipStream_t s)
+                 const float* records, float* image, float* depth, float* alpha, bool cull, hipStream_t s)
 {
     const int tiles = f.grid_x * f.grid_y;
-    hipLaunchKernelGGL(blend_kernel, dim3(tiles), dim3(256), 0, s, f, header, ranges, values, records, image, depth,
-                       alpha);
+    if (cull)
+        hipLaunchKernelGGL(blend_kernel<true>, dim3(tiles), dim3(256), 0, s, f, header, ranges, values, records, image,
+                           depth, alpha);
+    else
+        hipLaunchKernelGGL(blend_kernel<false>, dim3(tiles), dim3(256), 0, s, f, header, ranges, values, records, image,
+                           depth, alpha);
     GS355_CHECK_LAUNCH("blend");
     return GS355_OK;
 }

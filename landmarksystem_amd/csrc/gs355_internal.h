@@ -47,7 +47,7 @@ int launch_sort(const gs355_header* header, uint32_t n_cap, int passes, uint64_t
 int launch_ranges(const gs355_header* header, uint32_t n_cap, const uint64_t* keys, uint32_t* ranges, int tiles,
                   hipStream_t s);
 int launch_blend(const FrameArgs& f, const gs355_header* header, const uint32_t* ranges, const uint32_t* values, const float* records,
-                 float* image, float* depth, float* alpha, hipStream_t s);
+                 float* image, float* depth, float* alpha, bool cull, hipStream_t s);
 
 // generic exclusive scan of u32 (n <= 2^32-1); tmp needs scan_tmp_words(n) words
 size_t scan_tmp_words(size_t n);

@@ -190,10 +190,34 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
             cbl = out[2];
         }
 
+        // Reach of the splat for the blend stage's quadrant culling: half-extents
+        // (ex, ey) of the axis-aligned box around the region where alpha can reach
+        // 1/255, i.e. where 0.5 d^T Q d <= ln(255 * opacity).  The box is enlarged
+        // by more than the rounding error of the blend's fp32 evaluation of the
+        // exponent (bounded below by `noise`), so a quadrant outside the box is
+        // certain to take the blend's `alpha < 1/255` branch on all of its pixels.
+        // +inf = never cull (large or ill-conditioned splats), -inf = never visible.
+        const float opacity = g.opacities[i];
+        const float qx = cc * det_inv, qy = -cb * det_inv, qz = ca * det_inv;
+        float ex, ey;
+        {
+            const float reach = (float)rad + 24.0f;  // |d| over every pixel of every touched tile
+            const float noise = 2.4e-7f * (fabsf(qx) + fabsf(qy) + fabsf(qz)) * reach * reach;
+            if (opacity != opacity || !(noise < 0.02f)) {
+                ex = ey = INFINITY;
+            } else if (!(opacity * 255.0f * 1.0001f >= 1.0f)) {
+                ex = ey = -INFINITY;
+            } else {
+                const float tau = fmaxf(__logf(opacity * 255.0f), 0.0f) * 1.001f + 0.05f;
+                ex = sqrtf(2.0f * tau * ca) * 1.001f + 0.01f;
+                ey = sqrtf(2.0f * tau * cc) * 1.001f + 0.01f;
+            }
+        }
+
         float4* __restrict__ rec = reinterpret_cast<float4*>(records + (size_t)i * kRecordFloats);
-        rec[0] = make_float4(px, py, cc * det_inv, -cb * det_inv);
-        rec[1] = make_float4(ca * det_inv, g.opacities[i], cr, cg);
-        rec[2] = make_float4(cbl, vz, 0.0f, 0.0f);
+        rec[0] = make_float4(px, py, qx, qy);
+        rec[1] = make_float4(qz, opacity, cr, cg);
+        rec[2] = make_float4(cbl, vz, ex, ey);
     } while (false);
 
     radii[i] = radius;

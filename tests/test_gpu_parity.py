@@ -213,3 +213,26 @@ def test_rerun_is_bit_identical(gpu_device):
     b = run_all_stages(scene, gpu_device)
     for k in ("sorted_keys", "sorted_values", "ranges", "image", "depth", "alpha"):
         np.testing.assert_array_equal(a[k], b[k], err_msg=k)
+
+
+@pytest.mark.parametrize("make", [lambda: scenes.config3(P=400_000), lambda: scenes.config2(P=80_000),
+                                  lambda: scenes.tiny_scene(P=3000, width=333, height=211, sh_degree=1, seed=2,
+                                                            log_scale_mean=-1.0)])
+def test_quadrant_culling_is_result_neutral(gpu_device, make):
+    """The blend stage skips (8x8 quadrant, Gaussian) pairs whose bounding box
+    shows alpha < 1/255 on all 64 pixels; the verification variant evaluates
+    every pair.  Both must give identical bits."""
+    scene = make()
+    s = settings_for(scene, gpu_device)
+    inp = pipeline.FrameInputs(s, scene.means3D.to(gpu_device), opacities=scene.opacities.to(gpu_device),
+                               shs=scene.shs.to(gpu_device), scales=scene.scales.to(gpu_device),
+                               rotations=scene.rotations.to(gpu_device))
+    ws = pipeline.Workspace(gpu_device)
+    out = pipeline.render(inp, ws=ws)
+    torch.cuda.synchronize()
+    culled = [out.image.clone(), out.depth.clone(), out.alpha.clone()]
+    pipeline.run_stages(inp, out, ws, ws.key_capacity, _lib.STAGE_BLEND_PLAIN)
+    torch.cuda.synchronize()
+    for a, b in zip(culled, [out.image, out.depth, out.alpha]):
+        assert torch.equal(a, b)
+    assert float(out.alpha.max()) > 0.5

@@ -50,12 +50,7 @@ def settings_for(scene, device):
     )
 
 
-def stage_breakdown(torch, pipeline, _lib, inp, n_cap, steps):
-    """Average milliseconds per stage, HIP events on the launch stream."""
-    stages = [("preprocess", _lib.STAGE_PREPROCESS), ("scan", _lib.STAGE_SCAN), ("duplicate", _lib.STAGE_DUPLICATE),
-              ("sort", _lib.STAGE_SORT), ("ranges", _lib.STAGE_RANGES), ("blend", _lib.STAGE_BLEND)]
-    ws = pipeline.Workspace(inp.device)
-    out = pipeline.FrameOutputs(inp)
+def time_stages(torch, pipeline, inp, out, ws, n_cap, stages, steps):
     for _, m in stages:  # warm
         pipeline.run_stages(inp, out, ws, n_cap, m)
     torch.cuda.synchronize()
@@ -69,12 +64,27 @@ def stage_breakdown(torch, pipeline, _lib, inp, n_cap, steps):
         torch.cuda.synchronize()
         for k, (n, _) in enumerate(stages):
             acc[n] += evs[k].elapsed_time(evs[k + 1])
+    return {n: acc[n] / steps for n in acc}
+
+
+def stage_breakdown(torch, pipeline, _lib, inp, n_cap, steps):
+    """Average milliseconds per stage, HIP events on the launch stream: the
+    shipped pipeline (tile-bucketed sort) and, beside it, the classic
+    duplicate / LSD radix sort / ranges stages it replaces."""
+    ws = pipeline.Workspace(inp.device)
+    out = pipeline.FrameOutputs(inp)
+    fast = [("preprocess", _lib.STAGE_PREPROCESS), ("tile_count", _lib.STAGE_TILE_COUNT),
+            ("tile_scatter", _lib.STAGE_TILE_SCATTER), ("tile_sort", _lib.STAGE_TILESORT), ("blend", _lib.STAGE_BLEND)]
+    classic = [("scan", _lib.STAGE_SCAN), ("duplicate", _lib.STAGE_DUPLICATE), ("sort", _lib.STAGE_SORT),
+               ("ranges", _lib.STAGE_RANGES)]
+    ms = time_stages(torch, pipeline, inp, out, ws, n_cap, fast, steps)
+    ms.update(time_stages(torch, pipeline, inp, out, ws, n_cap, classic, max(3, steps // 4)))
     lay = _lib.workspace_layout(inp.P, n_cap, inp.width, inp.height)
     hdr = ws.view(lay, "header", inp.P, 0, inp.tiles).cpu()
     ranges = ws.view(lay, "ranges", inp.P, 0, inp.tiles).cpu().numpy().view("uint32")
     stats = {"num_keys": int(hdr[0]), "num_visible": int(hdr[2]) & 0xFFFFFFFF,
              "range_sum": int((ranges[:, 1].astype("int64") - ranges[:, 0]).sum()), "sort_passes": int(lay.sort_passes)}
-    return {n: acc[n] / steps for n in acc}, stats
+    return ms, stats
 
 
 def algorithmic_work(P, V, N, tiles, npix, sh_coeffs, passes, blend_pairs):
@@ -139,20 +149,36 @@ def main():
     # kernel-independent upper bound 256 * (sum of tile range lengths), as defined for the blend stage
     blend_pairs_upper = 256 * stats["range_sum"]
     work = algorithmic_work(P, V, N, tiles, npix, scene.shs.shape[1], stats["sort_passes"], blend_pairs_upper)
-    stages = {}
-    for name in ("preprocess", "scan", "duplicate", "sort", "ranges"):
-        ms = stage_ms[name]
-        stages[name] = {"ms": round(ms, 4), "bytes": work[name], "GBps": round(work[name] / ms / 1e6, 1),
-                        "frac_hbm": round(work[name] / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    def hbm(name, ms, nbytes):
+        return {"ms": round(ms, 4), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
+                "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    stages = {"preprocess": hbm("preprocess", stage_ms["preprocess"], work["preprocess"])}
+    # key generation + sort + ranges: the shipped tile-bucketed stages (bin, tile_sort) produce the same sorted
+    # pairs and ranges as duplicate + LSD radix sort + ranges, so they are charged the same algorithmic bytes
+    sort_bytes = work["scan"] + work["duplicate"] + work["sort"] + work["ranges"]
+    sort_ms = stage_ms["tile_count"] + stage_ms["tile_scatter"] + stage_ms["tile_sort"]
+    for name in ("tile_count", "tile_scatter", "tile_sort"):
+        stages[name] = {"ms": round(stage_ms[name], 4)}
+    stages["keys_sort_ranges"] = hbm("keys_sort_ranges", sort_ms, sort_bytes)
+    stages["keys_sort_ranges"]["floor_bytes"] = 24 * N
+    stages["classic_lsd_path"] = {"scan_ms": round(stage_ms["scan"], 4), "duplicate_ms": round(stage_ms["duplicate"], 4), "sort_ms": round(stage_ms["sort"], 4),
+                                  "ranges_ms": round(stage_ms["ranges"], 4),
+                                  "sort_GBps": round(work["sort"] / stage_ms["sort"] / 1e6, 1)}
     ms = stage_ms["blend"]
     stages["blend"] = {"ms": round(ms, 4), "flops_upper": work["blend_flops"],
                        "TFLOPs_upper": round(work["blend_flops"] / ms / 1e9, 2),
                        "frac_fp32_upper": round(work["blend_flops"] / ms / 1e9 / FP32_PEAK_TFLOPS, 4)}
+    pre_sort_bytes = work["preprocess"] + sort_bytes
+    pre_sort_ms = stage_ms["preprocess"] + sort_ms
+    stages["preprocess_plus_sort"] = hbm("preprocess_plus_sort", pre_sort_ms, pre_sort_bytes)
     stages["rates"] = {"gaussians_per_s_preprocess": round(P / stage_ms["preprocess"] * 1e3),
-                       "sorted_keys_per_s": round(N / stage_ms["sort"] * 1e3) if N else 0,
+                       "sorted_keys_per_s": round(N / sort_ms * 1e3) if N else 0,
                        "blend_frames_per_s": round(1e3 / stage_ms["blend"], 1)}
 
-    dominant = max(("preprocess", "scan", "duplicate", "sort", "ranges", "blend"), key=lambda n: stage_ms[n])
+    shipped = {"preprocess": stage_ms["preprocess"], "keys_sort_ranges": sort_ms,
+               "blend": stage_ms["blend"]}
+    dominant = max(shipped, key=lambda n: shipped[n])
     if dominant == "blend":
         roofline = {"bound": "mfma", "kernel": "blend_kernel", "achieved": stages["blend"]["TFLOPs_upper"],
                     "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": stages["blend"]["frac_fp32_upper"],

@@ -91,7 +91,8 @@ typedef struct gs355_outputs {
     int32_t *radii; /* [P] */
 } gs355_outputs;
 
-/* Words of the workspace header (u32 unless noted), written by the scan stage. */
+/* Words of the workspace header (u32 unless noted), written by the scan stage (classic pipeline) or the
+ * tile-count stage (fast pipeline). */
 typedef struct gs355_header {
     uint64_t num_keys_total; /* exact number of (tile, Gaussian) keys the frame needs */
     uint32_t num_keys;       /* min(num_keys_total, key capacity): what later stages process */
@@ -112,6 +113,10 @@ typedef struct gs355_layout {
     size_t values[2];     /* u32[n_cap] x 2 */
     size_t sort_hist;     /* u32[...] per-block digit histograms of the radix sort */
     size_t ranges;        /* u32[tiles][2] */
+    size_t bin_matrix;    /* u32[slices][tiles] pairs per (slice of Gaussians, tile), then their prefix over slices */
+    size_t tile_base;     /* u32[tiles]      first slot of each tile's bucket */
+    size_t bin_visible;   /* u32[slices]     visible Gaussians per slice */
+    size_t tile_lists;    /* u32[2+2*tiles]  counts and lists of buckets too large for the small sorter */
     size_t total_bytes;
     int32_t unsorted_buffer; /* which keys/values buffer the duplicate stage writes (0) */
     int32_t sorted_buffer;   /* which buffer holds the sorted pairs after the sort stage */
@@ -127,10 +132,21 @@ enum {
     GS355_STAGE_SORT = 8,       /* stable LSD radix sort of the pairs by key */
     GS355_STAGE_RANGES = 16,    /* per-tile [first, last) in the sorted keys */
     GS355_STAGE_BLEND = 32,     /* front-to-back alpha blending per 16x16 tile */
-    GS355_STAGE_ALL = 63,
+    GS355_STAGE_ALL = 63, /* the six stages above: the classic pipeline */
     /* Verification variant of the blend stage: every staged Gaussian is evaluated on every pixel of the tile
      * (no per-quadrant culling).  Produces the same image as GS355_STAGE_BLEND; not part of GS355_STAGE_ALL. */
-    GS355_STAGE_BLEND_PLAIN = 64
+    GS355_STAGE_BLEND_PLAIN = 64,
+    /* Tile-bucketed equivalent of SCAN + DUPLICATE + SORT + RANGES: same sorted keys, values, ranges and
+     * header, far less memory traffic, no global atomics.
+     *   TILE_COUNT    pairs per (slice of Gaussians, tile) in LDS-private counters; prefix over slices; tile
+     *                 bases = ranges; header (key count, overflow, visible count)
+     *   TILE_SCATTER  (depth bits << 32 | index) pairs into their tile's bucket
+     *   TILESORT      every bucket sorted by (depth bits, index) in LDS
+     * Needs tiles <= 36000 (the counters of one workgroup live in LDS); larger images use the classic stages. */
+    GS355_STAGE_TILE_COUNT = 128,
+    GS355_STAGE_TILESORT = 256,
+    GS355_STAGE_TILE_SCATTER = 512,
+    GS355_PIPELINE_FAST = 1 | 128 | 512 | 256 | 32
 };
 
 GS355_API int gs355_version(void);
@@ -149,7 +165,7 @@ GS355_API int gs355_workspace_layout(int32_t P, int64_t n_cap, int32_t width, in
 GS355_API int gs355_run(const gs355_frame *frame, const gs355_gaussians *g, void *workspace, size_t workspace_bytes,
               int64_t n_cap, const gs355_outputs *out, uint32_t stage_mask, void *stream);
 
-/* All stages: the body of GaussianRasterizer.forward. */
+/* The whole frame (GS355_PIPELINE_FAST): the body of GaussianRasterizer.forward. */
 GS355_API int gs355_render(const gs355_frame *frame, const gs355_gaussians *g, void *workspace, size_t workspace_bytes,
                  int64_t n_cap, const gs355_outputs *out, void *stream);
 

@@ -14,6 +14,9 @@ GS355_OK, GS355_EINVAL, GS355_ENOSPC, GS355_EOVERFLOW, GS355_EHIP = 0, -1, -2, -
 STAGE_PREPROCESS, STAGE_SCAN, STAGE_DUPLICATE, STAGE_SORT, STAGE_RANGES, STAGE_BLEND = 1, 2, 4, 8, 16, 32
 STAGE_ALL = 63
 STAGE_BLEND_PLAIN = 64
+STAGE_TILE_COUNT, STAGE_TILESORT, STAGE_TILE_SCATTER = 128, 256, 512
+PIPELINE_FAST = STAGE_PREPROCESS | STAGE_TILE_COUNT | STAGE_TILE_SCATTER | STAGE_TILESORT | STAGE_BLEND
+MAX_FAST_TILES = 36000
 
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
            "gs355_visible_filter")
@@ -73,6 +76,10 @@ class Layout(C.Structure):
         ("values", C.c_size_t * 2),
         ("sort_hist", C.c_size_t),
         ("ranges", C.c_size_t),
+        ("bin_matrix", C.c_size_t),
+        ("tile_base", C.c_size_t),
+        ("bin_visible", C.c_size_t),
+        ("tile_lists", C.c_size_t),
         ("total_bytes", C.c_size_t),
         ("unsorted_buffer", C.c_int32),
         ("sorted_buffer", C.c_int32),

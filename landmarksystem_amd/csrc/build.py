@@ -32,6 +32,7 @@ SOURCES = [
     ("gs355_preprocess.hip", ["-ffp-contract=off"]),
     ("gs355_scan.hip", []),
     ("gs355_sort.hip", []),
+    ("gs355_bin.hip", []),
     ("gs355_blend.hip", []),
 ]
 

@@ -25,6 +25,7 @@ int set_error(int code, const char* fmt, ...)
 namespace {
 
 constexpr size_t kAlign = 256;
+constexpr uint32_t kKnownStages = GS355_STAGE_ALL | GS355_STAGE_BLEND_PLAIN | GS355_STAGE_TILE_COUNT | GS355_STAGE_TILESORT | GS355_STAGE_TILE_SCATTER;
 constexpr int64_t kMaxKeys = (1ll << 32) - 1 - kSortTile;  // key slots are indexed with u32
 
 size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
@@ -79,6 +80,11 @@ int make_layout(int32_t P, int64_t n_cap, int32_t W, int32_t H, gs355_layout* L)
     L->values[1] = take(n * sizeof(uint32_t));
     L->sort_hist = take(hist_words * sizeof(uint32_t));
     L->ranges = take(tiles * 2 * sizeof(uint32_t));
+    const size_t slices = tiles <= (size_t)kBinMaxTiles ? (size_t)kBinMaxGroups : 0;
+    L->bin_matrix = take(slices * tiles * sizeof(uint32_t));
+    L->tile_base = take(tiles * sizeof(uint32_t));
+    L->bin_visible = take((size_t)kBinMaxGroups * sizeof(uint32_t));
+    L->tile_lists = take((2 + 2 * tiles) * sizeof(uint32_t));
     L->total_bytes = off;
     L->sort_bits = 32 + ceil_log2((uint32_t)tiles);
     L->sort_passes = (L->sort_bits + kRadixBits - 1) / kRadixBits;
@@ -176,7 +182,7 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
               int64_t n_cap, const gs355_outputs* out, uint32_t stage_mask, void* stream)
 {
     int rc;
-    if ((stage_mask & ~(uint32_t)(GS355_STAGE_ALL | GS355_STAGE_BLEND_PLAIN)) != 0 || stage_mask == 0)
+    if ((stage_mask & ~kKnownStages) != 0 || stage_mask == 0)
         return set_error(GS355_EINVAL, "stage_mask 0x%x selects no known stage", stage_mask);
     if ((rc = check_frame(frame, true))) return rc;
     if ((rc = check_geometry_inputs(g))) return rc;
@@ -187,6 +193,10 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     if ((stage_mask & (GS355_STAGE_BLEND | GS355_STAGE_BLEND_PLAIN)) && !out->image) return set_error(GS355_EINVAL, "outputs.image is NULL");
     gs355_layout L;
     if ((rc = make_layout(g->P, n_cap, frame->image_width, frame->image_height, &L))) return rc;
+    if ((stage_mask & (GS355_STAGE_TILE_COUNT | GS355_STAGE_TILE_SCATTER | GS355_STAGE_TILESORT)) &&
+        (int64_t)((frame->image_width + kTile - 1) / kTile) * ((frame->image_height + kTile - 1) / kTile) > kBinMaxTiles)
+        return set_error(GS355_EINVAL, "the tile-bucketed stages support at most %d tiles; use the classic stages",
+                         kBinMaxTiles);
     if (!workspace) return set_error(GS355_EINVAL, "workspace is NULL");
     if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
         return set_error(GS355_EINVAL, "workspace must be 256-byte aligned");
@@ -204,6 +214,10 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     uint32_t* vals[2] = {reinterpret_cast<uint32_t*>(ws + L.values[0]), reinterpret_cast<uint32_t*>(ws + L.values[1])};
     auto* hist = reinterpret_cast<uint32_t*>(ws + L.sort_hist);
     auto* ranges = reinterpret_cast<uint32_t*>(ws + L.ranges);
+    auto* bin_matrix = reinterpret_cast<uint32_t*>(ws + L.bin_matrix);
+    auto* tile_base = reinterpret_cast<uint32_t*>(ws + L.tile_base);
+    auto* bin_visible = reinterpret_cast<uint32_t*>(ws + L.bin_visible);
+    auto* tile_lists = reinterpret_cast<uint32_t*>(ws + L.tile_lists);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const FrameArgs fa = make_args(frame);
     const uint32_t cap = (uint32_t)n_cap;
@@ -219,6 +233,22 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
             return rc;
     if (stage_mask & GS355_STAGE_RANGES)
         if ((rc = launch_ranges(header, cap, keys[L.sorted_buffer], ranges, fa.grid_x * fa.grid_y, s))) return rc;
+    // tile-bucketed path: buckets live in the buffer the sorted keys do not use
+    const int tiles = fa.grid_x * fa.grid_y;
+    uint64_t* buckets = keys[1 - L.sorted_buffer];
+    if (stage_mask & GS355_STAGE_TILE_COUNT) {
+        if ((rc = launch_tile_count(fa, g->P, records, out->radii, bin_matrix, bin_visible, s))) return rc;
+        if ((rc = launch_tile_layout(g->P, bin_matrix, bin_visible, tiles, cap, header, tile_base, ranges, tile_lists,
+                                     s)))
+            return rc;
+    }
+    if (stage_mask & GS355_STAGE_TILE_SCATTER)
+        if ((rc = launch_tile_scatter(fa, g->P, records, out->radii, header, bin_matrix, tile_base, buckets, s)))
+            return rc;
+    if (stage_mask & GS355_STAGE_TILESORT)
+        if ((rc = launch_tile_sort(header, tiles, ranges, tile_lists, buckets, keys[L.sorted_buffer],
+                                   vals[L.sorted_buffer], s)))
+            return rc;
     if (stage_mask & (GS355_STAGE_BLEND | GS355_STAGE_BLEND_PLAIN))
         if ((rc = launch_blend(fa, header, ranges, vals[L.sorted_buffer], records, out->image, out->depth, out->alpha,
                                (stage_mask & GS355_STAGE_BLEND) != 0, s)))
@@ -229,7 +259,7 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
 int gs355_render(const gs355_frame* frame, const gs355_gaussians* g, void* workspace, size_t workspace_bytes,
                  int64_t n_cap, const gs355_outputs* out, void* stream)
 {
-    return gs355_run(frame, g, workspace, workspace_bytes, n_cap, out, GS355_STAGE_ALL, stream);
+    return gs355_run(frame, g, workspace, workspace_bytes, n_cap, out, GS355_PIPELINE_FAST, stream);
 }
 
 int gs355_visible_filter(const gs355_frame* frame, const gs355_gaussians* g, int32_t* radii, void* stream)

@@ -1,0 +1,564 @@
+// Tile-bucketed sort for gfx950: the fast equivalent of "duplicate keys ->
+// radix sort -> tile ranges" of the rasterizer behind
+// GaussianRasterizer.forward (benchmarks/nerf/origin_gs/gs_model.py:211-220).
+//
+// The 64-bit key is (tile_id << 32 | depth bits).  Its high word is known when
+// a pair is generated, so the most significant digit is resolved by counting:
+// pairs are counted per tile, an exclusive scan of the counts gives every tile
+// its slot range (these ARE the per-tile ranges), and pairs are scattered into
+// their tile's bucket.  What remains is an independent sort of each bucket by
+// its low word, done by one workgroup per tile as an LSD radix sort staged
+// entirely in LDS (up to 9216 pairs in the 160 KB of a CU; larger buckets run
+// the same passes through global memory).  Bucket order after the scatter is
+// arbitrary, so pairs are ordered by (depth bits, Gaussian index): exactly the
+// order a stable sort of the emission-ordered keys produces.
+//
+// No workgroup waits on another; persistent loops run over fixed lists.
+#include "gs355_internal.h"
+
+namespace gs355 {
+
+namespace {
+
+constexpr int kInlineTiles = 32;  // splats touching more tiles than this are expanded by the whole workgroup
+
+// ---------------------------------------------------------------------------
+// Binning.  Workgroup c owns Gaussians [c * per_group, (c+1) * per_group) and a
+// private array of per-tile counters in LDS, so no global atomic is ever issued:
+//   count:   s_tile[t] = pairs of this slice that fall in tile t  -> matrix[c][t]
+//   scatter: s_tile[t] = first free slot of tile t for this slice (tile base +
+//            the slices before it), bumped per pair -> buckets[slot]
+// A thread walks the tile rectangle of its own Gaussian; rectangles of more
+// than kInlineTiles tiles are queued and walked by all threads together.
+template <bool kScatter>
+__global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P, int per_group,
+                                                          const float* __restrict__ records,
+                                                          const int32_t* __restrict__ radii,
+                                                          const gs355_header* __restrict__ header,
+                                                          uint32_t* __restrict__ matrix,
+                                                          const uint32_t* __restrict__ tile_base,
+                                                          uint32_t* __restrict__ group_visible,
+                                                          uint64_t* __restrict__ buckets)
+{
+    extern __shared__ uint32_t s_tile[];  // [tiles]
+    __shared__ uint32_t s_queue[kBinThreads];
+    __shared__ uint32_t s_nqueue, s_visible;
+
+    if (kScatter && header->overflow) return;
+    const int T = f.grid_x * f.grid_y;
+    const int tid = threadIdx.x, c = blockIdx.x;
+    uint32_t* __restrict__ row = matrix + (size_t)c * T;
+    for (int t = tid; t < T; t += kBinThreads) s_tile[t] = kScatter ? tile_base[t] + row[t] : 0u;
+    if (tid == 0) s_visible = 0;
+    const int g_begin = c * per_group;
+    const int g_end = min(P, g_begin + per_group);
+    uint32_t visible = 0;
+
+    for (int base = g_begin; base < g_end; base += kBinThreads) {
+        if (tid == 0) s_nqueue = 0;
+        __syncthreads();
+        const int i = base + tid;
+        if (i < g_end) {
+            const int rad = radii[i];
+            if (rad > 0) {
+                ++visible;
+                const float* __restrict__ rec = records + (size_t)i * kRecordFloats;
+                const Rect q = tile_rect(rec[0], rec[1], rad, f.grid_x, f.grid_y);
+                const int w = q.x1 - q.x0, area = w * (q.y1 - q.y0);
+                if (area > kInlineTiles) {
+                    s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
+                } else {
+                    const uint64_t payload = ((uint64_t)__float_as_uint(rec[9]) << 32) | (uint64_t)(uint32_t)i;
+                    for (int ty = q.y0; ty < q.y1; ++ty)
+                        for (int tx = q.x0; tx < q.x1; ++tx) {
+                            const uint32_t slot = atomicAdd(&s_tile[ty * f.grid_x + tx], 1u);
+                            if (kScatter) buckets[slot] = payload;
+                        }
+                }
+            }
+        }
+        __syncthreads();
+        const uint32_t nq = s_nqueue;
+        for (uint32_t k = 0; k < nq; ++k) {
+            const uint32_t gi = s_queue[k];
+            const float* __restrict__ rec = records + (size_t)gi * kRecordFloats;
+            const Rect q = tile_rect(rec[0], rec[1], radii[gi], f.grid_x, f.grid_y);
+            const int w = q.x1 - q.x0, area = w * (q.y1 - q.y0);
+            const uint64_t payload = ((uint64_t)__float_as_uint(rec[9]) << 32) | (uint64_t)gi;
+            for (int e = tid; e < area; e += kBinThreads) {
+                const int ty = q.y0 + e / w, tx = q.x0 + e % w;
+                const uint32_t slot = atomicAdd(&s_tile[ty * f.grid_x + tx], 1u);
+                if (kScatter) buckets[slot] = payload;
+            }
+        }
+        __syncthreads();
+    }
+    if (!kScatter) {
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) visible += __shfl_down(visible, d, 64);
+        if ((tid & 63) == 0 && visible) atomicAdd(&s_visible, visible);
+        __syncthreads();
+        for (int t = tid; t < T; t += kBinThreads) row[t] = s_tile[t];
+        if (tid == 0) group_visible[c] = s_visible;
+    }
+}
+
+// Thread per tile: exclusive prefix of the tile's counts over the slices (in
+// place) and the tile's total.
+__global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict__ matrix, int groups, int tiles,
+                                                           uint32_t* __restrict__ totals)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= tiles) return;
+    uint32_t run = 0;
+    int c = 0;
+    for (; c + 8 <= groups; c += 8) {
+        uint32_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = matrix[(size_t)(c + k) * tiles + t];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            matrix[(size_t)(c + k) * tiles + t] = run;
+            run += v[k];
+        }
+    }
+    for (; c < groups; ++c) {
+        const uint32_t v = matrix[(size_t)c * tiles + t];
+        matrix[(size_t)c * tiles + t] = run;
+        run += v;
+    }
+    totals[t] = run;
+}
+
+// One workgroup: tile totals -> tile bases, ranges, the frame header and the
+// lists of buckets too large for the small sorter.  `totals` and `tile_base`
+// may be the same array.
+__global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* totals, uint32_t tiles,
+                                                           const uint32_t* __restrict__ group_visible, int groups,
+                                                           uint32_t n_cap, gs355_header* __restrict__ header,
+                                                           uint32_t* tile_base, uint32_t* __restrict__ ranges,
+                                                           uint32_t* __restrict__ lists)
+{
+    __shared__ uint64_t s_wave[16];
+    __shared__ uint64_t s_carry;
+    __shared__ uint32_t s_nl, s_nxl, s_vis;
+    if (threadIdx.x == 0) {
+        s_carry = 0;
+        s_nl = 0;
+        s_nxl = 0;
+        s_vis = 0;
+    }
+    __syncthreads();
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // pass 1: grand total (decides overflow before any range is published)
+    uint64_t mine = 0;
+    for (uint32_t t = threadIdx.x; t < tiles; t += 1024) mine += totals[t];
+    uint32_t vis = 0;
+    for (int c = threadIdx.x; c < groups; c += 1024) vis += group_visible[c];
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+        mine += __shfl_down(mine, d, 64);
+        vis += __shfl_down(vis, d, 64);
+    }
+    if (lane == 0) {
+        s_wave[wave] = mine;
+        if (vis) atomicAdd(&s_vis, vis);
+    }
+    __syncthreads();
+    uint64_t total = 0;
+    for (int w = 0; w < 16; ++w) total += s_wave[w];
+    const bool overflow = total > (uint64_t)n_cap;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        header->num_keys_total = total;
+        header->num_keys = overflow ? n_cap : (uint32_t)total;
+        header->overflow = overflow ? 1u : 0u;
+        header->num_visible = s_vis;
+    }
+    // pass 2: exclusive scan of the totals (skipped on overflow: later stages do nothing then)
+    for (uint32_t base = 0; base < tiles && !overflow; base += 1024) {
+        const uint32_t t = base + threadIdx.x;
+        const uint32_t v = t < tiles ? totals[t] : 0u;
+        uint64_t inc = v;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint64_t up = __shfl_up(inc, d, 64);
+            if (lane >= d) inc += up;
+        }
+        if (lane == 63) s_wave[wave] = inc;
+        __syncthreads();
+        uint64_t off = s_carry;
+        for (int w = 0; w < wave; ++w) off += s_wave[w];
+        const uint32_t first = (uint32_t)(off + inc - v);
+        if (t < tiles) {
+            ranges[2 * t] = v ? first : 0u;
+            ranges[2 * t + 1] = v ? first + v : 0u;
+            tile_base[t] = first;
+            if (v > (uint32_t)kTileSortLargeCap) lists[2 + tiles + atomicAdd(&s_nxl, 1u)] = t;
+            else if (v > (uint32_t)kTileSortSmallCap) lists[2 + atomicAdd(&s_nl, 1u)] = t;
+        }
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = off + inc;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        lists[0] = s_nl;
+        lists[1] = s_nxl;
+    }
+}
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kRounds = 4;                      // 64-key rounds per wave per chunk
+constexpr int kChunk = kWaves * kRounds * 64;  // 1024 pairs ranked per iteration
+
+// ---------------------------------------------------------------------------
+// Storage of a bucket during sorting: two words per pair.
+struct LdsPairs {
+    uint32_t* d;  // depth bits
+    uint32_t* i;  // Gaussian index
+    __device__ __forceinline__ void load(uint32_t j, uint32_t& kd, uint32_t& ki) const
+    {
+        kd = d[j];
+        ki = i[j];
+    }
+    __device__ __forceinline__ void store(uint32_t j, uint32_t kd, uint32_t ki) const
+    {
+        d[j] = kd;
+        i[j] = ki;
+    }
+};
+
+struct GlobalPairs {
+    uint64_t* p;  // depth bits << 32 | Gaussian index
+    __device__ __forceinline__ void load(uint32_t j, uint32_t& kd, uint32_t& ki) const
+    {
+        const uint64_t v = p[j];
+        kd = (uint32_t)(v >> 32);
+        ki = (uint32_t)v;
+    }
+    __device__ __forceinline__ void store(uint32_t j, uint32_t kd, uint32_t ki) const
+    {
+        p[j] = ((uint64_t)kd << 32) | (uint64_t)ki;
+    }
+};
+
+struct SortScratch {
+    uint32_t* hist;           // [256] digit totals, then running digit bases
+    uint32_t (*cnt)[256];     // [kWaves][256] per-wave digit counts of the current chunk
+    uint32_t* flags;          // [8] small flags / partial sums
+};
+
+// One stable 8-bit LSD pass over n pairs, digit taken from the depth word
+// (by_depth) or the index word.  Returns false (and moves nothing) when every
+// pair has the same digit.
+template <typename Src, typename Dst>
+__device__ bool radix_pass(const Src src, const Dst dst, uint32_t n, int shift, bool by_depth, const SortScratch sc)
+{
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    sc.hist[tid] = 0;
+    if (tid < 8) sc.flags[tid] = 0;
+    __syncthreads();
+    for (uint32_t j = tid; j < n; j += kThreads) {
+        uint32_t kd, ki;
+        src.load(j, kd, ki);
+        atomicAdd(&sc.hist[((by_depth ? kd : ki) >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    {
+        // exclusive scan of the 256 digit totals; detect the single-digit case
+        const uint32_t h = sc.hist[tid];
+        uint32_t inc = h;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(inc, d, 64);
+            if (lane >= d) inc += up;
+        }
+        if (lane == 63) sc.flags[wave] = inc;
+        if (h == n) sc.flags[4] = 1;
+        __syncthreads();
+        uint32_t off = 0;
+        for (int w = 0; w < wave; ++w) off += sc.flags[w];
+        sc.hist[tid] = off + inc - h;
+        const bool single = sc.flags[4] != 0;
+        __syncthreads();
+        if (single) return false;
+    }
+    const uint64_t lanes_below = (1ull << lane) - 1ull;
+    for (uint32_t c0 = 0; c0 < n; c0 += kChunk) {
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) sc.cnt[w][tid] = 0;
+        __syncthreads();
+        uint32_t kd[kRounds], ki[kRounds], rank[kRounds];
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r) {
+            const uint32_t j = c0 + (uint32_t)(wave * kRounds + r) * 64u + lane;
+            const bool valid = j < n;
+            kd[r] = 0;
+            ki[r] = 0;
+            if (valid) src.load(j, kd[r], ki[r]);
+            const uint32_t dgt = ((by_depth ? kd[r] : ki[r]) >> shift) & 255u;
+            uint64_t peers = __ballot(valid);
+#pragma unroll
+            for (int bit = 0; bit < 8; ++bit) {
+                const bool one = (dgt >> bit) & 1u;
+                const uint64_t m = __ballot(one);
+                peers &= one ? m : ~m;
+            }
+            uint32_t pre = 0;
+            const uint32_t below = (uint32_t)__popcll(peers & lanes_below);
+            if (valid) {
+                const int leader = __ffsll((unsigned long long)peers) - 1;
+                if (lane == leader) pre = atomicAdd(&sc.cnt[wave][dgt], (uint32_t)__popcll(peers));
+                pre = __shfl(pre, leader, 64);
+            }
+            rank[r] = pre + below;
+        }
+        __syncthreads();
+        {
+            uint32_t run = sc.hist[tid];
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                const uint32_t c = sc.cnt[w][tid];
+                sc.cnt[w][tid] = run;
+                run += c;
+            }
+            sc.hist[tid] = run;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r) {
+            const uint32_t j = c0 + (uint32_t)(wave * kRounds + r) * 64u + lane;
+            if (j < n) {
+                const uint32_t dgt = ((by_depth ? kd[r] : ki[r]) >> shift) & 255u;
+                dst.store(sc.cnt[wave][dgt] + rank[r], kd[r], ki[r]);
+            }
+        }
+        __syncthreads();
+    }
+    return true;
+}
+
+// Sort n pairs held in buffer A (B is scratch of the same size) by
+// (depth bits, index).  Returns true if the result is in B.
+template <typename Buf>
+__device__ bool sort_pairs(const Buf A, const Buf B, uint32_t n, const SortScratch sc)
+{
+    bool in_b = false;
+    // depth passes; pairs of one tile rarely share depth bits, so the index
+    // word is only brought in when a tie is actually present
+    for (int pass = 0; pass < 4; ++pass) {
+        const bool moved = in_b ? radix_pass(B, A, n, pass * 8, true, sc) : radix_pass(A, B, n, pass * 8, true, sc);
+        if (moved) in_b = !in_b;
+    }
+    {
+        const Buf cur = in_b ? B : A;
+        if (threadIdx.x == 0) sc.flags[5] = 0;
+        __syncthreads();
+        bool tie = false;
+        for (uint32_t j = threadIdx.x; j + 1 < n; j += kThreads) {
+            uint32_t d0, i0, d1, i1;
+            cur.load(j, d0, i0);
+            cur.load(j + 1, d1, i1);
+            tie |= (d0 == d1) && (i0 > i1);
+        }
+        if (tie) sc.flags[5] = 1;
+        __syncthreads();
+        const bool any = sc.flags[5] != 0;
+        __syncthreads();
+        if (!any) return in_b;
+    }
+    // equal depth bits out of index order: full (index, then depth) stable sort
+    for (int pass = 0; pass < 8; ++pass) {
+        const bool by_depth = pass >= 4;
+        const int shift = (pass & 3) * 8;
+        const bool moved = in_b ? radix_pass(B, A, n, shift, by_depth, sc) : radix_pass(A, B, n, shift, by_depth, sc);
+        if (moved) in_b = !in_b;
+    }
+    return in_b;
+}
+
+template <typename Buf>
+__device__ __forceinline__ void write_sorted(const Buf cur, uint32_t n, uint32_t tile, uint64_t* out_keys,
+                                             uint32_t* out_vals)
+{
+    for (uint32_t j = threadIdx.x; j < n; j += kThreads) {
+        uint32_t kd, ki;
+        cur.load(j, kd, ki);
+        out_keys[j] = ((uint64_t)tile << 32) | (uint64_t)kd;
+        out_vals[j] = ki;
+    }
+}
+
+__device__ __forceinline__ void sort_tile_in_lds(uint32_t tile, const uint32_t* __restrict__ ranges,
+                                                 const uint64_t* __restrict__ buckets, uint64_t* __restrict__ out_keys,
+                                                 uint32_t* __restrict__ out_vals, uint32_t* lds, uint32_t cap,
+                                                 uint32_t n_min, const SortScratch sc)
+{
+    const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
+    const uint32_t n = hi - lo;
+    if (n <= n_min || n > cap) return;  // uniform over the workgroup
+    const LdsPairs A = {lds, lds + cap}, B = {lds + 2 * cap, lds + 3 * cap};
+    for (uint32_t j = threadIdx.x; j < n; j += kThreads) {
+        const uint64_t v = buckets[lo + j];
+        A.store(j, (uint32_t)(v >> 32), (uint32_t)v);
+    }
+    __syncthreads();
+    const bool in_b = sort_pairs(A, B, n, sc);
+    write_sorted(in_b ? B : A, n, tile, out_keys + lo, out_vals + lo);
+    __syncthreads();
+}
+
+// Buckets of up to kTileSortSmallCap pairs: one workgroup per tile, 36 KB of LDS.
+__global__ __launch_bounds__(kThreads) void tile_sort_small_kernel(const gs355_header* __restrict__ header,
+                                                                   const uint32_t* __restrict__ ranges,
+                                                                   const uint64_t* __restrict__ buckets,
+                                                                   uint64_t* __restrict__ out_keys,
+                                                                   uint32_t* __restrict__ out_vals)
+{
+    __shared__ uint32_t s_pairs[4 * kTileSortSmallCap];
+    __shared__ uint32_t s_hist[256];
+    __shared__ uint32_t s_cnt[kWaves][256];
+    __shared__ uint32_t s_flags[8];
+    if (header->overflow) return;
+    const SortScratch sc = {s_hist, s_cnt, s_flags};
+    sort_tile_in_lds(blockIdx.x, ranges, buckets, out_keys, out_vals, s_pairs, kTileSortSmallCap, 0u, sc);
+}
+
+// Buckets of up to kTileSortLargeCap pairs: persistent workgroups over the list
+// made by tile_layout_kernel, ~148 KB of dynamic LDS each (one per CU).
+__global__ __launch_bounds__(kThreads) void tile_sort_large_kernel(const gs355_header* __restrict__ header,
+                                                                   const uint32_t* __restrict__ ranges,
+                                                                   const uint32_t* __restrict__ lists,
+                                                                   const uint64_t* __restrict__ buckets,
+                                                                   uint64_t* __restrict__ out_keys,
+                                                                   uint32_t* __restrict__ out_vals)
+{
+    extern __shared__ uint32_t s_dyn[];
+    __shared__ uint32_t s_hist[256];
+    __shared__ uint32_t s_cnt[kWaves][256];
+    __shared__ uint32_t s_flags[8];
+    if (header->overflow) return;
+    const SortScratch sc = {s_hist, s_cnt, s_flags};
+    const uint32_t count = lists[0];
+    for (uint32_t k = blockIdx.x; k < count; k += gridDim.x)
+        sort_tile_in_lds(lists[2 + k], ranges, buckets, out_keys, out_vals, s_dyn, kTileSortLargeCap,
+                         kTileSortSmallCap, sc);
+}
+
+// Buckets beyond the LDS capacity: the same passes through global memory,
+// ping-ponging between the bucket and the tile's slice of the output keys.
+__global__ __launch_bounds__(kThreads) void tile_sort_huge_kernel(const gs355_header* __restrict__ header,
+                                                                  const uint32_t* __restrict__ ranges,
+                                                                  const uint32_t* __restrict__ lists, uint32_t tiles,
+                                                                  uint64_t* __restrict__ buckets,
+                                                                  uint64_t* __restrict__ out_keys,
+                                                                  uint32_t* __restrict__ out_vals)
+{
+    __shared__ uint32_t s_hist[256];
+    __shared__ uint32_t s_cnt[kWaves][256];
+    __shared__ uint32_t s_flags[8];
+    if (header->overflow) return;
+    const SortScratch sc = {s_hist, s_cnt, s_flags};
+    const uint32_t count = lists[1];
+    for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) {
+        const uint32_t tile = lists[2 + tiles + k];
+        const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
+        const GlobalPairs A = {buckets + lo}, B = {out_keys + lo};
+        const bool in_b = sort_pairs(A, B, n, sc);
+        // when the result sits in the output slice itself, each element is
+        // rewritten in place by the thread that read it
+        write_sorted(in_b ? B : A, n, tile, out_keys + lo, out_vals + lo);
+        __syncthreads();
+    }
+}
+
+}  // namespace
+
+int bin_groups(int32_t P, int* per_group)
+{
+    // slices are multiples of the workgroup size so that every pass over a slice is full
+    int per = (P + kBinMaxGroups - 1) / kBinMaxGroups;
+    per = (per + kBinThreads - 1) / kBinThreads * kBinThreads;
+    if (per < kBinThreads) per = kBinThreads;
+    *per_group = per;
+    const int groups = (P + per - 1) / per;
+    return groups < 1 ? 1 : groups;
+}
+
+static int set_bin_lds(const void* fn, size_t bytes)
+{
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return set_error(GS355_EHIP, "bin: LDS attribute: %s", hipGetErrorString(e));
+    return GS355_OK;
+}
+
+int launch_tile_count(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii, uint32_t* matrix,
+                      uint32_t* group_visible, hipStream_t s)
+{
+    int per_group;
+    const int groups = bin_groups(P, &per_group);
+    const size_t lds = (size_t)f.grid_x * f.grid_y * sizeof(uint32_t);
+    int rc = set_bin_lds(reinterpret_cast<const void*>(bin_kernel<false>), lds);
+    if (rc) return rc;
+    hipLaunchKernelGGL(bin_kernel<false>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, records, radii,
+                       (const gs355_header*)nullptr, matrix, (const uint32_t*)nullptr, group_visible,
+                       (uint64_t*)nullptr);
+    GS355_CHECK_LAUNCH("bin: count");
+    return GS355_OK;
+}
+
+int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visible, int tiles, uint32_t n_cap,
+                       gs355_header* header, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s)
+{
+    int per_group;
+    const int groups = bin_groups(P, &per_group);
+    hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 255) / 256), dim3(256), 0, s, matrix, groups, tiles,
+                       tile_base);
+    GS355_CHECK_LAUNCH("bin: slice prefix");
+    hipLaunchKernelGGL(tile_layout_kernel, dim3(1), dim3(1024), 0, s, tile_base, (uint32_t)tiles, group_visible, groups,
+                       n_cap, header, tile_base, ranges, lists);
+    GS355_CHECK_LAUNCH("bin: layout");
+    return GS355_OK;
+}
+
+int launch_tile_scatter(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
+                        const gs355_header* header, const uint32_t* matrix, const uint32_t* tile_base,
+                        uint64_t* buckets, hipStream_t s)
+{
+    int per_group;
+    const int groups = bin_groups(P, &per_group);
+    const size_t lds = (size_t)f.grid_x * f.grid_y * sizeof(uint32_t);
+    int rc = set_bin_lds(reinterpret_cast<const void*>(bin_kernel<true>), lds);
+    if (rc) return rc;
+    hipLaunchKernelGGL(bin_kernel<true>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, records, radii,
+                       header, const_cast<uint32_t*>(matrix), tile_base, (uint32_t*)nullptr, buckets);
+    GS355_CHECK_LAUNCH("bin: scatter");
+    return GS355_OK;
+}
+
+int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, const uint32_t* lists,
+                     uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, hipStream_t s)
+{
+    hipLaunchKernelGGL(tile_sort_small_kernel, dim3(tiles), dim3(kThreads), 0, s, header, ranges, buckets, out_keys,
+                       out_vals);
+    GS355_CHECK_LAUNCH("tile sort: small");
+    static bool attr_set = false;  // idempotent; a race only repeats the call
+    const size_t dyn = (size_t)4 * kTileSortLargeCap * sizeof(uint32_t);
+    if (!attr_set) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(tile_sort_large_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+        if (e != hipSuccess) return set_error(GS355_EHIP, "tile sort: LDS attribute: %s", hipGetErrorString(e));
+        attr_set = true;
+    }
+    const int persistent = tiles < 256 ? tiles : 256;
+    hipLaunchKernelGGL(tile_sort_large_kernel, dim3(persistent), dim3(kThreads), dyn, s, header, ranges, lists, buckets,
+                       out_keys, out_vals);
+    GS355_CHECK_LAUNCH("tile sort: large");
+    hipLaunchKernelGGL(tile_sort_huge_kernel, dim3(persistent), dim3(kThreads), 0, s, header, ranges, lists,
+                       (uint32_t)tiles, buckets, out_keys, out_vals);
+    GS355_CHECK_LAUNCH("tile sort: huge");
+    return GS355_OK;
+}
+
+}  // namespace gs355

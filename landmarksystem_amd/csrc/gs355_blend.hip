@@ -166,12 +166,19 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
 
 }  // namespace
 
+int launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t s)
+{
+    if (n == 0) return GS355_OK;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
+    GS355_CHECK_LAUNCH("fill");
+    return GS355_OK;
+}
+
 int launch_ranges(const gs355_header* header, uint32_t n_cap, const uint64_t* keys, uint32_t* ranges, int tiles,
                   hipStream_t s)
 {
-    const size_t words = (size_t)tiles * 2;
-    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, ranges, words, 0u);
-    GS355_CHECK_LAUNCH("ranges: clear");
+    const int rc = launch_fill_u32(ranges, (size_t)tiles * 2, 0u, s);
+    if (rc) return rc;
     if (n_cap == 0) return GS355_OK;
     hipLaunchKernelGGL(ranges_kernel, dim3((n_cap + 255) / 256), dim3(256), 0, s, header, keys, ranges,
                        (uint32_t)tiles);

@@ -17,6 +17,10 @@ constexpr int kSortTile = kSortThreads * kSortItems;
 constexpr int kRadixBits = 8;
 constexpr int kRadix = 1 << kRadixBits;
 
+// tile-bucketed sort: bucket sizes handled in static LDS / dynamic LDS (148 KB); larger go through global memory
+constexpr int kTileSortSmallCap = 2048;
+constexpr int kTileSortLargeCap = 9216;
+
 // scan geometry: 256 threads x 16 items per workgroup
 constexpr int kScanThreads = 256;
 constexpr int kScanItems = 16;
@@ -34,6 +38,32 @@ struct FrameArgs {  // by-value kernel argument
 
 int set_error(int code, const char* fmt, ...);
 
+// Tile rectangle of a splat.  Only subtractions, additions and divisions by 16:
+// nothing a compiler could contract, so every translation unit gets the same
+// rectangle from the same (px, py, radius).
+struct Rect {
+    int x0, y0, x1, y1;
+};
+
+// min(grid, max(0, (int)v)) with truncation toward zero, defined for any v.
+__device__ __forceinline__ int tile_clamp(float v, int grid)
+{
+    if (!(v > 0.0f)) return 0;
+    if (v >= (float)grid) return grid;
+    return (int)v;
+}
+
+__device__ __forceinline__ Rect tile_rect(float px, float py, int radius, int grid_x, int grid_y)
+{
+    const float r = (float)radius;
+    Rect q;
+    q.x0 = tile_clamp((px - r) / 16.0f, grid_x);
+    q.y0 = tile_clamp((py - r) / 16.0f, grid_y);
+    q.x1 = tile_clamp((px + r + 15.0f) / 16.0f, grid_x);
+    q.y1 = tile_clamp((py + r + 15.0f) / 16.0f, grid_y);
+    return q;
+}
+
 // stage launchers (each returns a gs355_status)
 int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_only, float* records,
                       uint32_t* tiles_touched, int32_t* radii, hipStream_t s);
@@ -48,6 +78,23 @@ int launch_ranges(const gs355_header* header, uint32_t n_cap, const uint64_t* ke
                   hipStream_t s);
 int launch_blend(const FrameArgs& f, const gs355_header* header, const uint32_t* ranges, const uint32_t* values, const float* records,
                  float* image, float* depth, float* alpha, bool cull, hipStream_t s);
+
+int launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t s);
+
+// tile-bucketed path
+constexpr int kBinThreads = 1024;       // threads per binning workgroup
+constexpr int kBinMaxGroups = 512;      // binning workgroups (each owns a contiguous slice of the Gaussians)
+constexpr int kBinMaxTiles = 36000;     // per-tile counters of one workgroup must fit in LDS (4 B each)
+int bin_groups(int32_t P, int* per_group);
+int launch_tile_count(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii, uint32_t* matrix,
+                      uint32_t* group_visible, hipStream_t s);
+int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visible, int tiles, uint32_t n_cap,
+                       gs355_header* header, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s);
+int launch_tile_scatter(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
+                        const gs355_header* header, const uint32_t* matrix, const uint32_t* tile_base,
+                        uint64_t* buckets, hipStream_t s);
+int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, const uint32_t* lists,
+                     uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, hipStream_t s);
 
 // generic exclusive scan of u32 (n <= 2^32-1); tmp needs scan_tmp_words(n) words
 size_t scan_tmp_words(size_t n);

@@ -25,29 +25,6 @@ constexpr float kShC3[7] = {-0.5900435899266435f, 2.890611442640554f, -0.4570457
                             0.3731763325901154f, -0.4570457994644658f, 1.445305721320277f,
                             -0.5900435899266435f};
 
-struct Rect {
-    int x0, y0, x1, y1;
-};
-
-// min(grid, max(0, (int)v)) with truncation toward zero, defined for any v.
-__device__ __forceinline__ int tile_clamp(float v, int grid)
-{
-    if (!(v > 0.0f)) return 0;
-    if (v >= (float)grid) return grid;
-    return (int)v;
-}
-
-__device__ __forceinline__ Rect tile_rect(float px, float py, int radius, int grid_x, int grid_y)
-{
-    const float r = (float)radius;
-    Rect q;
-    q.x0 = tile_clamp((px - r) / 16.0f, grid_x);
-    q.y0 = tile_clamp((py - r) / 16.0f, grid_y);
-    q.x1 = tile_clamp((px + r + 15.0f) / 16.0f, grid_x);
-    q.y1 = tile_clamp((py + r + 15.0f) / 16.0f, grid_y);
-    return q;
-}
-
 // 3D covariance, packed upper triangle, from scale and (r,x,y,z) quaternion.
 __device__ __forceinline__ void covariance3d(const float* __restrict__ scale, float mod,
                                              const float* __restrict__ quat, float cov[6])
@@ -273,8 +250,7 @@ __global__ __launch_bounds__(256) void duplicate_kernel(FrameArgs f, int32_t P, 
         const int w = s_w[lo];
         const int ty = s_y0[lo] + (int)(local / (uint32_t)w);
         const int tx = s_x0[lo] + (int)(local % (uint32_t)w);
-        const uint64_t key = ((uint64_t)(uint32_t)(ty * f.grid_x + tx) << 32) | (uint64_t)s_depth[lo];
-        keys[j] = key;
+        keys[j] = ((uint64_t)(uint32_t)(ty * f.grid_x + tx) << 32) | (uint64_t)s_depth[lo];
         values[j] = (uint32_t)(g0 + lo);
     }
 }

@@ -205,8 +205,12 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
     out = FrameOutputs(inputs, want_depth, want_alpha)
     if ws.key_capacity == 0:
         ws.key_capacity = max(1 << 20, 4 * inputs.P)
-    front = _lib.STAGE_PREPROCESS | _lib.STAGE_SCAN
-    back = _lib.STAGE_DUPLICATE | _lib.STAGE_SORT | _lib.STAGE_RANGES | _lib.STAGE_BLEND
+    if inputs.tiles <= _lib.MAX_FAST_TILES:
+        front = _lib.STAGE_PREPROCESS | _lib.STAGE_TILE_COUNT
+        back = _lib.STAGE_TILE_SCATTER | _lib.STAGE_TILESORT | _lib.STAGE_BLEND
+    else:  # per-tile counters would not fit in LDS: classic duplicate / radix sort / ranges
+        front = _lib.STAGE_PREPROCESS | _lib.STAGE_SCAN
+        back = _lib.STAGE_DUPLICATE | _lib.STAGE_SORT | _lib.STAGE_RANGES | _lib.STAGE_BLEND
     for attempt in range(3):
         n_cap = ws.key_capacity
         layout = run_stages(inputs, out, ws, n_cap, front)

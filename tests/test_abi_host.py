@@ -32,14 +32,14 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(_lib.Frame) == 7 * 4 + 4 + 4 * 8  # 7 scalars, padding to 8, 4 pointers
     assert C.sizeof(_lib.Gaussians) == 8 + 7 * 8
     assert C.sizeof(_lib.Outputs) == 4 * 8
-    assert C.sizeof(_lib.Layout) == 12 * 8 + 4 * 4
+    assert C.sizeof(_lib.Layout) == 16 * 8 + 4 * 4
 
 
 def test_workspace_layout_is_aligned_ordered_and_sized():
     P, n_cap, W, H = 100_000, 1_500_000, 1920, 1080
     L = _lib.workspace_layout(P, n_cap, W, H)
     offs = [L.header, L.records, L.tiles_touched, L.offsets, L.scan_tmp, L.keys[0], L.keys[1], L.values[0],
-            L.values[1], L.sort_hist, L.ranges, L.total_bytes]
+            L.values[1], L.sort_hist, L.ranges, L.bin_matrix, L.tile_base, L.bin_visible, L.tile_lists, L.total_bytes]
     assert all(o % 256 == 0 for o in offs)
     assert offs == sorted(offs) and len(set(offs)) == len(offs)
     assert L.records - L.header >= 64
@@ -47,7 +47,8 @@ def test_workspace_layout_is_aligned_ordered_and_sized():
     assert L.keys[1] - L.keys[0] >= n_cap * 8
     assert L.values[1] - L.values[0] >= n_cap * 4
     tiles = 120 * 68
-    assert L.total_bytes - L.ranges >= tiles * 8
+    assert L.bin_matrix - L.ranges >= tiles * 8 and L.total_bytes - L.tile_lists >= (2 + 2 * tiles) * 4
+    assert L.tile_base - L.bin_matrix >= 512 * tiles * 4
     assert L.sort_bits == 32 + 13 and L.sort_passes == 6 and L.sorted_buffer == 0
     L4k = _lib.workspace_layout(10, 10, 3840, 2160)
     assert L4k.sort_bits == 47 and L4k.sort_passes == 6
@@ -108,7 +109,7 @@ def test_run_validates_before_any_hip_call():
     assert "frame is NULL" in _err(_lib.GS355_EINVAL, run, None, g, 0x1000, 1 << 30, 100, out, _lib.STAGE_ALL)
     assert "gaussians is NULL" in _err(_lib.GS355_EINVAL, run, f, None, 0x1000, 1 << 30, 100, out, _lib.STAGE_ALL)
     assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 0)
-    assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 128)
+    assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 1024)
     assert "SHs or precomputed colors" in _err(_lib.GS355_EINVAL, run, f, _gauss(shs=True, colors=True), 0x1000,
                                                 1 << 30, 100, out, _lib.STAGE_ALL)
     assert "SHs or precomputed colors" in _err(_lib.GS355_EINVAL, run, f, _gauss(shs=False, colors=False), 0x1000,

@@ -116,7 +116,7 @@ typedef struct gs355_layout {
     size_t bin_matrix;    /* u32[slices][tiles] pairs per (slice of Gaussians, tile), then their prefix over slices */
     size_t tile_base;     /* u32[tiles]      first slot of each tile's bucket */
     size_t bin_visible;   /* u32[slices]     visible Gaussians per slice */
-    size_t tile_lists;    /* u32[2+2*tiles]  counts and lists of buckets too large for the small sorter */
+    size_t tile_lists;    /* u32[4+4*tiles]  counts and lists of the buckets of each larger sorter size class */
     size_t total_bytes;
     int32_t unsorted_buffer; /* which keys/values buffer the duplicate stage writes (0) */
     int32_t sorted_buffer;   /* which buffer holds the sorted pairs after the sort stage */

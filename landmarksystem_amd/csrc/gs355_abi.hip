@@ -84,7 +84,7 @@ int make_layout(int32_t P, int64_t n_cap, int32_t W, int32_t H, gs355_layout* L)
     L->bin_matrix = take(slices * tiles * sizeof(uint32_t));
     L->tile_base = take(tiles * sizeof(uint32_t));
     L->bin_visible = take((size_t)kBinMaxGroups * sizeof(uint32_t));
-    L->tile_lists = take((2 + 2 * tiles) * sizeof(uint32_t));
+    L->tile_lists = take((4 + 4 * tiles) * sizeof(uint32_t));
     L->total_bytes = off;
     L->sort_bits = 32 + ceil_log2((uint32_t)tiles);
     L->sort_passes = (L->sort_bits + kRadixBits - 1) / kRadixBits;

@@ -141,11 +141,10 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
 {
     __shared__ uint64_t s_wave[16];
     __shared__ uint64_t s_carry;
-    __shared__ uint32_t s_nl, s_nxl, s_vis;
+    __shared__ uint32_t s_nlist[4], s_vis;
     if (threadIdx.x == 0) {
         s_carry = 0;
-        s_nl = 0;
-        s_nxl = 0;
+        s_nlist[0] = s_nlist[1] = s_nlist[2] = s_nlist[3] = 0;
         s_vis = 0;
     }
     __syncthreads();
@@ -194,17 +193,19 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
             ranges[2 * t] = v ? first : 0u;
             ranges[2 * t + 1] = v ? first + v : 0u;
             tile_base[t] = first;
-            if (v > (uint32_t)kTileSortLargeCap) lists[2 + tiles + atomicAdd(&s_nxl, 1u)] = t;
-            else if (v > (uint32_t)kTileSortSmallCap) lists[2 + atomicAdd(&s_nl, 1u)] = t;
+            // buckets beyond the smallest sorter's capacity go on the list of their size class
+            int cls = -1;
+            if (v > (uint32_t)kTileSortCap[3]) cls = 3;
+            else if (v > (uint32_t)kTileSortCap[2]) cls = 2;
+            else if (v > (uint32_t)kTileSortCap[1]) cls = 1;
+            else if (v > (uint32_t)kTileSortCap[0]) cls = 0;
+            if (cls >= 0) lists[4 + (size_t)cls * tiles + atomicAdd(&s_nlist[cls], 1u)] = t;
         }
         __syncthreads();
         if (threadIdx.x == 1023) s_carry = off + inc;
         __syncthreads();
     }
-    if (threadIdx.x == 0) {
-        lists[0] = s_nl;
-        lists[1] = s_nxl;
-    }
+    if (threadIdx.x < 4) lists[threadIdx.x] = s_nlist[threadIdx.x];
 }
 
 constexpr int kThreads = 256;
@@ -390,60 +391,237 @@ __device__ __forceinline__ void write_sorted(const Buf cur, uint32_t n, uint32_t
     }
 }
 
-__device__ __forceinline__ void sort_tile_in_lds(uint32_t tile, const uint32_t* __restrict__ ranges,
-                                                 const uint64_t* __restrict__ buckets, uint64_t* __restrict__ out_keys,
-                                                 uint32_t* __restrict__ out_vals, uint32_t* lds, uint32_t cap,
-                                                 uint32_t n_min, const SortScratch sc)
-{
-    const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
-    const uint32_t n = hi - lo;
-    if (n <= n_min || n > cap) return;  // uniform over the workgroup
-    const LdsPairs A = {lds, lds + cap}, B = {lds + 2 * cap, lds + 3 * cap};
-    for (uint32_t j = threadIdx.x; j < n; j += kThreads) {
-        const uint64_t v = buckets[lo + j];
-        A.store(j, (uint32_t)(v >> 32), (uint32_t)v);
+// ---------------------------------------------------------------------------
+// In-LDS bucket sorter: kT threads, up to kT * kR pairs, every pass ranks the
+// whole bucket at once (each wavefront owns kR * 64 consecutive positions).
+// LDS holds the bucket once (depth bits, index: 8 B per pair) plus two 16-bit
+// permutations that ping-pong between passes (4 B per pair).
+template <int kT, int kR>
+struct LdsSorter {
+    static constexpr int kW = kT / 64;
+    static constexpr int kCap = kT * kR;
+    static constexpr size_t kBytes = (size_t)kCap * 12 + (size_t)kW * 256 * 4 + 64;
+
+    uint32_t* depth;     // [kCap]
+    uint32_t* index;     // [kCap]
+    uint16_t* perm0;     // two permutations of [kCap] each, back to back
+    uint32_t (*cnt)[256];  // [kW][256]
+    uint32_t* flags;     // [16]
+
+    __device__ explicit LdsSorter(uint32_t* lds)
+    {
+        depth = lds;
+        index = lds + kCap;
+        perm0 = reinterpret_cast<uint16_t*>(lds + 2 * kCap);
+        cnt = reinterpret_cast<uint32_t(*)[256]>(lds + 3 * kCap);
+        flags = lds + 3 * kCap + kW * 256;
     }
-    __syncthreads();
-    const bool in_b = sort_pairs(A, B, n, sc);
-    write_sorted(in_b ? B : A, n, tile, out_keys + lo, out_vals + lo);
-    __syncthreads();
-}
 
-// Buckets of up to kTileSortSmallCap pairs: one workgroup per tile, 36 KB of LDS.
-__global__ __launch_bounds__(kThreads) void tile_sort_small_kernel(const gs355_header* __restrict__ header,
-                                                                   const uint32_t* __restrict__ ranges,
-                                                                   const uint64_t* __restrict__ buckets,
-                                                                   uint64_t* __restrict__ out_keys,
-                                                                   uint32_t* __restrict__ out_vals)
-{
-    __shared__ uint32_t s_pairs[4 * kTileSortSmallCap];
-    __shared__ uint32_t s_hist[256];
-    __shared__ uint32_t s_cnt[kWaves][256];
-    __shared__ uint32_t s_flags[8];
-    if (header->overflow) return;
-    const SortScratch sc = {s_hist, s_cnt, s_flags};
-    sort_tile_in_lds(blockIdx.x, ranges, buckets, out_keys, out_vals, s_pairs, kTileSortSmallCap, 0u, sc);
-}
+    __device__ __forceinline__ uint16_t* perm(int which) const { return perm0 + which * kCap; }
 
-// Buckets of up to kTileSortLargeCap pairs: persistent workgroups over the list
-// made by tile_layout_kernel, ~148 KB of dynamic LDS each (one per CU).
-__global__ __launch_bounds__(kThreads) void tile_sort_large_kernel(const gs355_header* __restrict__ header,
-                                                                   const uint32_t* __restrict__ ranges,
-                                                                   const uint32_t* __restrict__ lists,
-                                                                   const uint64_t* __restrict__ buckets,
-                                                                   uint64_t* __restrict__ out_keys,
-                                                                   uint32_t* __restrict__ out_vals)
+    // One stable pass.  `src` < 0: the input order is the identity.  Returns the
+    // buffer holding the output order (unchanged when all digits are equal).
+    __device__ int pass(uint32_t n, int shift, bool by_depth, int src) const
+    {
+        const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+        for (int k = tid; k < kW * 256; k += kT) (&cnt[0][0])[k] = 0;
+        if (tid == 0) flags[8] = 0;
+        __syncthreads();
+        const int dst = src == 0 ? 1 : 0;
+        const uint64_t lanes_below = (1ull << lane) - 1ull;
+        uint32_t ent[kR];  // entry | digit << 16
+        uint32_t rank[kR];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            ent[r] = 0;
+            rank[r] = 0;
+            if ((uint32_t)(wave * kR + r) * 64u >= n) continue;  // whole round past the end (uniform per wavefront)
+            const uint32_t j = (uint32_t)(wave * kR + r) * 64u + lane;
+            const bool valid = j < n;
+            const uint32_t e = valid ? (src < 0 ? j : (uint32_t)perm(src)[j]) : 0u;
+            const uint32_t key = valid ? (by_depth ? depth[e] : index[e]) : 0u;
+            const uint32_t dgt = (key >> shift) & 255u;
+            uint64_t peers = __ballot(valid);
+#pragma unroll
+            for (int bit = 0; bit < 8; ++bit) {
+                const bool one = (dgt >> bit) & 1u;
+                const uint64_t m = __ballot(one);
+                peers &= one ? m : ~m;
+            }
+            uint32_t pre = 0;
+            const uint32_t below = (uint32_t)__popcll(peers & lanes_below);
+            if (valid) {
+                const int leader = __ffsll((unsigned long long)peers) - 1;
+                if (lane == leader) pre = atomicAdd(&cnt[wave][dgt], (uint32_t)__popcll(peers));
+                pre = __shfl(pre, leader, 64);
+            }
+            rank[r] = pre + below;
+            ent[r] = e | (dgt << 16);
+        }
+        __syncthreads();
+        // digit totals, exclusive scan over the 256 digits (wavefronts 0..3), per-wave bases
+        uint32_t total = 0, inc = 0;
+        if (tid < 256) {
+#pragma unroll
+            for (int w = 0; w < kW; ++w) total += cnt[w][tid];
+            if (total == n) flags[8] = 1;  // every pair has this digit: nothing to move
+            inc = total;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t up = __shfl_up(inc, d, 64);
+                if (lane >= d) inc += up;
+            }
+            if (lane == 63) flags[wave] = inc;
+        }
+        __syncthreads();
+        if (tid < 256) {
+            uint32_t base = inc - total;
+            for (int w = 0; w < wave; ++w) base += flags[w];
+#pragma unroll
+            for (int w = 0; w < kW; ++w) {
+                const uint32_t c = cnt[w][tid];
+                cnt[w][tid] = base;
+                base += c;
+            }
+        }
+        __syncthreads();
+        const bool single = flags[8] != 0;
+        if (!single) {
+#pragma unroll
+            for (int r = 0; r < kR; ++r) {
+                const uint32_t j = (uint32_t)(wave * kR + r) * 64u + lane;
+                if (j < n) perm(dst)[cnt[wave][ent[r] >> 16] + rank[r]] = (uint16_t)ent[r];
+            }
+        }
+        __syncthreads();
+        return single ? src : dst;
+    }
+
+    // Sort the n loaded pairs by (depth bits, index); returns the buffer with
+    // the final order.
+    __device__ int sort(uint32_t n, uint32_t varying) const
+    {
+        int cur = -1;
+        // bytes of the depth word that are identical in every pair need no pass
+        // (inside one tile the exponent byte of the depths usually is)
+        for (int p = 0; p < 4; ++p)
+            if ((varying >> (p * 8)) & 255u) cur = pass(n, p * 8, true, cur);
+        if (cur < 0) {  // no pass moved anything (all depth bits equal, or n == 1): start from the identity
+            for (uint32_t j = threadIdx.x; j < n; j += kT) perm(0)[j] = (uint16_t)j;
+            cur = 0;
+            __syncthreads();
+        }
+        // Bucket order before the sort is arbitrary, so pairs with equal depth
+        // bits may be out of index order.  Such runs are rare and short: a few
+        // rounds of odd-even transposition inside runs settle them; only if a
+        // round still swaps after that is the full (index, depth) sort run.
+        uint16_t* const P = perm(cur);
+        bool unsettled = true;
+        for (int round = 0; round < 4 && unsettled; ++round) {
+            if (threadIdx.x == 0) flags[10] = 0;
+            __syncthreads();
+            bool swapped = false;
+            for (int phase = 0; phase < 2; ++phase) {
+                for (uint32_t j = 2u * threadIdx.x + phase; j + 1 < n; j += 2u * kT) {
+                    const uint32_t e0 = P[j], e1 = P[j + 1];
+                    if (depth[e0] == depth[e1] && index[e0] > index[e1]) {
+                        P[j] = (uint16_t)e1;
+                        P[j + 1] = (uint16_t)e0;
+                        swapped = true;
+                    }
+                }
+                __syncthreads();
+            }
+            if (swapped) flags[10] = 1;
+            __syncthreads();
+            unsettled = flags[10] != 0;
+            __syncthreads();
+        }
+        if (!unsettled) return cur;
+        for (int p = 0; p < 8; ++p) cur = pass(n, (p & 3) * 8, p >= 4, cur);
+        return cur;
+    }
+
+    __device__ void run(uint32_t tile, const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ buckets,
+                        uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals) const
+    {
+        const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
+        if (n == 0 || n > (uint32_t)kCap) return;  // uniform over the workgroup
+        if (threadIdx.x == 0) flags[11] = 0;
+        __syncthreads();
+        const uint32_t d0 = (uint32_t)(buckets[lo] >> 32);
+        uint32_t diff = 0;
+        for (uint32_t j = threadIdx.x; j < n; j += kT) {
+            const uint64_t v = buckets[lo + j];
+            depth[j] = (uint32_t)(v >> 32);
+            index[j] = (uint32_t)v;
+            diff |= depth[j] ^ d0;
+        }
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) diff |= __shfl_xor(diff, d, 64);
+        if ((threadIdx.x & 63) == 0 && diff) atomicOr(&flags[11], diff);
+        __syncthreads();
+        const int cur = sort(n, flags[11]);
+        for (uint32_t j = threadIdx.x; j < n; j += kT) {
+            const uint32_t e = cur < 0 ? j : (uint32_t)perm(cur)[j];
+            out_keys[lo + j] = ((uint64_t)tile << 32) | (uint64_t)depth[e];
+            out_vals[lo + j] = index[e];
+        }
+        __syncthreads();
+    }
+};
+
+// Smallest size class: one workgroup per tile (tiles with larger buckets leave at once).
+template <int kT, int kR>
+__global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* __restrict__ header,
+                                                            const uint32_t* __restrict__ ranges,
+                                                            const uint64_t* __restrict__ buckets,
+                                                            uint64_t* __restrict__ out_keys,
+                                                            uint32_t* __restrict__ out_vals)
 {
     extern __shared__ uint32_t s_dyn[];
-    __shared__ uint32_t s_hist[256];
-    __shared__ uint32_t s_cnt[kWaves][256];
-    __shared__ uint32_t s_flags[8];
     if (header->overflow) return;
-    const SortScratch sc = {s_hist, s_cnt, s_flags};
-    const uint32_t count = lists[0];
-    for (uint32_t k = blockIdx.x; k < count; k += gridDim.x)
-        sort_tile_in_lds(lists[2 + k], ranges, buckets, out_keys, out_vals, s_dyn, kTileSortLargeCap,
-                         kTileSortSmallCap, sc);
+    const LdsSorter<kT, kR> sorter(s_dyn);
+    sorter.run(blockIdx.x, ranges, buckets, out_keys, out_vals);
+}
+
+// Larger size classes: persistent workgroups over the class list made by tile_layout_kernel.
+template <int kT, int kR>
+__device__ __forceinline__ void tile_sort_list_body(const gs355_header* __restrict__ header,
+                                                    const uint32_t* __restrict__ ranges,
+                                                    const uint32_t* __restrict__ list,
+                                                    const uint32_t* __restrict__ list_count,
+                                                    const uint64_t* __restrict__ buckets,
+                                                    uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals,
+                                                    uint32_t* lds)
+{
+    if (header->overflow) return;
+    const LdsSorter<kT, kR> sorter(lds);
+    const uint32_t count = *list_count;
+    for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) sorter.run(list[k], ranges, buckets, out_keys, out_vals);
+}
+
+// 1024 threads x 5 rounds, held to 64 VGPRs so that two workgroups share a CU
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void tile_sort_list_1024x5_kernel(
+    const gs355_header* __restrict__ header, const uint32_t* __restrict__ ranges, const uint32_t* __restrict__ list,
+    const uint32_t* __restrict__ list_count, const uint64_t* __restrict__ buckets, uint64_t* __restrict__ out_keys,
+    uint32_t* __restrict__ out_vals)
+{
+    extern __shared__ uint32_t s_dyn[];
+    tile_sort_list_body<1024, 5>(header, ranges, list, list_count, buckets, out_keys, out_vals, s_dyn);
+}
+
+template <int kT, int kR>
+__global__ __launch_bounds__(kT) void tile_sort_list_kernel(const gs355_header* __restrict__ header,
+                                                            const uint32_t* __restrict__ ranges,
+                                                            const uint32_t* __restrict__ list,
+                                                            const uint32_t* __restrict__ list_count,
+                                                            const uint64_t* __restrict__ buckets,
+                                                            uint64_t* __restrict__ out_keys,
+                                                            uint32_t* __restrict__ out_vals)
+{
+    extern __shared__ uint32_t s_dyn[];
+    tile_sort_list_body<kT, kR>(header, ranges, list, list_count, buckets, out_keys, out_vals, s_dyn);
 }
 
 // Buckets beyond the LDS capacity: the same passes through global memory,
@@ -460,9 +638,9 @@ __global__ __launch_bounds__(kThreads) void tile_sort_huge_kernel(const gs355_he
     __shared__ uint32_t s_flags[8];
     if (header->overflow) return;
     const SortScratch sc = {s_hist, s_cnt, s_flags};
-    const uint32_t count = lists[1];
+    const uint32_t count = lists[3];
     for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) {
-        const uint32_t tile = lists[2 + tiles + k];
+        const uint32_t tile = lists[4 + 3 * (size_t)tiles + k];
         const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
         const GlobalPairs A = {buckets + lo}, B = {out_keys + lo};
         const bool in_b = sort_pairs(A, B, n, sc);
@@ -537,27 +715,44 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const float* records, con
     return GS355_OK;
 }
 
+template <typename K>
+static int allow_lds(K kernel, size_t bytes)
+{
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return set_error(GS355_EHIP, "tile sort: LDS attribute: %s", hipGetErrorString(e));
+    return GS355_OK;
+}
+
 int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, const uint32_t* lists,
                      uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, hipStream_t s)
 {
-    hipLaunchKernelGGL(tile_sort_small_kernel, dim3(tiles), dim3(kThreads), 0, s, header, ranges, buckets, out_keys,
-                       out_vals);
-    GS355_CHECK_LAUNCH("tile sort: small");
-    static bool attr_set = false;  // idempotent; a race only repeats the call
-    const size_t dyn = (size_t)4 * kTileSortLargeCap * sizeof(uint32_t);
-    if (!attr_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(tile_sort_large_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
-        if (e != hipSuccess) return set_error(GS355_EHIP, "tile sort: LDS attribute: %s", hipGetErrorString(e));
-        attr_set = true;
-    }
-    const int persistent = tiles < 256 ? tiles : 256;
-    hipLaunchKernelGGL(tile_sort_large_kernel, dim3(persistent), dim3(kThreads), dyn, s, header, ranges, lists, buckets,
+    using S0 = LdsSorter<256, 4>;    // <= 1024 pairs, one workgroup per tile
+    using S1 = LdsSorter<512, 4>;    // <= 2048
+    using S2 = LdsSorter<1024, 5>;   // <= 5120
+    using S3 = LdsSorter<1024, 10>;  // <= 10240
+    static_assert(S0::kCap == kTileSortCap[0] && S1::kCap == kTileSortCap[1] && S2::kCap == kTileSortCap[2] &&
+                      S3::kCap == kTileSortCap[3], "size classes out of step with the layout kernel");
+    int rc;
+    if ((rc = allow_lds(tile_sort_list_1024x5_kernel, S2::kBytes))) return rc;
+    if ((rc = allow_lds(tile_sort_list_kernel<1024, 10>, S3::kBytes))) return rc;
+    const uint32_t* list0 = lists + 4;
+    hipLaunchKernelGGL((tile_sort_each_kernel<256, 4>), dim3(tiles), dim3(256), S0::kBytes, s, header, ranges, buckets,
                        out_keys, out_vals);
-    GS355_CHECK_LAUNCH("tile sort: large");
-    hipLaunchKernelGGL(tile_sort_huge_kernel, dim3(persistent), dim3(kThreads), 0, s, header, ranges, lists,
-                       (uint32_t)tiles, buckets, out_keys, out_vals);
-    GS355_CHECK_LAUNCH("tile sort: huge");
+    GS355_CHECK_LAUNCH("tile sort: class 0");
+    auto grid = [&](int want) { return dim3(tiles < want ? tiles : want); };
+    hipLaunchKernelGGL((tile_sort_list_kernel<512, 4>), grid(1024), dim3(512), S1::kBytes, s, header, ranges, list0,
+                       lists + 0, buckets, out_keys, out_vals);
+    GS355_CHECK_LAUNCH("tile sort: class 1");
+    hipLaunchKernelGGL(tile_sort_list_1024x5_kernel, grid(512), dim3(1024), S2::kBytes, s, header, ranges,
+                       list0 + (size_t)tiles, lists + 1, buckets, out_keys, out_vals);
+    GS355_CHECK_LAUNCH("tile sort: class 2");
+    hipLaunchKernelGGL((tile_sort_list_kernel<1024, 10>), grid(256), dim3(1024), S3::kBytes, s, header, ranges,
+                       list0 + 2 * (size_t)tiles, lists + 2, buckets, out_keys, out_vals);
+    GS355_CHECK_LAUNCH("tile sort: class 3");
+    hipLaunchKernelGGL(tile_sort_huge_kernel, grid(256), dim3(kThreads), 0, s, header, ranges, lists, (uint32_t)tiles,
+                       buckets, out_keys, out_vals);
+    GS355_CHECK_LAUNCH("tile sort: beyond LDS");
     return GS355_OK;
 }
 

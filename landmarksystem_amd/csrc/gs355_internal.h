@@ -17,9 +17,8 @@ constexpr int kSortTile = kSortThreads * kSortItems;
 constexpr int kRadixBits = 8;
 constexpr int kRadix = 1 << kRadixBits;
 
-// tile-bucketed sort: bucket sizes handled in static LDS / dynamic LDS (148 KB); larger go through global memory
-constexpr int kTileSortSmallCap = 2048;
-constexpr int kTileSortLargeCap = 9216;
+// tile-bucketed sort: buckets up to kTileSortCap[3] pairs are sorted in LDS; larger ones go through global memory
+constexpr int kTileSortCap[4] = {1024, 2048, 5120, 10240};  // in-LDS sorter size classes (pairs per bucket)
 
 // scan geometry: 256 threads x 16 items per workgroup
 constexpr int kScanThreads = 256;
@@ -83,7 +82,7 @@ int launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t s);
 
 // tile-bucketed path
 constexpr int kBinThreads = 1024;       // threads per binning workgroup
-constexpr int kBinMaxGroups = 512;      // binning workgroups (each owns a contiguous slice of the Gaussians)
+constexpr int kBinMaxGroups = 256;      // binning workgroups (each owns a contiguous slice of the Gaussians)
 constexpr int kBinMaxTiles = 36000;     // per-tile counters of one workgroup must fit in LDS (4 B each)
 int bin_groups(int32_t P, int* per_group);
 int launch_tile_count(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii, uint32_t* matrix,

@@ -46,25 +46,66 @@ __device__ __forceinline__ void covariance3d(const float* __restrict__ scale, fl
     cov[5] = (l20 * l20 + l21 * l21) + l22 * l22;
 }
 
+// SH degree 0..3 -> RGB for one Gaussian; `sh` points at its [M,3] block
+// (coefficient-major, RGB innermost) in global memory or in LDS.
+__device__ __forceinline__ void sh_to_rgb(int degree, const float* sh, float dx, float dy, float dz, float out[3])
+{
+    const float len = sqrtf((dx * dx + dy * dy) + dz * dz);
+    dx = dx / len;
+    dy = dy / len;
+    dz = dz / len;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+        float res = kShC0 * sh[c];
+        if (degree > 0) {
+            res = res - kShC1 * dy * sh[3 + c] + kShC1 * dz * sh[6 + c] - kShC1 * dx * sh[9 + c];
+            if (degree > 1) {
+                const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
+                const float xy = dx * dy, yz = dy * dz, xz = dx * dz;
+                res = res + kShC2[0] * xy * sh[12 + c] + kShC2[1] * yz * sh[15 + c] +
+                      kShC2[2] * (2.0f * zz - xx - yy) * sh[18 + c] + kShC2[3] * xz * sh[21 + c] +
+                      kShC2[4] * (xx - yy) * sh[24 + c];
+                if (degree > 2) {
+                    res = res + kShC3[0] * dy * (3.0f * xx - yy) * sh[27 + c] + kShC3[1] * xy * dz * sh[30 + c] +
+                          kShC3[2] * dy * (4.0f * zz - xx - yy) * sh[33 + c] +
+                          kShC3[3] * dz * (2.0f * zz - 3.0f * xx - 3.0f * yy) * sh[36 + c] +
+                          kShC3[4] * dx * (4.0f * zz - xx - yy) * sh[39 + c] + kShC3[5] * dz * (xx - yy) * sh[42 + c] +
+                          kShC3[6] * dx * (xx - 3.0f * yy) * sh[45 + c];
+                }
+            }
+        }
+        res += 0.5f;
+        out[c] = res < 0.0f ? 0.0f : res;
+    }
+}
+
+constexpr int kShStride = 52;  // floats per Gaussian in the LDS staging area: 48 + 4 keeps 16-B reads conflict-free
+
 template <bool kRadiiOnly>
 __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaussians g,
                                                          float* __restrict__ records,
                                                          uint32_t* __restrict__ tiles_touched,
                                                          int32_t* __restrict__ radii)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= g.P) return;
+    // staging area for the 16-coefficient SH blocks of each wavefront's 64 Gaussians
+    __shared__ float4 s_sh[kRadiiOnly ? 1 : 4 * 64 * kShStride / 4];
 
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool valid = i < g.P;
     const float* __restrict__ V = f.viewmatrix;
     const float* __restrict__ M = f.projmatrix;
 
+    // ---- geometry: cull, covariance, EWA projection, conic, radius, tile rectangle ----
     int radius = 0;
     uint32_t touched = 0;
-    do {
-        const float x = g.means3D[3 * (size_t)i], y = g.means3D[3 * (size_t)i + 1], z = g.means3D[3 * (size_t)i + 2];
+    float x = 0.f, y = 0.f, z = 0.f, vz = 0.f, px = 0.f, py = 0.f, ca = 0.f, cc = 0.f, qx = 0.f, qy = 0.f, qz = 0.f;
+    if (valid) do {
+        x = g.means3D[3 * (size_t)i];
+        y = g.means3D[3 * (size_t)i + 1];
+        z = g.means3D[3 * (size_t)i + 2];
         const float vx = ((V[0] * x + V[4] * y) + V[8] * z) + V[12];
         const float vy = ((V[1] * x + V[5] * y) + V[9] * z) + V[13];
-        const float vz = ((V[2] * x + V[6] * y) + V[10] * z) + V[14];
+        vz = ((V[2] * x + V[6] * y) + V[10] * z) + V[14];
         if (vz <= 0.2f) break;  // behind or too close to the camera plane
 
         const float hx = ((M[0] * x + M[4] * y) + M[8] * z) + M[12];
@@ -100,9 +141,9 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
         const float b11 = (a10 * cov[1] + a11 * cov[3]) + a12 * cov[4];
         const float b12 = (a10 * cov[2] + a11 * cov[4]) + a12 * cov[5];
         // 2D covariance b * a^T with the 0.3 px low-pass on the diagonal
-        const float ca = ((b00 * a00 + b01 * a01) + b02 * a02) + 0.3f;
+        ca = ((b00 * a00 + b01 * a01) + b02 * a02) + 0.3f;
         const float cb = (b00 * a10 + b01 * a11) + b02 * a12;
-        const float cc = ((b10 * a10 + b11 * a11) + b12 * a12) + 0.3f;
+        cc = ((b10 * a10 + b11 * a11) + b12 * a12) + 0.3f;
 
         const float det = ca * cc - cb * cb;
         if (det == 0.0f) break;
@@ -114,91 +155,86 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
         if (!(rf < 1073741824.0f)) break;  // non-finite or absurd footprint
         const int rad = (int)rf;
 
-        const float px = ((ndc_x + 1.0f) * (float)f.W - 1.0f) * 0.5f;
-        const float py = ((ndc_y + 1.0f) * (float)f.H - 1.0f) * 0.5f;
+        px = ((ndc_x + 1.0f) * (float)f.W - 1.0f) * 0.5f;
+        py = ((ndc_y + 1.0f) * (float)f.H - 1.0f) * 0.5f;
         const Rect q = tile_rect(px, py, rad, f.grid_x, f.grid_y);
         const int area = (q.x1 - q.x0) * (q.y1 - q.y0);
         if (area == 0) break;
 
         radius = rad;
         touched = (uint32_t)area;
-        if (kRadiiOnly) break;
-
-        float cr, cg, cbl;
-        if (g.colors_precomp) {
-            cr = g.colors_precomp[3 * (size_t)i];
-            cg = g.colors_precomp[3 * (size_t)i + 1];
-            cbl = g.colors_precomp[3 * (size_t)i + 2];
-        } else {
-            const float* __restrict__ sh = g.shs + (size_t)i * f.sh_coeffs * 3;
-            float dx = x - f.campos[0], dy = y - f.campos[1], dz = z - f.campos[2];
-            const float len = sqrtf((dx * dx + dy * dy) + dz * dz);
-            dx = dx / len;
-            dy = dy / len;
-            dz = dz / len;
-            float out[3];
-#pragma unroll
-            for (int c = 0; c < 3; ++c) {
-                float res = kShC0 * sh[c];
-                if (f.sh_degree > 0) {
-                    res = res - kShC1 * dy * sh[3 + c] + kShC1 * dz * sh[6 + c] - kShC1 * dx * sh[9 + c];
-                    if (f.sh_degree > 1) {
-                        const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
-                        const float xy = dx * dy, yz = dy * dz, xz = dx * dz;
-                        res = res + kShC2[0] * xy * sh[12 + c] + kShC2[1] * yz * sh[15 + c] +
-                              kShC2[2] * (2.0f * zz - xx - yy) * sh[18 + c] + kShC2[3] * xz * sh[21 + c] +
-                              kShC2[4] * (xx - yy) * sh[24 + c];
-                        if (f.sh_degree > 2) {
-                            res = res + kShC3[0] * dy * (3.0f * xx - yy) * sh[27 + c] +
-                                  kShC3[1] * xy * dz * sh[30 + c] +
-                                  kShC3[2] * dy * (4.0f * zz - xx - yy) * sh[33 + c] +
-                                  kShC3[3] * dz * (2.0f * zz - 3.0f * xx - 3.0f * yy) * sh[36 + c] +
-                                  kShC3[4] * dx * (4.0f * zz - xx - yy) * sh[39 + c] +
-                                  kShC3[5] * dz * (xx - yy) * sh[42 + c] +
-                                  kShC3[6] * dx * (xx - 3.0f * yy) * sh[45 + c];
-                        }
-                    }
-                }
-                res += 0.5f;
-                out[c] = res < 0.0f ? 0.0f : res;
-            }
-            cr = out[0];
-            cg = out[1];
-            cbl = out[2];
-        }
-
-        // Reach of the splat for the blend stage's quadrant culling: half-extents
-        // (ex, ey) of the axis-aligned box around the region where alpha can reach
-        // 1/255, i.e. where 0.5 d^T Q d <= ln(255 * opacity).  The box is enlarged
-        // by more than the rounding error of the blend's fp32 evaluation of the
-        // exponent (bounded below by `noise`), so a quadrant outside the box is
-        // certain to take the blend's `alpha < 1/255` branch on all of its pixels.
-        // +inf = never cull (large or ill-conditioned splats), -inf = never visible.
-        const float opacity = g.opacities[i];
-        const float qx = cc * det_inv, qy = -cb * det_inv, qz = ca * det_inv;
-        float ex, ey;
-        {
-            const float reach = (float)rad + 24.0f;  // |d| over every pixel of every touched tile
-            const float noise = 2.4e-7f * (fabsf(qx) + fabsf(qy) + fabsf(qz)) * reach * reach;
-            if (opacity != opacity || !(noise < 0.02f)) {
-                ex = ey = INFINITY;
-            } else if (!(opacity * 255.0f * 1.0001f >= 1.0f)) {
-                ex = ey = -INFINITY;
-            } else {
-                const float tau = fmaxf(__logf(opacity * 255.0f), 0.0f) * 1.001f + 0.05f;
-                ex = sqrtf(2.0f * tau * ca) * 1.001f + 0.01f;
-                ey = sqrtf(2.0f * tau * cc) * 1.001f + 0.01f;
-            }
-        }
-
-        float4* __restrict__ rec = reinterpret_cast<float4*>(records + (size_t)i * kRecordFloats);
-        rec[0] = make_float4(px, py, qx, qy);
-        rec[1] = make_float4(qz, opacity, cr, cg);
-        rec[2] = make_float4(cbl, vz, ex, ey);
+        qx = cc * det_inv;
+        qy = -cb * det_inv;
+        qz = ca * det_inv;
     } while (false);
 
-    radii[i] = radius;
-    if (!kRadiiOnly) tiles_touched[i] = touched;
+    if (valid) radii[i] = radius;
+    if (kRadiiOnly) return;
+    if (valid) tiles_touched[i] = touched;
+    const bool alive = radius > 0;
+
+    // ---- colour ----
+    float rgb[3] = {0.f, 0.f, 0.f};
+    if (g.colors_precomp) {
+        if (alive) {
+            rgb[0] = g.colors_precomp[3 * (size_t)i];
+            rgb[1] = g.colors_precomp[3 * (size_t)i + 1];
+            rgb[2] = g.colors_precomp[3 * (size_t)i + 2];
+        }
+    } else {
+        const float dx = x - f.campos[0], dy = y - f.campos[1], dz = z - f.campos[2];
+        // When most of the wavefront survived and the blocks are the full 192 B,
+        // the 12 KB of SH of its 64 Gaussians are fetched with fully coalesced
+        // 16-B loads into LDS and each lane reads its own block back from there;
+        // otherwise every survivor fetches its own block.  Same values either way.
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        const int wave_first = blockIdx.x * blockDim.x + wave * 64;
+        const bool staged = f.sh_coeffs == 16 && (reinterpret_cast<uintptr_t>(g.shs) & 15u) == 0 &&
+                            __popcll(__ballot(alive)) >= 32;  // uniform per wavefront
+        if (staged) {
+            float4* __restrict__ mine = s_sh + wave * (64 * kShStride / 4);
+            const float4* __restrict__ src = reinterpret_cast<const float4*>(g.shs + (size_t)wave_first * 48);
+            const int count4 = min(64, g.P - wave_first) * 12;
+#pragma unroll
+            for (int it = 0; it < 12; ++it) {
+                const int q4 = it * 64 + lane;
+                if (q4 < count4) mine[(q4 / 12) * (kShStride / 4) + q4 % 12] = src[q4];
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (alive) sh_to_rgb(f.sh_degree, reinterpret_cast<const float*>(mine) + lane * kShStride, dx, dy, dz, rgb);
+        } else if (alive) {
+            sh_to_rgb(f.sh_degree, g.shs + (size_t)i * f.sh_coeffs * 3, dx, dy, dz, rgb);
+        }
+    }
+    if (!alive) return;
+
+    // Reach of the splat for the blend stage's quadrant culling: half-extents
+    // (ex, ey) of the axis-aligned box around the region where alpha can reach
+    // 1/255, i.e. where 0.5 d^T Q d <= ln(255 * opacity).  The box is enlarged
+    // by more than the rounding error of the blend's fp32 evaluation of the
+    // exponent (bounded below by `noise`), so a quadrant outside the box is
+    // certain to take the blend's `alpha < 1/255` branch on all of its pixels.
+    // +inf = never cull (large or ill-conditioned splats), -inf = never visible.
+    const float opacity = g.opacities[i];
+    float ex, ey;
+    {
+        const float reach = (float)radius + 24.0f;  // |d| over every pixel of every touched tile
+        const float noise = 2.4e-7f * (fabsf(qx) + fabsf(qy) + fabsf(qz)) * reach * reach;
+        if (opacity != opacity || !(noise < 0.02f)) {
+            ex = ey = INFINITY;
+        } else if (!(opacity * 255.0f * 1.0001f >= 1.0f)) {
+            ex = ey = -INFINITY;
+        } else {
+            const float tau = fmaxf(__logf(opacity * 255.0f), 0.0f) * 1.001f + 0.05f;
+            ex = sqrtf(2.0f * tau * ca) * 1.001f + 0.01f;
+            ey = sqrtf(2.0f * tau * cc) * 1.001f + 0.01f;
+        }
+    }
+
+    float4* __restrict__ rec = reinterpret_cast<float4*>(records + (size_t)i * kRecordFloats);
+    rec[0] = make_float4(px, py, qx, qy);
+    rec[1] = make_float4(qz, opacity, rgb[0], rgb[1]);
+    rec[2] = make_float4(rgb[2], vz, ex, ey);
 }
 
 // One workgroup expands the keys of 256 consecutive Gaussians.  Output slots

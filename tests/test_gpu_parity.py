@@ -275,8 +275,10 @@ def crowded_scene(P, width=64, height=64, duplicates=0, seed=0):
     (lambda: scenes.config2(P=100_000), "C2/100k"),
     (lambda: scenes.config3(P=300_000), "C3/300k"),
     (lambda: scenes.tiny_scene(P=300, width=33, height=17, sh_degree=2, seed=5), "ragged"),
-    (lambda: crowded_scene(1500, duplicates=300), "small buckets with ties"),
-    (lambda: crowded_scene(5000, duplicates=500), "LDS-large buckets with ties"),
+    (lambda: crowded_scene(800, duplicates=200), "class0 buckets with ties"),
+    (lambda: crowded_scene(1500, duplicates=300), "class1 buckets with ties"),
+    (lambda: crowded_scene(5000, duplicates=500), "class2 buckets with ties"),
+    (lambda: crowded_scene(8000, width=32, height=32, duplicates=500), "class3 buckets with ties"),
     (lambda: crowded_scene(12_000, width=32, height=32, duplicates=700), "beyond-LDS buckets with ties"),
 ])
 def test_tile_bucketed_path_equals_oracle(gpu_device, make, label):
@@ -295,7 +297,8 @@ def test_tile_bucketed_path_equals_oracle(gpu_device, make, label):
         k = got["sorted_keys"]
         assert (k[1:] == k[:-1]).any()
         lens = (ref["ranges"][:, 1].astype(np.int64) - ref["ranges"][:, 0])
-        want = {"small": (1, 2048), "LDS-large": (2049, 9216), "beyond-LDS": (9217, 1 << 30)}[label.split(" ")[0]]
+        want = {"class0": (1, 1024), "class1": (1025, 2048), "class2": (2049, 5120), "class3": (5121, 10240),
+                "beyond-LDS": (10241, 1 << 30)}[label.split(" ")[0]]
         assert want[0] <= lens.max() <= want[1], lens.max()
 
 

@@ -174,6 +174,53 @@ GS355_API int gs355_render(const gs355_frame *frame, const gs355_gaussians *g, v
  * `g` are ignored and may be NULL. */
 GS355_API int gs355_visible_filter(const gs355_frame *frame, const gs355_gaussians *g, int32_t *radii, void *stream);
 
+/* ---------------------------------------------------------------------------
+ * Anchor decode for Scaffold-GS / Octree-GS: replaces AnchorDecoder.forward in eval mode
+ * (landmark/nerf_components/model_components/fields/anchor_decoder.py:108-242) and the kernels of its
+ * fused twin (fused_anchor_decoder.py:69-244: fusedKernels.*, FusedMatmul.simple2layer -- an empty
+ * third-party submodule in the reference tree).  Supported configuration: feat_dim 32, 1..10 offsets,
+ * no feature bank, no level / appearance inputs (the Scaffold-GS model's, scaffold_gs/gs_model.py:126-134).
+ * Heads are indexed 0 = opacity (tanh), 1 = covariance (7 per offset), 2 = colour (sigmoid). */
+typedef struct gs355_decoder {
+    int32_t feat_dim;    /* 32 */
+    int32_t n_offsets;   /* 1..10 */
+    int32_t in_dim[3];   /* 36 = [feat | view | dist], 35 = [feat | view] (the head's add_*_dist is False) */
+    const float *w0[3];  /* device f32[32, in_dim]   nn.Linear weight layout [out, in] */
+    const float *b0[3];  /* device f32[32] */
+    const float *w1[3];  /* device f32[k, 32], k = n_offsets, 7 n_offsets, 3 n_offsets */
+    const float *b1[3];  /* device f32[k] */
+} gs355_decoder;
+
+typedef struct gs355_anchors {
+    int32_t A;
+    const float *anchor;         /* [A,3] */
+    const float *feat;           /* [A,32], 16-byte aligned */
+    const float *offset;         /* [A,n_offsets,3] */
+    const float *scaling;        /* [A,6] (exp-activated; 0..2 scale offsets, 3..5 scale Gaussians) */
+    const uint8_t *visible_mask; /* [A] 0/1 (a torch.bool tensor) */
+    const float *campos;         /* device f32[3] */
+} gs355_anchors;
+
+typedef struct gs355_decoded {
+    float *xyz;     /* [G,3] */
+    float *color;   /* [G,3] */
+    float *opacity; /* [G,1] */
+    float *scaling; /* [G,3] */
+    float *rot;     /* [G,4] */
+} gs355_decoded;
+
+GS355_API int gs355_decode_scratch_bytes(int32_t A, size_t *bytes);
+
+/* Pass 1: counts[a] = offsets of anchor a with opacity > 0 (0 for invisible anchors); offsets = exclusive
+ * prefix sum of counts.  G = offsets[A-1] + counts[A-1] is the number of Gaussians pass 2 emits. */
+GS355_API int gs355_decode_count(const gs355_decoder *dec, const gs355_anchors *an, uint32_t *counts, uint32_t *offsets,
+                       void *scratch, size_t scratch_bytes, void *stream);
+
+/* Pass 2: decode all heads and write the kept Gaussians in boolean-mask order (row-major over visible anchor,
+ * offset) into outputs with room for `capacity` Gaussians. */
+GS355_API int gs355_decode_emit(const gs355_decoder *dec, const gs355_anchors *an, const uint32_t *offsets, int64_t capacity,
+                      const gs355_decoded *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

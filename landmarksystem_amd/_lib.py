@@ -19,7 +19,7 @@ PIPELINE_FAST = STAGE_PREPROCESS | STAGE_TILE_COUNT | STAGE_TILE_SCATTER | STAGE
 MAX_FAST_TILES = 36000
 
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
-           "gs355_visible_filter")
+           "gs355_visible_filter", "gs355_decode_scratch_bytes", "gs355_decode_count", "gs355_decode_emit")
 
 
 class Frame(C.Structure):
@@ -88,6 +88,35 @@ class Layout(C.Structure):
     ]
 
 
+class Decoder(C.Structure):
+    _fields_ = [
+        ("feat_dim", C.c_int32),
+        ("n_offsets", C.c_int32),
+        ("in_dim", C.c_int32 * 3),
+        ("w0", C.c_void_p * 3),
+        ("b0", C.c_void_p * 3),
+        ("w1", C.c_void_p * 3),
+        ("b1", C.c_void_p * 3),
+    ]
+
+
+class Anchors(C.Structure):
+    _fields_ = [
+        ("A", C.c_int32),
+        ("anchor", C.c_void_p),
+        ("feat", C.c_void_p),
+        ("offset", C.c_void_p),
+        ("scaling", C.c_void_p),
+        ("visible_mask", C.c_void_p),
+        ("campos", C.c_void_p),
+    ]
+
+
+class Decoded(C.Structure):
+    _fields_ = [("xyz", C.c_void_p), ("color", C.c_void_p), ("opacity", C.c_void_p), ("scaling", C.c_void_p),
+                ("rot", C.c_void_p)]
+
+
 class Gs355Error(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__("gs355 error %d: %s" % (code, message))
@@ -120,6 +149,14 @@ def load() -> C.CDLL:
     lib.gs355_render.restype = C.c_int
     lib.gs355_visible_filter.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_void_p, C.c_void_p]
     lib.gs355_visible_filter.restype = C.c_int
+    lib.gs355_decode_scratch_bytes.argtypes = [C.c_int32, C.POINTER(C.c_size_t)]
+    lib.gs355_decode_scratch_bytes.restype = C.c_int
+    lib.gs355_decode_count.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.c_size_t, C.c_void_p]
+    lib.gs355_decode_count.restype = C.c_int
+    lib.gs355_decode_emit.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_int64,
+                                      C.POINTER(Decoded), C.c_void_p]
+    lib.gs355_decode_emit.restype = C.c_int
     _lib = lib
     return lib
 

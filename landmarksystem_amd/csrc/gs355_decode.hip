@@ -1,0 +1,368 @@
+// Scaffold-GS / Octree-GS anchor decode on the gfx950 matrix cores.
+//
+// Replaces AnchorDecoder.forward in eval mode (landmark/nerf_components/
+// model_components/fields/anchor_decoder.py:108-242; MLP shapes :79-104; the
+// reference's fused twin is fused_anchor_decoder.py:69-244, whose CUDA kernels
+// are an empty submodule) for the configuration the Scaffold-GS model builds
+// (scaffold_gs/gs_model.py:126-134): no feature bank, no level / appearance
+// inputs, three two-layer MLPs  [feat(32) | view(3) | dist(1)] -> 32 -> ReLU ->
+// {n, 7n, 3n}  with tanh / none / sigmoid, mask opacity > 0, then
+// scaling = anchor_scaling[3:6] * sigmoid(cov[0:3]), rot = normalize(cov[3:7]),
+// xyz = anchor + offset * anchor_scaling[0:3].
+//
+// Everything is computed transposed so that the two layers chain without any
+// data movement: weights are the A operand (rows = output units), 32 anchors
+// are the columns of one v_mfma_f32_32x32x8_f16 tile, and the accumulator
+// layout of layer 1 (lane = anchor, registers = hidden units 8b+4*half+t) is
+// exactly the B-operand layout layer 2 needs.
+//
+// Precision: weights and anchor features are rounded to fp16 (exact for fp16
+// checkpoints); the four fp32-only inputs (view direction, distance) and the
+// hidden activations enter the matrix cores as hi + lo fp16 pairs, so the
+// result carries fp32-level accuracy with fp32 accumulation.
+//
+// Output order is the reference's boolean-mask order: row-major over (visible
+// anchor, offset).  Two launches: count kept offsets per anchor (opacity head
+// only) -> exclusive scan -> emit (all heads; the opacity head is recomputed
+// with the identical instruction sequence, so counts and emission agree).
+#include "gs355_internal.h"
+
+namespace gs355 {
+
+namespace {
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kFeat = 32;
+
+struct DecodeArgs {
+    int A, n;       // anchors, offsets per anchor
+    int in_dim[3];  // 35 or 36 per head (opacity, cov, color)
+    const float* anchor;
+    const float* feat;
+    const float* offset;
+    const float* scaling;
+    const uint8_t* visible;
+    const float* campos;
+    const float* w0[3];
+    const float* b0[3];
+    const float* w1[3];
+    const float* b1[3];
+};
+
+__device__ __forceinline__ half4_t to_half4(float a, float b, float c, float d)
+{
+    half4_t h;
+    h[0] = (_Float16)a;
+    h[1] = (_Float16)b;
+    h[2] = (_Float16)c;
+    h[3] = (_Float16)d;
+    return h;
+}
+
+// A fragment of a [rows x cols] row-major fp32 weight matrix for k-step s:
+// lane (row = lane % 32, half = lane / 32) holds W[row0 + row][8s + 4*half + 0..3].
+__device__ __forceinline__ half4_t weight_fragment(const float* __restrict__ w, int rows, int cols, int row, int k0)
+{
+    float v[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) v[t] = (row < rows && k0 + t < cols) ? w[(size_t)row * cols + k0 + t] : 0.0f;
+    return to_half4(v[0], v[1], v[2], v[3]);
+}
+
+// Bias for an accumulator: register v = 4b + t holds row 8b + 4*half + t.
+__device__ __forceinline__ floatx16 bias_rows(const float* __restrict__ bias, int rows, int row0, int half)
+{
+    floatx16 c;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int r = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
+        c[v] = r < rows ? bias[r] : 0.0f;
+    }
+    return c;
+}
+
+// One head for one tile of 32 anchors: returns up to kTiles accumulators of the
+// second layer (rows = outputs 32r + 8b + 4*half + t, column = this lane's anchor).
+template <int kTiles>
+__device__ __forceinline__ void run_head(const DecodeArgs& d, int head, int outputs, const half4_t X[5], int row,
+                                         int half, floatx16 out[kTiles])
+{
+    // layer 1: hidden = W0 [32 x in] * X^T + b0
+    floatx16 h = bias_rows(d.b0[head], kFeat, 0, half);
+    const int in = d.in_dim[head];
+#pragma unroll
+    for (int s = 0; s < 5; ++s) {
+        // k-step 4 carries the fp32-only inputs twice: hi parts on the low half of the lanes, lo parts on the
+        // high half, both against the same weights W0[:, 32..35]
+        const int k0 = s < 4 ? 8 * s + 4 * half : 32;
+        const half4_t a = weight_fragment(d.w0[head], kFeat, in, row, k0);
+        h = __builtin_amdgcn_mfma_f32_32x32x8f16(a, X[s], h, 0, 0, 0);
+    }
+    // ReLU, then hi/lo split: registers 4s..4s+3 are the B operand of k-step s
+    half4_t hh[4], hl[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        float r[4], lo[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            r[t] = fmaxf(h[4 * s + t], 0.0f);
+            const _Float16 top = (_Float16)r[t];
+            lo[t] = r[t] - (float)top;
+        }
+        hh[s] = to_half4(r[0], r[1], r[2], r[3]);
+        hl[s] = to_half4(lo[0], lo[1], lo[2], lo[3]);
+    }
+    // layer 2: out = W1 [outputs x 32] * hidden + b1
+#pragma unroll
+    for (int r = 0; r < kTiles; ++r) {
+        floatx16 c = bias_rows(d.b1[head], outputs, 32 * r, half);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const half4_t a = weight_fragment(d.w1[head], outputs, kFeat, 32 * r + row, 8 * s + 4 * half);
+            c = __builtin_amdgcn_mfma_f32_32x32x8f16(a, hh[s], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x8f16(a, hl[s], c, 0, 0, 0);
+        }
+        out[r] = c;
+    }
+}
+
+// Store the rows of an accumulator that exist (< outputs) into the tile's LDS block.
+__device__ __forceinline__ void store_rows(float* __restrict__ dst_anchor, int base, int outputs, int row0, int half,
+                                           const floatx16& c)
+{
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int r = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
+        if (r < outputs) dst_anchor[base + r] = c[v];
+    }
+}
+
+template <bool kCountOnly>
+__global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
+                                                     const uint32_t* __restrict__ offsets, uint32_t capacity,
+                                                     float* __restrict__ xyz, float* __restrict__ color,
+                                                     float* __restrict__ opacity, float* __restrict__ scaling_out,
+                                                     float* __restrict__ rot)
+{
+    // per wavefront: [32 anchors][stride] floats; stride odd -> conflict-free column access
+    constexpr int kStrideMax = kCountOnly ? 11 : 113;
+    __shared__ float s_out[4][32 * kStrideMax];
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
+    const int n = d.n;
+    const int stride = kCountOnly ? 11 : 11 * n + 3;
+    const int tiles = (d.A + 31) / 32;
+    float* __restrict__ mine = s_out[wave];
+    const float cx = d.campos[0], cy = d.campos[1], cz = d.campos[2];
+
+    for (int tile = blockIdx.x * 4 + wave; tile < tiles; tile += gridDim.x * 4) {
+        const int a = tile * 32 + col;  // this lane's anchor (lanes l and l+32 share it)
+        const bool vis = a < d.A && d.visible[a] != 0;
+        const uint64_t any = __ballot(vis);
+        if (any == 0ull) {  // nothing visible in these 32 anchors
+            if (kCountOnly && half == 0 && a < d.A) counts[a] = 0;
+            continue;
+        }
+        // B operand: X^T, column = anchor, k = 8s + 4*half + t
+        half4_t X[5];
+        float ax = 0.f, ay = 0.f, az = 0.f;
+        if (vis) {
+            const float4* __restrict__ f4 = reinterpret_cast<const float4*>(d.feat + (size_t)a * kFeat);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float4 v = f4[2 * s + half];
+                X[s] = to_half4(v.x, v.y, v.z, v.w);
+            }
+            ax = d.anchor[3 * (size_t)a];
+            ay = d.anchor[3 * (size_t)a + 1];
+            az = d.anchor[3 * (size_t)a + 2];
+            float vx = ax - cx, vy = ay - cy, vz = az - cz;
+            const float dist = sqrtf(vx * vx + vy * vy + vz * vz);
+            vx /= dist;
+            vy /= dist;
+            vz /= dist;
+            const float in4[4] = {vx, vy, vz, dist};
+            float part[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const _Float16 top = (_Float16)in4[t];
+                part[t] = half ? in4[t] - (float)top : (float)top;
+            }
+            X[4] = to_half4(part[0], part[1], part[2], part[3]);
+        } else {
+#pragma unroll
+            for (int s = 0; s < 5; ++s) X[s] = to_half4(0.f, 0.f, 0.f, 0.f);
+        }
+
+        // ---- opacity head ----
+        floatx16 op[1];
+        run_head<1>(d, 0, n, X, col, half, op);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) op[0][v] = tanhf(op[0][v]);
+        store_rows(mine + col * stride, 0, n, 0, half, op[0]);
+        if (kCountOnly) {
+            __builtin_amdgcn_wave_barrier();
+            if (half == 0 && a < d.A) {
+                uint32_t kept = 0;
+                if (vis)
+                    for (int m = 0; m < n; ++m) kept += mine[col * stride + m] > 0.0f ? 1u : 0u;
+                counts[a] = kept;
+            }
+            __builtin_amdgcn_wave_barrier();
+            continue;
+        }
+
+        // ---- covariance and colour heads ----
+        floatx16 cv[3];
+        run_head<3>(d, 1, 7 * n, X, col, half, cv);
+#pragma unroll
+        for (int r = 0; r < 3; ++r) store_rows(mine + col * stride, n, 7 * n, 32 * r, half, cv[r]);
+        floatx16 cl[1];
+        run_head<1>(d, 2, 3 * n, X, col, half, cl);
+        store_rows(mine + col * stride, 8 * n, 3 * n, 0, half, cl[0]);
+        __builtin_amdgcn_wave_barrier();
+
+        // ---- per (anchor, offset): mask, post-process, write at its slot ----
+        const int items = 32 * n;
+        for (int it = lane; it < items; it += 64) {
+            const int al = it / n, m = it - al * n;
+            const int ga = tile * 32 + al;
+            if (ga >= d.A || d.visible[ga] == 0) continue;
+            const float* __restrict__ o = mine + al * stride;
+            const float opac = o[m];
+            if (!(opac > 0.0f)) continue;
+            uint32_t rank = 0;
+            for (int mm = 0; mm < m; ++mm) rank += o[mm] > 0.0f ? 1u : 0u;
+            const uint32_t pos = offsets[ga] + rank;
+            if (pos >= capacity) continue;  // cannot happen when capacity comes from the count pass
+            const float* __restrict__ c7 = o + n + 7 * m;
+            const float* __restrict__ c3 = o + 8 * n + 3 * m;
+            const float* __restrict__ sc = d.scaling + 6 * (size_t)ga;
+            const float* __restrict__ of = d.offset + (size_t)ga * n * 3 + 3 * m;
+            const float* __restrict__ an = d.anchor + 3 * (size_t)ga;
+            opacity[pos] = opac;
+#pragma unroll
+            for (int k = 0; k < 3; ++k) {
+                color[3 * (size_t)pos + k] = 1.0f / (1.0f + expf(-c3[k]));
+                scaling_out[3 * (size_t)pos + k] = sc[3 + k] * (1.0f / (1.0f + expf(-c7[k])));
+                xyz[3 * (size_t)pos + k] = an[k] + of[k] * sc[k];
+            }
+            const float q0 = c7[3], q1 = c7[4], q2 = c7[5], q3 = c7[6];
+            const float norm = fmaxf(sqrtf(q0 * q0 + q1 * q1 + q2 * q2 + q3 * q3), 1e-12f);
+            rot[4 * (size_t)pos + 0] = q0 / norm;
+            rot[4 * (size_t)pos + 1] = q1 / norm;
+            rot[4 * (size_t)pos + 2] = q2 / norm;
+            rot[4 * (size_t)pos + 3] = q3 / norm;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+}  // namespace
+
+struct DecodeLaunch {
+    DecodeArgs args;
+};
+
+static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, DecodeArgs* out)
+{
+    if (!dec || !an) return set_error(GS355_EINVAL, "decoder / anchors is NULL");
+    if (dec->feat_dim != kFeat)
+        return set_error(GS355_EINVAL, "anchor decode supports feat_dim 32 only (got %d)", dec->feat_dim);
+    if (dec->n_offsets < 1 || dec->n_offsets > 10)
+        return set_error(GS355_EINVAL, "anchor decode supports 1..10 offsets per anchor (got %d)", dec->n_offsets);
+    if (an->A < 0) return set_error(GS355_EINVAL, "A must be >= 0 (got %d)", an->A);
+    for (int j = 0; j < 3; ++j) {
+        if (dec->in_dim[j] != kFeat + 3 && dec->in_dim[j] != kFeat + 4)
+            return set_error(GS355_EINVAL, "head %d: input width must be 35 or 36 (got %d)", j, dec->in_dim[j]);
+        if (!dec->w0[j] || !dec->b0[j] || !dec->w1[j] || !dec->b1[j])
+            return set_error(GS355_EINVAL, "head %d: weight or bias pointer is NULL", j);
+    }
+    if (an->A > 0 && (!an->anchor || !an->feat || !an->offset || !an->scaling || !an->visible_mask || !an->campos))
+        return set_error(GS355_EINVAL, "anchor inputs must all be non-NULL");
+    if (an->A > 0 && (reinterpret_cast<uintptr_t>(an->feat) & 15u) != 0)
+        return set_error(GS355_EINVAL, "anchor features must be 16-byte aligned");
+    DecodeArgs a;
+    a.A = an->A;
+    a.n = dec->n_offsets;
+    a.anchor = an->anchor;
+    a.feat = an->feat;
+    a.offset = an->offset;
+    a.scaling = an->scaling;
+    a.visible = an->visible_mask;
+    a.campos = an->campos;
+    for (int j = 0; j < 3; ++j) {
+        a.in_dim[j] = dec->in_dim[j];
+        a.w0[j] = dec->w0[j];
+        a.b0[j] = dec->b0[j];
+        a.w1[j] = dec->w1[j];
+        a.b1[j] = dec->b1[j];
+    }
+    *out = a;
+    return GS355_OK;
+}
+
+static dim3 decode_grid(int A)
+{
+    const int tiles = (A + 31) / 32;
+    int blocks = (tiles + 3) / 4;
+    if (blocks > 2048) blocks = 2048;
+    if (blocks < 1) blocks = 1;
+    return dim3(blocks);
+}
+
+}  // namespace gs355
+
+using namespace gs355;
+
+extern "C" {
+
+int gs355_decode_scratch_bytes(int32_t A, size_t* bytes)
+{
+    if (!bytes) return set_error(GS355_EINVAL, "bytes is NULL");
+    if (A < 0) return set_error(GS355_EINVAL, "A must be >= 0 (got %d)", A);
+    *bytes = scan_tmp_words((size_t)A) * sizeof(uint32_t) + 256;
+    return GS355_OK;
+}
+
+int gs355_decode_count(const gs355_decoder* dec, const gs355_anchors* an, uint32_t* counts, uint32_t* offsets,
+                       void* scratch, size_t scratch_bytes, void* stream)
+{
+    DecodeArgs a;
+    int rc = fill_args(dec, an, &a);
+    if (rc) return rc;
+    if (a.A == 0) return GS355_OK;
+    if (!counts || !offsets || !scratch) return set_error(GS355_EINVAL, "counts / offsets / scratch is NULL");
+    size_t need = 0;
+    gs355_decode_scratch_bytes(a.A, &need);
+    if (scratch_bytes < need)
+        return set_error(GS355_ENOSPC, "decode scratch has %zu bytes, %zu needed", scratch_bytes, need);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(decode_kernel<true>, decode_grid(a.A), dim3(256), 0, s, a, counts, (const uint32_t*)nullptr, 0u,
+                       (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr);
+    GS355_CHECK_LAUNCH("decode: count");
+    return launch_exclusive_scan(counts, offsets, (size_t)a.A, static_cast<uint32_t*>(scratch), s);
+}
+
+int gs355_decode_emit(const gs355_decoder* dec, const gs355_anchors* an, const uint32_t* offsets, int64_t capacity,
+                      const gs355_decoded* out, void* stream)
+{
+    DecodeArgs a;
+    int rc = fill_args(dec, an, &a);
+    if (rc) return rc;
+    if (a.A == 0 || capacity == 0) return GS355_OK;
+    if (capacity < 0 || capacity > 0xFFFFFFFFll)
+        return set_error(GS355_EINVAL, "capacity must be in [0, 2^32) (got %lld)", (long long)capacity);
+    if (!offsets) return set_error(GS355_EINVAL, "offsets is NULL");
+    if (!out || !out->xyz || !out->color || !out->opacity || !out->scaling || !out->rot)
+        return set_error(GS355_EINVAL, "decoded outputs must all be non-NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(decode_kernel<false>, decode_grid(a.A), dim3(256), 0, s, a, (uint32_t*)nullptr, offsets,
+                       (uint32_t)capacity, out->xyz, out->color, out->opacity, out->scaling, out->rot);
+    GS355_CHECK_LAUNCH("decode: emit");
+    return GS355_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,296 @@
+"""Host-side counterparts of the reference's three Gaussian-splatting models:
+the callers on either side of the rasterizer.
+
+  GaussianModel  benchmarks/nerf/origin_gs/gs_model.py:112-228 (forward), :280-331 (prefilter_voxel);
+                 parameter getters / activations: landmark/nerf_components/model_components/fields/
+                 encodings/gaussian_encoding.py:89-97, 745-853
+  ScaffoldGS     benchmarks/nerf/scaffold_gs/gs_model.py:162-238, :385-436;
+                 getters: .../encodings/scaffoldgs_encoding.py:701-775
+  OctreeGS       benchmarks/nerf/octree_gs/gs_model.py:228-325, :445-497;
+                 level-of-detail mask: .../encodings/octreegs_encoding.py:238-294
+
+They keep the reference's call sequence (visibility prefilter -> optional
+anchor decode -> settings record re-assigned on the renderer -> rasterize),
+its eval-mode gather of the visible Gaussians and its `act_cache` behaviour,
+and its parameter names so checkpoints map one to one.  Forward / eval only:
+training, densification and checkpoint I/O are not part of this package.
+Activations and gathers are a handful of torch elementwise calls, as in the
+reference; everything per-Gaussian and per-pixel runs in the HIP library.
+"""
+import math
+from typing import Optional
+
+import torch
+from torch import nn
+
+from .anchor_decoder import FusedAnchorDecoder
+from .rasterizer import GaussianRasterizationSettings, GaussianRasterizer
+
+
+def _settings(camera, bg, scaling_modifier, sh_degree):
+    return GaussianRasterizationSettings(
+        image_height=int(camera.height), image_width=int(camera.width),
+        tanfovx=math.tan(camera.FovX * 0.5), tanfovy=math.tan(camera.FovY * 0.5), bg=bg,
+        scale_modifier=scaling_modifier, viewmatrix=camera.world_view_transform,
+        projmatrix=camera.full_proj_transform, sh_degree=sh_degree, campos=camera.camera_center,
+        prefiltered=False, debug=False,
+    )
+
+
+def _placeholder_renderer(bg):
+    # the reference builds its renderer once with empty placeholders (origin_gs/gs_model.py:82-97)
+    return GaussianRasterizer(raster_settings=GaussianRasterizationSettings(
+        image_height=0, image_width=0, tanfovx=0, tanfovy=0, bg=bg, scale_modifier=0, viewmatrix=torch.Tensor([]),
+        projmatrix=torch.Tensor([]), sh_degree=0, campos=torch.Tensor([]), prefiltered=False, debug=False))
+
+
+class GaussianModel(nn.Module):
+    """Vanilla 3DGS: raw parameters with exp / sigmoid / normalize activations."""
+
+    def __init__(self, xyz, features_dc, features_rest, scaling, rotation, opacity, sh_degree: int = 3,
+                 white_bkgd: bool = False, act_cache: bool = False, compute_cov3D_python: bool = False,
+                 convert_SHs_python: bool = False):
+        super().__init__()
+        self._xyz = nn.Parameter(xyz, requires_grad=False)  # [P,3]
+        self._features_dc = nn.Parameter(features_dc, requires_grad=False)  # [P,1,3]
+        self._features_rest = nn.Parameter(features_rest, requires_grad=False)  # [P,(deg+1)^2-1,3]
+        self._scaling = nn.Parameter(scaling, requires_grad=False)  # [P,3] log
+        self._rotation = nn.Parameter(rotation, requires_grad=False)  # [P,4]
+        self._opacity = nn.Parameter(opacity, requires_grad=False)  # [P,1] logit
+        self.active_sh_degree = self.max_sh_degree = sh_degree
+        self.act_cache = act_cache
+        self.compute_cov3D_python, self.convert_SHs_python = compute_cov3D_python, convert_SHs_python
+        self.register_buffer("background", torch.tensor([1.0, 1.0, 1.0] if white_bkgd else [0.0, 0.0, 0.0]))
+        self.renderer = _placeholder_renderer(self.background)
+        self._cache = {}
+        self.radii = self.visibility_filter = None
+
+    @classmethod
+    def from_activated(cls, means3D, scales, rotations, opacities, shs, **kw):
+        """Build from activated values (e.g. a synthetic scene) by inverting the activations."""
+        eps = 1e-7
+        op = opacities.clamp(eps, 1 - eps)
+        return cls(means3D, shs[:, :1].contiguous(), shs[:, 1:].contiguous(), torch.log(scales), rotations,
+                   torch.log(op / (1 - op)), **kw)
+
+    def _cached(self, name, fn):
+        if self.act_cache and not self.training:
+            if name not in self._cache:
+                self._cache[name] = fn()
+            return self._cache[name]
+        return fn()
+
+    @property
+    def get_xyz(self):
+        return self._xyz
+
+    @property
+    def get_scaling(self):
+        return self._cached("scaling", lambda: torch.exp(self._scaling))
+
+    @property
+    def get_rotation(self):
+        return self._cached("rotation", lambda: torch.nn.functional.normalize(self._rotation))
+
+    @property
+    def get_opacity(self):
+        return self._cached("opacity", lambda: torch.sigmoid(self._opacity))
+
+    @property
+    def get_features(self):
+        return self._cached("features", lambda: torch.cat((self._features_dc, self._features_rest), dim=1))
+
+    def get_covariance(self, scaling_modifier=1.0):
+        # L = R diag(mod * s), Sigma = L L^T packed (xx,xy,xz,yy,yz,zz): gaussian_encoding.py:22-38
+        s = scaling_modifier * self.get_scaling
+        q = self.get_rotation
+        r, x, y, z = q[:, 0], q[:, 1], q[:, 2], q[:, 3]
+        R = torch.stack([1 - 2 * (y * y + z * z), 2 * (x * y - r * z), 2 * (x * z + r * y),
+                         2 * (x * y + r * z), 1 - 2 * (x * x + z * z), 2 * (y * z - r * x),
+                         2 * (x * z - r * y), 2 * (y * z + r * x), 1 - 2 * (x * x + y * y)], dim=1).view(-1, 3, 3)
+        L = R * s[:, None, :]
+        S = L @ L.transpose(1, 2)
+        return torch.stack([S[:, 0, 0], S[:, 0, 1], S[:, 0, 2], S[:, 1, 1], S[:, 1, 2], S[:, 2, 2]], dim=1)
+
+    def prefilter_voxel(self, viewpoint_camera, scaling_modifier=1.0):
+        rasterizer = GaussianRasterizer(raster_settings=_settings(viewpoint_camera, self.background,
+                                                                  scaling_modifier, 1))
+        scales = rotations = cov3D_precomp = None
+        if self.compute_cov3D_python:
+            cov3D_precomp = self.get_covariance(scaling_modifier)
+        else:
+            scales, rotations = self.get_scaling, self.get_rotation
+        radii_pure = rasterizer.visible_filter(means3D=self.get_xyz, scales=None if scales is None else scales[:, :3],
+                                               rotations=rotations, cov3D_precomp=cov3D_precomp)
+        return radii_pure > 0
+
+    @torch.no_grad()
+    def forward(self, viewpoint_camera, scaling_modifier=1.0, override_color=None, render_exclude_filter=None):
+        viewpoint_camera = viewpoint_camera.to(self._xyz.device)
+        voxel_visible_mask = self.prefilter_voxel(viewpoint_camera)
+        if render_exclude_filter is not None:
+            voxel_visible_mask = voxel_visible_mask & render_exclude_filter
+        self.renderer.raster_settings = _settings(viewpoint_camera, self.background, scaling_modifier,
+                                                  self.active_sh_degree)
+        means3D, opacity = self.get_xyz, self.get_opacity
+        scales = rotations = cov3D_precomp = shs = colors_precomp = None
+        if self.compute_cov3D_python:
+            cov3D_precomp = self.get_covariance(scaling_modifier)
+        else:
+            scales, rotations = self.get_scaling, self.get_rotation
+        if override_color is not None:
+            colors_precomp = override_color
+        elif self.convert_SHs_python:
+            raise NotImplementedError("convert_SHs_python: SH -> RGB runs inside the preprocess kernel")
+        else:
+            shs = self.get_features
+        if not self.training:  # the reference renders only what its prefilter kept (origin_gs/gs_model.py:199-208)
+            mask = voxel_visible_mask.nonzero().squeeze(-1)
+            pick = lambda t: None if t is None else t[mask]  # noqa: E731
+            means3D, shs, colors_precomp, opacity = pick(means3D), pick(shs), pick(colors_precomp), pick(opacity)
+            scales, rotations, cov3D_precomp = pick(scales), pick(rotations), pick(cov3D_precomp)
+        rendered_image, radii, _ = self.renderer(
+            means3D=means3D, means2D=None, shs=shs, colors_precomp=colors_precomp, opacities=opacity, scales=scales,
+            rotations=rotations, cov3D_precomp=cov3D_precomp)
+        self.visibility_filter, self.radii = voxel_visible_mask, radii
+        return rendered_image
+
+
+class ScaffoldGS(nn.Module):
+    """Scaffold-GS: anchors decoded into neural Gaussians per frame."""
+
+    def __init__(self, anchor, anchor_feat, offset, scaling, rotation, n_offsets: int = 10, feat_dim: int = 32,
+                 add_opacity_dist: bool = True, add_cov_dist: bool = True, add_color_dist: bool = True,
+                 white_bkgd: bool = False, act_cache: bool = False):
+        super().__init__()
+        self._anchor = nn.Parameter(anchor, requires_grad=False)  # [A,3]
+        self._anchor_feat = nn.Parameter(anchor_feat, requires_grad=False)  # [A,32]
+        self._offset = nn.Parameter(offset, requires_grad=False)  # [A,n,3]
+        self._scaling = nn.Parameter(scaling, requires_grad=False)  # [A,6] log
+        self._rotation = nn.Parameter(rotation, requires_grad=False)  # [A,4]
+        self.act_cache = act_cache
+        self.anchor_decoder = FusedAnchorDecoder(
+            use_feat_bank=False, add_opacity_dist=add_opacity_dist, add_color_dist=add_color_dist,
+            add_cov_dist=add_cov_dist, view_dim=3, feat_dim=feat_dim, n_offsets=n_offsets)
+        self.register_buffer("background", torch.tensor([1.0, 1.0, 1.0] if white_bkgd else [0.0, 0.0, 0.0]))
+        self.renderer = _placeholder_renderer(self.background)
+        self._cache = {}
+        self.visibility_filter = self.voxel_visible_mask = None
+
+    @classmethod
+    def from_scene(cls, scene, **kw):
+        m = cls(scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation,
+                n_offsets=scene.n_offsets, **kw)
+        state = {}
+        for name, head in (("mlp_opacity", "opacity"), ("mlp_cov", "cov"), ("mlp_color", "color")):
+            w0, b0, w1, b1 = scene.mlp[head]
+            state.update({name + ".0.weight": w0, name + ".0.bias": b0, name + ".2.weight": w1, name + ".2.bias": b1})
+        m.anchor_decoder.load_state_dict(state)
+        return m
+
+    def _cached(self, name, fn):
+        if self.act_cache and not self.training:
+            if name not in self._cache:
+                self._cache[name] = fn()
+            return self._cache[name]
+        return fn()
+
+    @property
+    def get_anchor(self):
+        return self._anchor
+
+    @property
+    def get_anchor_feat(self):
+        return self._anchor_feat
+
+    @property
+    def get_offset(self):
+        return self._offset
+
+    @property
+    def get_scaling(self):
+        return self._cached("scaling", lambda: torch.exp(self._scaling))
+
+    @property
+    def get_rotation(self):
+        return self._cached("rotation", lambda: torch.nn.functional.normalize(self._rotation))
+
+    def _anchor_subset(self):
+        return None  # Scaffold-GS filters all anchors
+
+    def prefilter_voxel(self, viewpoint_camera, scaling_modifier=1.0):
+        rasterizer = GaussianRasterizer(raster_settings=_settings(viewpoint_camera, self.background,
+                                                                  scaling_modifier, 1))
+        subset = self._anchor_subset()
+        means3D, scales, rotations = self.get_anchor, self.get_scaling, self.get_rotation
+        if subset is not None:
+            means3D, scales, rotations = means3D[subset], scales[subset], rotations[subset]
+        radii_pure = rasterizer.visible_filter(means3D=means3D, scales=scales[:, :3], rotations=rotations,
+                                               cov3D_precomp=None)
+        if subset is None:
+            return radii_pure > 0
+        visible_mask = subset.clone()
+        visible_mask[subset] = radii_pure > 0
+        return visible_mask
+
+    def _before_prefilter(self, viewpoint_camera):
+        pass
+
+    @torch.no_grad()
+    def forward(self, viewpoint_camera, scaling_modifier=1.0, retain_grad=False, render_exclude_filter=None):
+        viewpoint_camera = viewpoint_camera.to(self._anchor.device)
+        self._before_prefilter(viewpoint_camera)
+        voxel_visible_mask = self.prefilter_voxel(viewpoint_camera)
+        if render_exclude_filter is not None:
+            voxel_visible_mask = voxel_visible_mask & render_exclude_filter
+        xyz, color, opacity, scaling, rot, _, _ = self.anchor_decoder(
+            camera_center=viewpoint_camera.camera_center, anchor=self.get_anchor, anchor_feat=self.get_anchor_feat,
+            offset=self.get_offset, scaling=self.get_scaling, visible_mask=voxel_visible_mask)
+        self.renderer.raster_settings = _settings(viewpoint_camera, self.background, scaling_modifier, 1)
+        rendered_image, radii, _ = self.renderer(
+            means3D=xyz, means2D=None, shs=None, colors_precomp=color, opacities=opacity, scales=scaling,
+            rotations=rot, cov3D_precomp=None)
+        self.visibility_filter, self.voxel_visible_mask = radii > 0, voxel_visible_mask
+        return rendered_image
+
+
+class OctreeGS(ScaffoldGS):
+    """Octree-GS: Scaffold-GS plus a per-frame level-of-detail mask over the anchors."""
+
+    def __init__(self, anchor, anchor_feat, offset, scaling, rotation, level, voxel_size: float, standard_dist: float,
+                 fork: int = 2, extra_level=None, enable_lod: bool = True, dist2level: str = "round", **kw):
+        super().__init__(anchor, anchor_feat, offset, scaling, rotation, **kw)
+        if dist2level not in ("floor", "round", "ceil"):
+            raise NotImplementedError("dist2level=%r (the progressive mode is dead code from the reference's model, "
+                                      "octree_gs/gs_model.py:247)" % dist2level)
+        self.register_buffer("_level", level.reshape(-1, 1).float())  # [A,1]
+        self.register_buffer("_extra_level", torch.zeros(anchor.shape[0]) if extra_level is None else extra_level)
+        self.voxel_size, self.standard_dist, self.fork = float(voxel_size), float(standard_dist), int(fork)
+        self.enable_lod, self.dist2level = enable_lod, dist2level
+        self._anchor_mask: Optional[torch.Tensor] = None
+
+    def set_anchor_mask(self, cam_center, iteration, resolution_scale):
+        """octreegs_encoding.py:238-264 in eval mode: keep anchors whose level does not exceed the level
+        predicted from their distance to the camera."""
+        if not self.enable_lod:
+            self._anchor_mask = torch.ones(self._level.shape[0], dtype=torch.bool, device=self._level.device)
+            return
+        anchor_pos = self._anchor + (self.voxel_size / 2) / (float(self.fork) ** self._level)
+        dist = torch.sqrt(torch.sum((anchor_pos - cam_center) ** 2, dim=1)) * resolution_scale
+        pred_level = torch.log2(self.standard_dist / dist) / math.log2(self.fork) + self._extra_level
+        cur_level = torch.max(self._level) - torch.min(self._level)
+        if self.dist2level == "floor":
+            int_level = torch.floor(pred_level).int()
+        elif self.dist2level == "round":
+            int_level = torch.round(pred_level).int()
+        else:
+            int_level = torch.ceil(pred_level).int()
+        int_level = torch.clamp(int_level, min=0, max=int(cur_level.item()))
+        self._anchor_mask = self._level.squeeze(dim=1) <= int_level
+
+    def _before_prefilter(self, viewpoint_camera):
+        if not self.training:
+            self.set_anchor_mask(viewpoint_camera.camera_center, -1, viewpoint_camera.resolution_scale)
+
+    def _anchor_subset(self):
+        return self._anchor_mask

@@ -148,3 +148,44 @@ def test_visible_filter_validates():
     half = _gauss()
     half.rotations = None
     assert "scale/rotation" in _err(_lib.GS355_EINVAL, vf, f, half, 0x1000)
+
+
+def _decoder(feat=32, n=10, in_dim=(36, 36, 36), ptr=0x1000):
+    d = _lib.Decoder()
+    d.feat_dim, d.n_offsets = feat, n
+    for j in range(3):
+        d.in_dim[j] = in_dim[j]
+        d.w0[j] = d.b0[j] = d.w1[j] = d.b1[j] = ptr
+    return d
+
+
+def _anchors(A=10, ptr=0x1000):
+    a = _lib.Anchors()
+    a.A = A
+    a.anchor = a.feat = a.offset = a.scaling = a.visible_mask = a.campos = ptr
+    return a
+
+
+def test_decode_validates_before_any_hip_call():
+    lib = _lib.load()
+    count = lambda d, a, c, o, s, n: lib.gs355_decode_count(C.byref(d), C.byref(a), c, o, s, n, None)  # noqa: E731
+    assert "feat_dim" in _err(_lib.GS355_EINVAL, count, _decoder(feat=64), _anchors(), 0x1000, 0x1000, 0x1000, 1 << 20)
+    assert "offsets per anchor" in _err(_lib.GS355_EINVAL, count, _decoder(n=11), _anchors(), 0x1000, 0x1000, 0x1000,
+                                        1 << 20)
+    assert "input width" in _err(_lib.GS355_EINVAL, count, _decoder(in_dim=(36, 40, 36)), _anchors(), 0x1000, 0x1000,
+                                 0x1000, 1 << 20)
+    bad = _decoder()
+    bad.w1[2] = None
+    assert "head 2" in _err(_lib.GS355_EINVAL, count, bad, _anchors(), 0x1000, 0x1000, 0x1000, 1 << 20)
+    missing = _anchors()
+    missing.offset = None
+    assert "non-NULL" in _err(_lib.GS355_EINVAL, count, _decoder(), missing, 0x1000, 0x1000, 0x1000, 1 << 20)
+    assert "aligned" in _err(_lib.GS355_EINVAL, count, _decoder(), _anchors(ptr=0x1004), 0x1000, 0x1000, 0x1000, 1 << 20)
+    assert "scratch" in _err(_lib.GS355_EINVAL, count, _decoder(), _anchors(), 0x1000, 0x1000, None, 1 << 20)
+    assert "needed" in _err(_lib.GS355_ENOSPC, count, _decoder(), _anchors(A=100_000), 0x1000, 0x1000, 0x1000, 16)
+    out = _lib.Decoded()
+    emit = lambda d, a, o, cap, dst: lib.gs355_decode_emit(C.byref(d), C.byref(a), o, cap, C.byref(dst), None)  # noqa: E731
+    assert "outputs" in _err(_lib.GS355_EINVAL, emit, _decoder(), _anchors(), 0x1000, 10, out)
+    assert "capacity" in _err(_lib.GS355_EINVAL, emit, _decoder(), _anchors(), 0x1000, -1, out)
+    need = C.c_size_t()
+    assert lib.gs355_decode_scratch_bytes(1000, C.byref(need)) == 0 and need.value >= 256

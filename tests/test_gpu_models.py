@@ -1,0 +1,108 @@
+"""GPU tests of the model-side callers (landmarksystem_amd/models.py): the
+vanilla / Scaffold / Octree forward sequences of the reference, end to end,
+with the rasterizer checked against the oracle on the Gaussians it was given."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from landmarksystem_amd import scenes
+from landmarksystem_amd.models import GaussianModel, OctreeGS, ScaffoldGS
+from oracle import anchor_oracle as ao
+from oracle import c_oracle as co
+from tests.helpers import oracle_frame, oracle_gaussians, psnr
+
+pytestmark = pytest.mark.gpu
+
+
+def test_vanilla_model_forward(gpu_device):
+    scene = scenes.config2(P=50_000, width=640, height=360)
+    model = GaussianModel.from_activated(scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs,
+                                         sh_degree=3, act_cache=True).to(gpu_device).eval()
+    image = model(scene.camera)
+    # activations round-trip (log/exp, logit/sigmoid) perturb the inputs by an ulp: feed the oracle the
+    # model's own activated tensors
+    act = scenes.GaussianScene("act", model.get_xyz.cpu(), model.get_scaling.cpu(), model.get_rotation.cpu(),
+                               model.get_opacity.cpu(), model.get_features.cpu(), 3, scene.cameras, scene.bg)
+    ref = co.render(oracle_frame(act), oracle_gaussians(act))
+    solid = ref["fragile"] == 0
+    assert np.abs(image.cpu().numpy() - ref["image"])[:, solid].max() <= 1e-4
+    assert psnr(image.cpu().numpy(), ref["image"]) >= 60.0
+    vis = ref["radii"] > 0
+    assert torch.equal(model.visibility_filter.cpu(), torch.from_numpy(vis))
+    assert model.radii.shape[0] == int(vis.sum())  # eval mode renders the prefiltered subset
+    np.testing.assert_array_equal(model.radii.cpu().numpy(), ref["radii"][vis])
+    assert "scaling" in model._cache  # act_cache: activations computed once
+    again = model(scene.camera)
+    assert torch.equal(image, again)
+
+
+def scaffold_reference_image(scene, model, cam, visible_mask):
+    """Oracle decode (fp32 torch) -> oracle rasterizer."""
+    dec = ao.decode(cam.camera_center, scene.anchor, scene.anchor_feat, scene.offset, scene.scaling,
+                    visible_mask, scene.mlp, scene.n_offsets)
+    tmp = scenes.GaussianScene("dec", dec["xyz"], dec["scaling"], dec["rot"], dec["opacity"],
+                               torch.zeros(dec["xyz"].shape[0], 1, 3), 1, [cam], scene.bg)
+    return co.render(oracle_frame(tmp, sh_degree=1), oracle_gaussians(tmp, colors_precomp=dec["color"].numpy())), dec
+
+
+def test_scaffold_model_forward(gpu_device):
+    scene = scenes.config5(A=30_000, width=640, height=360)
+    model = ScaffoldGS.from_scene(scene).to(gpu_device).eval()
+    cam = scene.camera
+    image = model(cam)
+    assert image.shape == (3, 360, 640)
+    # (1) anchor-level visibility equals the oracle's visible filter on the anchors
+    vis_ref = co.visible_filter(oracle_frame(scenes.GaussianScene("a", scene.anchor, scene.scaling[:, :3],
+                                scene.rotation, torch.zeros(1), torch.zeros(1, 1, 3), 1, [cam], scene.bg),
+                                sh_degree=1), scene.anchor.numpy(), scales=model.get_scaling[:, :3].cpu().numpy(),
+                                rotations=model.get_rotation.cpu().numpy()) > 0
+    assert torch.equal(model.voxel_visible_mask.cpu(), torch.from_numpy(vis_ref))
+    # (2) end to end against oracle decode + oracle rasterizer.  The decoded Gaussians agree to ~1e-5, so the
+    # discrete radius / tile decisions can differ for a few of them: compare images with a PSNR bar.
+    ref, dec = scaffold_reference_image(scene, model, cam, torch.from_numpy(vis_ref))
+    assert abs(int(model.visibility_filter.shape[0]) - dec["xyz"].shape[0]) <= 2
+    assert psnr(image.cpu().numpy(), ref["image"]) >= 50.0
+    # (3) bit-level rasterizer parity on the Gaussians the GPU decoder produced
+    xyz, color, opacity, scaling, rot, _, _ = model.anchor_decoder(
+        camera_center=cam.camera_center.to(gpu_device), anchor=model.get_anchor, anchor_feat=model.get_anchor_feat,
+        offset=model.get_offset, scaling=model.get_scaling, visible_mask=model.voxel_visible_mask)
+    tmp = scenes.GaussianScene("gpu-dec", xyz.cpu(), scaling.cpu(), rot.cpu(), opacity.cpu(),
+                               torch.zeros(xyz.shape[0], 1, 3), 1, [cam], scene.bg)
+    ref2 = co.render(oracle_frame(tmp, sh_degree=1), oracle_gaussians(tmp, colors_precomp=color.cpu().numpy()))
+    np.testing.assert_array_equal((model.visibility_filter.cpu().numpy()), ref2["radii"] > 0)
+    solid = ref2["fragile"] == 0
+    assert np.abs(image.cpu().numpy() - ref2["image"])[:, solid].max() <= 1e-4
+    assert psnr(image.cpu().numpy(), ref2["image"]) >= 60.0
+
+
+def test_octree_lod_mask_and_forward(gpu_device):
+    scene = scenes.config5(A=20_000, width=480, height=270)
+    g = torch.Generator().manual_seed(5)
+    level = torch.randint(0, 5, (20_000,), generator=g)
+    common = dict(n_offsets=scene.n_offsets)
+    model = OctreeGS(scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
+                     voxel_size=0.5, standard_dist=250.0, fork=2, **common)
+    scaffold = ScaffoldGS.from_scene(scene)
+    model.anchor_decoder.load_state_dict(scaffold.anchor_decoder.state_dict())
+    model = model.to(gpu_device).eval()
+    cam = scene.camera
+    image = model(cam)
+    # level-of-detail mask against the closed form level <= round(log2(standard_dist / dist)) clamped to [0, L-1]
+    pos = scene.anchor.double() + (0.5 / 2) / (2.0 ** level.double())[:, None]
+    dist = (pos - cam.camera_center.double()).norm(dim=1)
+    want_level = torch.clamp(torch.round(torch.log2(250.0 / dist)), 0, 4)
+    want = level.double() <= want_level
+    got = model._anchor_mask.cpu()
+    near_half = (torch.log2(250.0 / dist) % 1 - 0.5).abs() < 1e-4  # fp32 vs fp64 rounding at .5 boundaries
+    assert torch.equal(got[~near_half], want[~near_half])
+    assert 0 < int(got.sum()) < 20_000
+    # anchors outside the mask never become visible
+    assert not bool((model.voxel_visible_mask.cpu() & ~got).any())
+    # the frame equals a Scaffold-GS render with the masked-out anchors excluded
+    scaffold = scaffold.to(gpu_device).eval()
+    image2 = scaffold(cam, render_exclude_filter=model._anchor_mask)
+    assert torch.equal(image, image2)
+    model.enable_lod = False
+    assert torch.equal(model(cam), scaffold(cam))

@@ -48,7 +48,7 @@ def test_workspace_layout_is_aligned_ordered_and_sized():
     assert L.values[1] - L.values[0] >= n_cap * 4
     tiles = 120 * 68
     assert L.bin_matrix - L.ranges >= tiles * 8 and L.total_bytes - L.tile_lists >= (4 + 4 * tiles) * 4
-    assert L.tile_base - L.bin_matrix >= 512 * tiles * 4
+    assert L.tile_base - L.bin_matrix >= 256 * tiles * 4
     assert L.sort_bits == 32 + 13 and L.sort_passes == 6 and L.sorted_buffer == 0
     L4k = _lib.workspace_layout(10, 10, 3840, 2160)
     assert L4k.sort_bits == 47 and L4k.sort_passes == 6

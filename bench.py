@@ -23,6 +23,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+# HBM bytes per launch of the heaviest kernels on the default workload (6M Gaussians, 1080p), from two
+# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what
+# the same counter reads for the 1 GiB copy of --calibration-copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
+MEASURED_TRAFFIC_BYTES = {"blend": 1849.0e6, "preprocess": 1727.6e6}
 FP32_PEAK_TFLOPS = 157.3  # MI355X fp32 vector peak (packed FMA); this build issues unpacked FP32 only
 
 
@@ -35,6 +40,9 @@ def parse_args():
     ap.add_argument("--gaussians", type=int, default=None, help="override the Gaussian count (not the headline workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--stage-steps", type=int, default=20)
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
 
 
@@ -137,6 +145,13 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     fps = args.steps / elapsed
 
+    if args.calibration_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # 1 GiB read + 1 GiB written
+        torch.cuda.synchronize()
+        del src, dst
+
     # per-stage breakdown on the same inputs
     inp = pipeline.FrameInputs(rast.raster_settings, d.means3D, opacities=d.opacities, shs=d.shs, scales=d.scales,
                                rotations=d.rotations)
@@ -176,18 +191,20 @@ def main():
                        "sorted_keys_per_s": round(N / sort_ms * 1e3) if N else 0,
                        "blend_frames_per_s": round(1e3 / stage_ms["blend"], 1)}
 
+    # counter-measured traffic only applies to the workload it was measured on
+    traffic = MEASURED_TRAFFIC_BYTES if (args.config == 3 and not args.gaussians) else {}
     shipped = {"preprocess": stage_ms["preprocess"], "keys_sort_ranges": sort_ms,
                "blend": stage_ms["blend"]}
     dominant = max(shipped, key=lambda n: shipped[n])
     if dominant == "blend":
         roofline = {"bound": "mfma", "kernel": "blend_kernel", "achieved": stages["blend"]["TFLOPs_upper"],
                     "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": stages["blend"]["frac_fp32_upper"],
-                    "traffic": None,
+                    "traffic": traffic.get("blend"),
                     "note": "FP32 VALU kernel (no MFMA); peak is the MI355X fp32 figure; flops = 25 x 256 x sum of "
                             "tile range lengths (upper bound on evaluated pixel-Gaussian pairs)"}
     else:
         roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": None}
+                    "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": traffic.get(dominant)}
 
     result = {
         "metric": "1080p frames/sec at 6M Gaussians (1 GPU)",

@@ -42,37 +42,46 @@ __global__ __launch_bounds__(256) void ranges_kernel(const gs355_header* __restr
     if (j == n - 1) ranges[2 * t + 1] = n;
 }
 
-// exp(power) -> alpha, the three discrete tests and the accumulation for one
-// (pixel, Gaussian) pair.  `power` is evaluated with unfused multiplies and
-// adds in a fixed order so that the sign test and the alpha threshold see the
-// same exponent as a scalar evaluation of the same formula.
+// One (pixel, Gaussian) pair: exponent, alpha, the three discrete tests and the
+// accumulation.  The exponent is evaluated with unfused multiplies and adds in
+// a fixed order (contraction is switched off for it), so the sign test and the
+// alpha threshold see the same value as a scalar evaluation of the formula.
+//
+// A pixel's transmittance T stays >= 1e-4 while it is live, so the sign of T
+// carries the "finished" state: T > 0 live, T <= 0 finished with |T| the final
+// transmittance (pixels outside the image start at -1).  A finished pixel can
+// neither accumulate (its test_T is <= 0) nor finish again.
 struct PixelState {
     float T, c0, c1, c2, depth;
-    bool done;
 };
+
+__device__ __forceinline__ float splat_exponent(float dx, float dy, float qx, float qy, float qz)
+{
+#pragma clang fp contract(off)
+    const float t1 = (qx * dx) * dx;
+    const float t2 = (qz * dy) * dy;
+    const float t3 = (qy * dx) * dy;
+    return -0.5f * (t1 + t2) - t3;
+}
 
 __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, const float4 a, const float4 b,
                                           const float4 c)
 {
     const float dx = a.x - pxf, dy = a.y - pyf;
-    const float t1 = __fmul_rn(__fmul_rn(a.z, dx), dx);
-    const float t2 = __fmul_rn(__fmul_rn(b.x, dy), dy);
-    const float t3 = __fmul_rn(__fmul_rn(a.w, dx), dy);
-    const float power = __fsub_rn(__fmul_rn(-0.5f, __fadd_rn(t1, t2)), t3);
-    if (power > 0.0f) return;
+    const float power = splat_exponent(dx, dy, a.z, a.w, b.x);
     const float alpha = fminf(0.99f, b.y * __expf(power));
-    if (alpha < 1.0f / 255.0f) return;
+    if (power > 0.0f || alpha < 1.0f / 255.0f) return;
     const float test_T = p.T * (1.0f - alpha);
-    if (test_T < 0.0001f) {
-        p.done = true;
-        return;
+    if (test_T >= 0.0001f) {
+        const float w = alpha * p.T;
+        p.c0 += b.z * w;
+        p.c1 += b.w * w;
+        p.c2 += c.x * w;
+        p.depth += c.y * w;
+        p.T = test_T;
+    } else if (p.T > 0.0f) {
+        p.T = -p.T;  // this Gaussian is not applied; the pixel is finished
     }
-    const float w = alpha * p.T;
-    p.c0 += b.z * w;
-    p.c1 += b.w * w;
-    p.c2 += c.x * w;
-    p.depth += c.y * w;
-    p.T = test_T;
 }
 
 // kCull: each wavefront first tests the staged Gaussians against its own 8x8
@@ -104,10 +113,10 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
     const float qx_lo = (float)qx0, qx_hi = (float)(qx0 + 7), qy_lo = (float)qy0, qy_hi = (float)(qy0 + 7);
 
     const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
-    PixelState p = {1.0f, 0.0f, 0.0f, 0.0f, 0.0f, !inside};
+    PixelState p = {inside ? 1.0f : -1.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 
     for (uint32_t base = lo; base < hi; base += 256) {
-        const bool wave_done = __ballot(!p.done) == 0ull;
+        const bool wave_done = __ballot(p.T > 0.0f) == 0ull;
         if (lane == 0) s_wave_done[wave] = wave_done ? 1u : 0u;
         const uint32_t j = base + tid;
         if (j < hi) {
@@ -136,8 +145,8 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
                     while (todo != 0ull) {
                         const int kk = chunk + (int)__builtin_ctzll(todo);
                         todo &= todo - 1ull;
-                        if (!p.done) blend_one(p, pxf, pyf, s_a[kk], s_b[kk], s_c[kk]);
-                        if (__ballot(!p.done) == 0ull) {
+                        blend_one(p, pxf, pyf, s_a[kk], s_b[kk], s_c[kk]);
+                        if (__ballot(p.T > 0.0f) == 0ull) {
                             finished = true;
                             break;
                         }
@@ -145,8 +154,8 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
                 }
             } else {
                 for (int k = 0; k < count; ++k) {
-                    if (__ballot(!p.done) == 0ull) break;
-                    if (!p.done) blend_one(p, pxf, pyf, s_a[k], s_b[k], s_c[k]);
+                    if (__ballot(p.T > 0.0f) == 0ull) break;
+                    blend_one(p, pxf, pyf, s_a[k], s_b[k], s_c[k]);
                 }
             }
         }
@@ -156,11 +165,12 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
     if (inside) {
         const size_t plane = (size_t)f.W * f.H;
         const size_t o = (size_t)py * f.W + px;
-        image[o] = p.c0 + p.T * f.bg[0];
-        image[plane + o] = p.c1 + p.T * f.bg[1];
-        image[2 * plane + o] = p.c2 + p.T * f.bg[2];
+        const float T = fabsf(p.T);
+        image[o] = p.c0 + T * f.bg[0];
+        image[plane + o] = p.c1 + T * f.bg[1];
+        image[2 * plane + o] = p.c2 + T * f.bg[2];
         if (out_depth) out_depth[o] = p.depth;
-        if (out_alpha) out_alpha[o] = 1.0f - p.T;
+        if (out_alpha) out_alpha[o] = 1.0f - T;
     }
 }
 

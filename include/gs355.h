@@ -107,6 +107,8 @@ typedef struct gs355_layout {
     size_t header;        /* gs355_header */
     size_t records;       /* f32[P][12]: px, py, conic_x, conic_y, conic_z, opacity, r, g, b, depth, reach_x, reach_y */
     size_t tiles_touched; /* u32[P] */
+    size_t rects;         /* u16[P][4] tile rectangle (x0, y0, x1, y1), all zero when culled */
+    size_t depth_bits;    /* u32[P]    view depth as raw bits (written for survivors only) */
     size_t offsets;       /* u32[P]   inclusive prefix sum of tiles_touched */
     size_t scan_tmp;      /* u32[...] block sums of the scans */
     size_t keys[2];       /* u64[n_cap] x 2 (ping-pong) */

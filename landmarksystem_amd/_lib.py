@@ -70,6 +70,8 @@ class Layout(C.Structure):
         ("header", C.c_size_t),
         ("records", C.c_size_t),
         ("tiles_touched", C.c_size_t),
+        ("rects", C.c_size_t),
+        ("depth_bits", C.c_size_t),
         ("offsets", C.c_size_t),
         ("scan_tmp", C.c_size_t),
         ("keys", C.c_size_t * 2),

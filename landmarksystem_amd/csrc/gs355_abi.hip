@@ -46,6 +46,8 @@ int check_dims(int32_t P, int64_t n_cap, int32_t W, int32_t H)
         return set_error(GS355_EOVERFLOW, "n_cap %lld exceeds the 32-bit key index range (%lld)", (long long)n_cap,
                          (long long)kMaxKeys);
     const int64_t gx = (W + kTile - 1) / kTile, gy = (H + kTile - 1) / kTile;
+    if (gx > 65535 || gy > 65535)
+        return set_error(GS355_EOVERFLOW, "image %dx%d has more than 65535 tiles along an axis", W, H);
     if (gx * gy > (1ll << 24))
         return set_error(GS355_EOVERFLOW, "image %dx%d has more than 2^24 tiles", W, H);
     return GS355_OK;
@@ -72,6 +74,8 @@ int make_layout(int32_t P, int64_t n_cap, int32_t W, int32_t H, gs355_layout* L)
     L->header = take(sizeof(gs355_header));
     L->records = take(p * kRecordFloats * sizeof(float));
     L->tiles_touched = take(p * sizeof(uint32_t));
+    L->rects = take(p * sizeof(uint64_t));
+    L->depth_bits = take(p * sizeof(uint32_t));
     L->offsets = take(p * sizeof(uint32_t));
     L->scan_tmp = take(tmp_words * sizeof(uint32_t));
     L->keys[0] = take(n * sizeof(uint64_t));
@@ -208,6 +212,8 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     auto* header = reinterpret_cast<gs355_header*>(ws + L.header);
     auto* records = reinterpret_cast<float*>(ws + L.records);
     auto* touched = reinterpret_cast<uint32_t*>(ws + L.tiles_touched);
+    auto* rects = reinterpret_cast<uint64_t*>(ws + L.rects);
+    auto* depth_bits = reinterpret_cast<uint32_t*>(ws + L.depth_bits);
     auto* offsets = reinterpret_cast<uint32_t*>(ws + L.offsets);
     auto* scan_tmp = reinterpret_cast<uint32_t*>(ws + L.scan_tmp);
     uint64_t* keys[2] = {reinterpret_cast<uint64_t*>(ws + L.keys[0]), reinterpret_cast<uint64_t*>(ws + L.keys[1])};
@@ -223,7 +229,7 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     const uint32_t cap = (uint32_t)n_cap;
 
     if (stage_mask & GS355_STAGE_PREPROCESS)
-        if ((rc = launch_preprocess(fa, *g, false, records, touched, out->radii, s))) return rc;
+        if ((rc = launch_preprocess(fa, *g, false, records, touched, rects, depth_bits, out->radii, s))) return rc;
     if (stage_mask & GS355_STAGE_SCAN)
         if ((rc = launch_scan_offsets(touched, out->radii, g->P, offsets, scan_tmp, header, cap, s))) return rc;
     if (stage_mask & GS355_STAGE_DUPLICATE)
@@ -237,13 +243,13 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     const int tiles = fa.grid_x * fa.grid_y;
     uint64_t* buckets = keys[1 - L.sorted_buffer];
     if (stage_mask & GS355_STAGE_TILE_COUNT) {
-        if ((rc = launch_tile_count(fa, g->P, records, out->radii, bin_matrix, bin_visible, s))) return rc;
+        if ((rc = launch_tile_count(fa, g->P, rects, bin_matrix, bin_visible, s))) return rc;
         if ((rc = launch_tile_layout(g->P, bin_matrix, bin_visible, tiles, cap, header, tile_base, ranges, tile_lists,
                                      s)))
             return rc;
     }
     if (stage_mask & GS355_STAGE_TILE_SCATTER)
-        if ((rc = launch_tile_scatter(fa, g->P, records, out->radii, header, bin_matrix, tile_base, buckets, s)))
+        if ((rc = launch_tile_scatter(fa, g->P, rects, depth_bits, header, bin_matrix, tile_base, buckets, s)))
             return rc;
     if (stage_mask & GS355_STAGE_TILESORT)
         if ((rc = launch_tile_sort(header, tiles, ranges, tile_lists, buckets, keys[L.sorted_buffer],
@@ -269,7 +275,7 @@ int gs355_visible_filter(const gs355_frame* frame, const gs355_gaussians* g, int
     if ((rc = check_geometry_inputs(g))) return rc;
     if (g->P > 0 && !radii) return set_error(GS355_EINVAL, "radii is NULL");
     const FrameArgs fa = make_args(frame);
-    return launch_preprocess(fa, *g, true, nullptr, nullptr, radii, static_cast<hipStream_t>(stream));
+    return launch_preprocess(fa, *g, true, nullptr, nullptr, nullptr, nullptr, radii, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

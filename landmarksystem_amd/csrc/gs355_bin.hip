@@ -32,8 +32,8 @@ constexpr int kInlineTiles = 32;  // splats touching more tiles than this are ex
 // than kInlineTiles tiles are queued and walked by all threads together.
 template <bool kScatter>
 __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P, int per_group,
-                                                          const float* __restrict__ records,
-                                                          const int32_t* __restrict__ radii,
+                                                          const uint64_t* __restrict__ rects,
+                                                          const uint32_t* __restrict__ depth_bits,
                                                           const gs355_header* __restrict__ header,
                                                           uint32_t* __restrict__ matrix,
                                                           const uint32_t* __restrict__ tile_base,
@@ -59,18 +59,18 @@ __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P
         __syncthreads();
         const int i = base + tid;
         if (i < g_end) {
-            const int rad = radii[i];
-            if (rad > 0) {
+            const uint64_t r = rects[i];
+            const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
+                      y1 = (int)(r >> 48);
+            const int w = x1 - x0, area = w * (y1 - y0);
+            if (area > 0) {
                 ++visible;
-                const float* __restrict__ rec = records + (size_t)i * kRecordFloats;
-                const Rect q = tile_rect(rec[0], rec[1], rad, f.grid_x, f.grid_y);
-                const int w = q.x1 - q.x0, area = w * (q.y1 - q.y0);
                 if (area > kInlineTiles) {
                     s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
                 } else {
-                    const uint64_t payload = ((uint64_t)__float_as_uint(rec[9]) << 32) | (uint64_t)(uint32_t)i;
-                    for (int ty = q.y0; ty < q.y1; ++ty)
-                        for (int tx = q.x0; tx < q.x1; ++tx) {
+                    const uint64_t payload = kScatter ? ((uint64_t)depth_bits[i] << 32) | (uint64_t)(uint32_t)i : 0ull;
+                    for (int ty = y0; ty < y1; ++ty)
+                        for (int tx = x0; tx < x1; ++tx) {
                             const uint32_t slot = atomicAdd(&s_tile[ty * f.grid_x + tx], 1u);
                             if (kScatter) buckets[slot] = payload;
                         }
@@ -81,12 +81,13 @@ __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P
         const uint32_t nq = s_nqueue;
         for (uint32_t k = 0; k < nq; ++k) {
             const uint32_t gi = s_queue[k];
-            const float* __restrict__ rec = records + (size_t)gi * kRecordFloats;
-            const Rect q = tile_rect(rec[0], rec[1], radii[gi], f.grid_x, f.grid_y);
-            const int w = q.x1 - q.x0, area = w * (q.y1 - q.y0);
-            const uint64_t payload = ((uint64_t)__float_as_uint(rec[9]) << 32) | (uint64_t)gi;
+            const uint64_t r = rects[gi];
+            const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
+                      y1 = (int)(r >> 48);
+            const int w = x1 - x0, area = w * (y1 - y0);
+            const uint64_t payload = kScatter ? ((uint64_t)depth_bits[gi] << 32) | (uint64_t)gi : 0ull;
             for (int e = tid; e < area; e += kBinThreads) {
-                const int ty = q.y0 + e / w, tx = q.x0 + e % w;
+                const int ty = y0 + e / w, tx = x0 + e % w;
                 const uint32_t slot = atomicAdd(&s_tile[ty * f.grid_x + tx], 1u);
                 if (kScatter) buckets[slot] = payload;
             }
@@ -671,17 +672,17 @@ static int set_bin_lds(const void* fn, size_t bytes)
     return GS355_OK;
 }
 
-int launch_tile_count(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii, uint32_t* matrix,
-                      uint32_t* group_visible, hipStream_t s)
+int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint32_t* matrix, uint32_t* group_visible,
+                      hipStream_t s)
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
     const size_t lds = (size_t)f.grid_x * f.grid_y * sizeof(uint32_t);
     int rc = set_bin_lds(reinterpret_cast<const void*>(bin_kernel<false>), lds);
     if (rc) return rc;
-    hipLaunchKernelGGL(bin_kernel<false>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, records, radii,
-                       (const gs355_header*)nullptr, matrix, (const uint32_t*)nullptr, group_visible,
-                       (uint64_t*)nullptr);
+    hipLaunchKernelGGL(bin_kernel<false>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, rects,
+                       (const uint32_t*)nullptr, (const gs355_header*)nullptr, matrix, (const uint32_t*)nullptr,
+                       group_visible, (uint64_t*)nullptr);
     GS355_CHECK_LAUNCH("bin: count");
     return GS355_OK;
 }
@@ -700,7 +701,7 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
     return GS355_OK;
 }
 
-int launch_tile_scatter(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
+int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
                         const gs355_header* header, const uint32_t* matrix, const uint32_t* tile_base,
                         uint64_t* buckets, hipStream_t s)
 {
@@ -709,7 +710,7 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const float* records, con
     const size_t lds = (size_t)f.grid_x * f.grid_y * sizeof(uint32_t);
     int rc = set_bin_lds(reinterpret_cast<const void*>(bin_kernel<true>), lds);
     if (rc) return rc;
-    hipLaunchKernelGGL(bin_kernel<true>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, records, radii,
+    hipLaunchKernelGGL(bin_kernel<true>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, rects, depth_bits,
                        header, const_cast<uint32_t*>(matrix), tile_base, (uint32_t*)nullptr, buckets);
     GS355_CHECK_LAUNCH("bin: scatter");
     return GS355_OK;

@@ -65,7 +65,7 @@ __device__ __forceinline__ Rect tile_rect(float px, float py, int radius, int gr
 
 // stage launchers (each returns a gs355_status)
 int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_only, float* records,
-                      uint32_t* tiles_touched, int32_t* radii, hipStream_t s);
+                      uint32_t* tiles_touched, uint64_t* rects, uint32_t* depth_bits, int32_t* radii, hipStream_t s);
 int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int32_t P, uint32_t* offsets,
                         uint32_t* scan_tmp, gs355_header* header, uint32_t n_cap, hipStream_t s);
 int launch_duplicate(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
@@ -85,11 +85,11 @@ constexpr int kBinThreads = 1024;       // threads per binning workgroup
 constexpr int kBinMaxGroups = 256;      // binning workgroups (each owns a contiguous slice of the Gaussians)
 constexpr int kBinMaxTiles = 36000;     // per-tile counters of one workgroup must fit in LDS (4 B each)
 int bin_groups(int32_t P, int* per_group);
-int launch_tile_count(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii, uint32_t* matrix,
-                      uint32_t* group_visible, hipStream_t s);
+int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint32_t* matrix, uint32_t* group_visible,
+                      hipStream_t s);
 int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visible, int tiles, uint32_t n_cap,
                        gs355_header* header, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s);
-int launch_tile_scatter(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
+int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
                         const gs355_header* header, const uint32_t* matrix, const uint32_t* tile_base,
                         uint64_t* buckets, hipStream_t s);
 int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, const uint32_t* lists,

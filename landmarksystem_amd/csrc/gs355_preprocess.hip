@@ -85,6 +85,8 @@ template <bool kRadiiOnly>
 __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaussians g,
                                                          float* __restrict__ records,
                                                          uint32_t* __restrict__ tiles_touched,
+                                                         uint64_t* __restrict__ rects,
+                                                         uint32_t* __restrict__ depth_bits,
                                                          int32_t* __restrict__ radii)
 {
     // staging area for the 16-coefficient SH blocks of each wavefront's 64 Gaussians
@@ -98,6 +100,7 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
     // ---- geometry: cull, covariance, EWA projection, conic, radius, tile rectangle ----
     int radius = 0;
     uint32_t touched = 0;
+    uint64_t rect_packed = 0;  // x0 | y0 << 16 | x1 << 32 | y1 << 48, zero when culled
     float x = 0.f, y = 0.f, z = 0.f, vz = 0.f, px = 0.f, py = 0.f, ca = 0.f, cc = 0.f, qx = 0.f, qy = 0.f, qz = 0.f;
     if (valid) do {
         x = g.means3D[3 * (size_t)i];
@@ -163,6 +166,7 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
 
         radius = rad;
         touched = (uint32_t)area;
+        rect_packed = (uint64_t)q.x0 | ((uint64_t)q.y0 << 16) | ((uint64_t)q.x1 << 32) | ((uint64_t)q.y1 << 48);
         qx = cc * det_inv;
         qy = -cb * det_inv;
         qz = ca * det_inv;
@@ -170,7 +174,10 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
 
     if (valid) radii[i] = radius;
     if (kRadiiOnly) return;
-    if (valid) tiles_touched[i] = touched;
+    if (valid) {
+        tiles_touched[i] = touched;
+        rects[i] = rect_packed;
+    }
     const bool alive = radius > 0;
 
     // ---- colour ----
@@ -235,6 +242,7 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
     rec[0] = make_float4(px, py, qx, qy);
     rec[1] = make_float4(qz, opacity, rgb[0], rgb[1]);
     rec[2] = make_float4(rgb[2], vz, ex, ey);
+    depth_bits[i] = __float_as_uint(vz);
 }
 
 // One workgroup expands the keys of 256 consecutive Gaussians.  Output slots
@@ -294,14 +302,16 @@ __global__ __launch_bounds__(256) void duplicate_kernel(FrameArgs f, int32_t P, 
 }  // namespace
 
 int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_only, float* records,
-                      uint32_t* tiles_touched, int32_t* radii, hipStream_t s)
+                      uint32_t* tiles_touched, uint64_t* rects, uint32_t* depth_bits, int32_t* radii, hipStream_t s)
 {
     if (g.P == 0) return GS355_OK;
     const dim3 block(256), grid((g.P + 255) / 256);
     if (radii_only)
-        hipLaunchKernelGGL(preprocess_kernel<true>, grid, block, 0, s, f, g, records, tiles_touched, radii);
+        hipLaunchKernelGGL(preprocess_kernel<true>, grid, block, 0, s, f, g, records, tiles_touched, rects, depth_bits,
+                           radii);
     else
-        hipLaunchKernelGGL(preprocess_kernel<false>, grid, block, 0, s, f, g, records, tiles_touched, radii);
+        hipLaunchKernelGGL(preprocess_kernel<false>, grid, block, 0, s, f, g, records, tiles_touched, rects, depth_bits,
+                           radii);
     GS355_CHECK_LAUNCH("preprocess");
     return GS355_OK;
 }

@@ -32,18 +32,18 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(_lib.Frame) == 7 * 4 + 4 + 4 * 8  # 7 scalars, padding to 8, 4 pointers
     assert C.sizeof(_lib.Gaussians) == 8 + 7 * 8
     assert C.sizeof(_lib.Outputs) == 4 * 8
-    assert C.sizeof(_lib.Layout) == 16 * 8 + 4 * 4
+    assert C.sizeof(_lib.Layout) == 18 * 8 + 4 * 4
 
 
 def test_workspace_layout_is_aligned_ordered_and_sized():
     P, n_cap, W, H = 100_000, 1_500_000, 1920, 1080
     L = _lib.workspace_layout(P, n_cap, W, H)
-    offs = [L.header, L.records, L.tiles_touched, L.offsets, L.scan_tmp, L.keys[0], L.keys[1], L.values[0],
+    offs = [L.header, L.records, L.tiles_touched, L.rects, L.depth_bits, L.offsets, L.scan_tmp, L.keys[0], L.keys[1], L.values[0],
             L.values[1], L.sort_hist, L.ranges, L.bin_matrix, L.tile_base, L.bin_visible, L.tile_lists, L.total_bytes]
     assert all(o % 256 == 0 for o in offs)
     assert offs == sorted(offs) and len(set(offs)) == len(offs)
     assert L.records - L.header >= 64
-    assert L.tiles_touched - L.records >= P * 48
+    assert L.tiles_touched - L.records >= P * 48 and L.depth_bits - L.rects >= P * 8
     assert L.keys[1] - L.keys[0] >= n_cap * 8
     assert L.values[1] - L.values[0] >= n_cap * 4
     tiles = 120 * 68

@@ -137,9 +137,23 @@ def config3(P: int = 6_000_000, width: int = 1920, height: int = 1080) -> Gaussi
     return GaussianScene("C3", means, scales, rots, opac, shs, 3, [cam])
 
 
-def aerial_poses(n: int, width: int, height: int, g: torch.Generator, target_half: float = 150.0) -> List[Camera]:
+def frustum_fraction(cam: Camera, points: torch.Tensor) -> float:
+    """Fraction of `points` whose centre lies inside the camera frustum (z_view > 0.2, |ndc| < 1)."""
+    hom = torch.cat([points, torch.ones(points.shape[0], 1)], dim=1)
+    view_z = (hom @ cam.world_view_transform)[:, 2]
+    clip = hom @ cam.full_proj_transform
+    ndc = clip[:, :2] / (clip[:, 3:4] + 1e-7)
+    inside = (view_z > 0.2) & (ndc.abs() < 1.0).all(dim=1)
+    return float(inside.float().mean())
+
+
+def aerial_poses(n: int, width: int, height: int, g: torch.Generator, target_half: float = 150.0,
+                 points: Optional[torch.Tensor] = None, keep=(0.22, 0.58)) -> List[Camera]:
+    """Random aerial poses: altitude U[100,300], pitch U[30,60] deg, yaw U[0,360), look-at target on the ground.
+    With `points`, candidates are drawn (deterministically, from the same generator) until the fraction of
+    points inside the frustum falls in `keep`, so that 20-60 % of the scene survives culling in every frame."""
     cams = []
-    for _ in range(n):
+    while len(cams) < n:
         r = torch.rand(5, generator=g).tolist()
         alt = 100.0 + 200.0 * r[0]
         pitch = math.radians(30.0 + 30.0 * r[1])
@@ -147,7 +161,10 @@ def aerial_poses(n: int, width: int, height: int, g: torch.Generator, target_hal
         tx, ty = (2 * r[3] - 1) * target_half, (2 * r[4] - 1) * target_half
         ground = alt / math.tan(pitch)
         eye = [tx - ground * math.cos(yaw), ty - ground * math.sin(yaw), alt]
-        cams.append(Camera.look_at(eye, [tx, ty, 0.0], [0.0, 0.0, 1.0], width, height, math.radians(60.0)))
+        cam = Camera.look_at(eye, [tx, ty, 0.0], [0.0, 0.0, 1.0], width, height, math.radians(60.0))
+        if points is not None and not keep[0] <= frustum_fraction(cam, points) <= keep[1]:
+            continue
+        cams.append(cam)
     return cams
 
 
@@ -158,7 +175,7 @@ def config4(P: int = 20_000_000, width: int = 3840, height: int = 2160, n_poses:
     rots = _unit_quats(P, g)
     opac = torch.sigmoid(torch.randn(P, 1, generator=g) * 1.5 + 0.5)
     shs = _shs(P, 3, g)
-    cams = aerial_poses(n_poses, width, height, g)
+    cams = aerial_poses(n_poses, width, height, g, points=means[: min(P, 100_000)])
     return GaussianScene("C4", means, scales, rots, opac, shs, 3, cams)
 
 

@@ -267,7 +267,7 @@ def timed_baseline(scene, blend_budget_s: float = 12.0):
         lens = (ranges[:, 1] - ranges[:, 0]).double()
         total_len = float(lens.sum())
         # probe a few tiles to size the sample
-        stride = 64
+        stride = 8
         sample_len, t_blend, done_tiles = 0.0, 0.0, 0
         tb0 = time.perf_counter()
         for t in range(0, gx * gy, stride):

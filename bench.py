@@ -236,6 +236,25 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     fps = args.steps / elapsed
 
+    # model-level frame rate: the reference's forward sequence (visibility prefilter, gather of the survivors,
+    # rasterize) and the fused single-pass variant that produces the same frame
+    from landmarksystem_amd.models import GaussianModel
+    model_fps = {}
+    for name, fuse in (("reference_sequence", False), ("fused_prefilter", True)):
+        model = GaussianModel(d.means3D, d.shs[:, :1].contiguous(), d.shs[:, 1:].contiguous(), torch.log(d.scales),
+                              d.rotations, torch.logit(d.opacities.clamp(1e-6, 1 - 1e-6)), sh_degree=scene.sh_degree,
+                              act_cache=True, fuse_prefilter=fuse).eval()
+        for _ in range(5):
+            model(scene.camera)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n_model = max(10, args.steps // 4)
+        for _ in range(n_model):
+            model(scene.camera)
+        torch.cuda.synchronize()
+        model_fps[name] = round(n_model / (time.perf_counter() - t0), 2)
+        del model
+
     if args.calibration_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
         dst = torch.empty_like(src)
@@ -315,6 +334,7 @@ def main():
                    "visible": V, "keys": N, "tiles": tiles, "scene_gen_s": round(gen_s, 1)},
         "roofline": roofline,
         "stages": stages,
+        "model_forward_frames_per_s": model_fps,
     }
     if not args.no_cpu_baseline:
         try:

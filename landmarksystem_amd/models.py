@@ -49,8 +49,13 @@ class GaussianModel(nn.Module):
 
     def __init__(self, xyz, features_dc, features_rest, scaling, rotation, opacity, sh_degree: int = 3,
                  white_bkgd: bool = False, act_cache: bool = False, compute_cov3D_python: bool = False,
-                 convert_SHs_python: bool = False):
+                 convert_SHs_python: bool = False, fuse_prefilter: bool = False):
         super().__init__()
+        # fuse_prefilter: render all Gaussians in one pass instead of "visibility prefilter, gather the survivors,
+        # render them".  The prefilter applies the same cull / radius / tile-rectangle tests as the rasterizer's own
+        # preprocess with the same camera, and a boolean-mask gather keeps relative order, so image, visibility_filter
+        # and radii come out identical; the second per-Gaussian pass and the 236 B/Gaussian gathers disappear.
+        self.fuse_prefilter = fuse_prefilter
         self._xyz = nn.Parameter(xyz, requires_grad=False)  # [P,3]
         self._features_dc = nn.Parameter(features_dc, requires_grad=False)  # [P,1,3]
         self._features_rest = nn.Parameter(features_rest, requires_grad=False)  # [P,(deg+1)^2-1,3]
@@ -127,9 +132,12 @@ class GaussianModel(nn.Module):
     @torch.no_grad()
     def forward(self, viewpoint_camera, scaling_modifier=1.0, override_color=None, render_exclude_filter=None):
         viewpoint_camera = viewpoint_camera.to(self._xyz.device)
-        voxel_visible_mask = self.prefilter_voxel(viewpoint_camera)
-        if render_exclude_filter is not None:
-            voxel_visible_mask = voxel_visible_mask & render_exclude_filter
+        fused = (self.fuse_prefilter and not self.training and render_exclude_filter is None
+                 and scaling_modifier == 1.0)  # the reference's prefilter always uses scale modifier 1
+        if not fused:
+            voxel_visible_mask = self.prefilter_voxel(viewpoint_camera)
+            if render_exclude_filter is not None:
+                voxel_visible_mask = voxel_visible_mask & render_exclude_filter
         self.renderer.raster_settings = _settings(viewpoint_camera, self.background, scaling_modifier,
                                                   self.active_sh_degree)
         means3D, opacity = self.get_xyz, self.get_opacity
@@ -144,6 +152,13 @@ class GaussianModel(nn.Module):
             raise NotImplementedError("convert_SHs_python: SH -> RGB runs inside the preprocess kernel")
         else:
             shs = self.get_features
+        if fused:
+            rendered_image, radii, _ = self.renderer(
+                means3D=means3D, means2D=None, shs=shs, colors_precomp=colors_precomp, opacities=opacity,
+                scales=scales, rotations=rotations, cov3D_precomp=cov3D_precomp)
+            self.visibility_filter = radii > 0
+            self.radii = radii[self.visibility_filter]
+            return rendered_image
         if not self.training:  # the reference renders only what its prefilter kept (origin_gs/gs_model.py:199-208)
             mask = voxel_visible_mask.nonzero().squeeze(-1)
             pick = lambda t: None if t is None else t[mask]  # noqa: E731

@@ -106,3 +106,20 @@ def test_octree_lod_mask_and_forward(gpu_device):
     assert torch.equal(image, image2)
     model.enable_lod = False
     assert torch.equal(model(cam), scaffold(cam))
+
+
+def test_fused_prefilter_gives_the_same_frame(gpu_device):
+    scene = scenes.config3(P=200_000, width=960, height=540)
+    args = (scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs)
+    plain = GaussianModel.from_activated(*args, sh_degree=3, act_cache=True).to(gpu_device).eval()
+    fused = GaussianModel.from_activated(*args, sh_degree=3, act_cache=True, fuse_prefilter=True).to(gpu_device).eval()
+    a, b = plain(scene.camera), fused(scene.camera)
+    assert torch.equal(a, b)
+    assert torch.equal(plain.visibility_filter, fused.visibility_filter)
+    assert torch.equal(plain.radii, fused.radii)
+    assert 0 < int(fused.visibility_filter.sum()) < scene.P
+    # a render_exclude_filter or a scale modifier falls back to the reference's two-pass sequence
+    keep = torch.ones(scene.P, dtype=torch.bool, device=gpu_device)
+    keep[::2] = False
+    assert torch.equal(plain(scene.camera, render_exclude_filter=keep), fused(scene.camera, render_exclude_filter=keep))
+    assert torch.equal(plain(scene.camera, scaling_modifier=0.7), fused(scene.camera, scaling_modifier=0.7))

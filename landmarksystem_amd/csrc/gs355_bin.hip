@@ -401,13 +401,13 @@ template <int kT, int kR>
 struct LdsSorter {
     static constexpr int kW = kT / 64;
     static constexpr int kCap = kT * kR;
-    static constexpr size_t kBytes = (size_t)kCap * 12 + (size_t)kW * 256 * 4 + 64;
+    static constexpr size_t kBytes = (size_t)kCap * 12 + (size_t)kW * 256 * 4 + 192;
 
     uint32_t* depth;     // [kCap]
     uint32_t* index;     // [kCap]
     uint16_t* perm0;     // two permutations of [kCap] each, back to back
     uint32_t (*cnt)[256];  // [kW][256]
-    uint32_t* flags;     // [16]
+    uint32_t* flags;     // [48]
 
     __device__ explicit LdsSorter(uint32_t* lds)
     {
@@ -543,26 +543,174 @@ struct LdsSorter {
         return cur;
     }
 
+    // Fast path: one counting pass over a monotone map of the depth onto kT bins leaves a handful of pairs per
+    // bin; every pair then ranks itself among the members of its bin by (depth bits, index).  Bins are ordered and
+    // each bin is fully ordered, so the result is the exact total order whatever order the LDS atomics ran in.
+    // Depths along the rays of a tile cluster (most splats sit near the ground), so the map is adaptive: a
+    // 256-bin histogram over [dmin, dmax] gives a piecewise-linear estimate of each pair's final position, and
+    // the bin is that position scaled to kT.  Returns the buffer holding the order, or -2 when some bin is still
+    // too full for this to pay: the caller then runs the radix passes.
+    static constexpr uint32_t kMaxBin = 256;
+
+    __device__ int bucket_sort(uint32_t n, uint32_t dmin, uint32_t dmax) const
+    {
+        const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+        uint32_t* const count = &cnt[0][0];  // [kT] pairs per bin, then the bin's first slot
+        uint32_t* const coarse = count + kT;  // [256] pairs per coarse bin, then their exclusive prefix
+        const uint32_t range = dmax - dmin;
+        if (range == 0) return -2;
+        // coarse(d) = floor((d - dmin) * 256 / (range + 1)) as the high word of a 32x32 multiply, whose low word is
+        // the position inside the coarse bin as a 0.32 fraction; a range below 256 gives every depth its own bin
+        const bool direct = range < 256u;
+        const uint32_t mult = direct ? 0u : (uint32_t)((256ull << 32) / ((uint64_t)range + 1ull));
+        // position -> bin: floor(pos * kT / n) for n > kT, else the position itself (one pair per bin)
+        const bool spread = n > (uint32_t)kT;
+        const uint32_t to_bin = spread ? (uint32_t)(((uint64_t)kT << 32) / (uint64_t)n) : 0u;
+        count[tid] = 0;
+        if (tid < 256) coarse[tid] = 0;
+        if (tid == 0) flags[8] = 0;
+        __syncthreads();
+        uint32_t cbin[kR], frac[kR];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t j = (uint32_t)r * kT + tid;
+            cbin[r] = 0;
+            frac[r] = 0;
+            if (j < n) {
+                const uint32_t rel = depth[j] - dmin;
+                const uint64_t wide = (uint64_t)rel * mult;
+                cbin[r] = direct ? rel : (uint32_t)(wide >> 32);
+                frac[r] = direct ? 0u : (uint32_t)wide;
+                atomicAdd(&coarse[cbin[r]], 1u);
+            }
+        }
+        __syncthreads();
+        uint32_t csize = 0;
+        if (tid < 256) {  // exclusive scan of the coarse counts (wavefronts 0..3)
+            csize = coarse[tid];
+            uint32_t inc = csize;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t up = __shfl_up(inc, d, 64);
+                if (lane >= d) inc += up;
+            }
+            if (lane == 63) flags[16 + wave] = inc;
+            csize = inc - csize;  // exclusive within the wavefront
+        }
+        __syncthreads();
+        if (tid < 256) {
+            for (int w = 0; w < wave; ++w) csize += flags[16 + w];
+        }
+        __syncthreads();
+        uint32_t my_size = 0;
+        if (tid < 256) {
+            my_size = coarse[tid];  // read the count before it is replaced by the prefix
+        }
+        __syncthreads();
+        if (tid < 256) {
+            coarse[tid] = csize;
+            coarse[256 + tid] = my_size;
+        }
+        __syncthreads();
+        uint32_t bin[kR], slot[kR];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t j = (uint32_t)r * kT + tid;
+            bin[r] = 0;
+            slot[r] = 0;
+            if (j < n) {
+                const uint32_t pos = coarse[cbin[r]] + __umulhi(frac[r], coarse[256 + cbin[r]]);  // in [0, n)
+                bin[r] = min(spread ? __umulhi(pos, to_bin) : pos, (uint32_t)kT - 1u);
+                slot[r] = atomicAdd(&count[bin[r]], 1u);
+            }
+        }
+        __syncthreads();
+        // exclusive scan of the kT bin counts; remember whether any bin is over-full
+        const uint32_t c = count[tid];
+        uint32_t inc = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(inc, d, 64);
+            if (lane >= d) inc += up;
+        }
+        if (lane == 63) flags[16 + wave] = inc;
+        if (c > kMaxBin) flags[8] = 1;
+        __syncthreads();
+        if (flags[8] != 0) {
+            __syncthreads();
+            return -2;
+        }
+        uint32_t first = inc - c;
+        for (int w = 0; w < wave; ++w) first += flags[16 + w];
+        count[tid] = first;
+        __syncthreads();
+        uint16_t* const P = perm(0);
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t j = (uint32_t)r * kT + tid;
+            if (j < n) P[count[bin[r]] + slot[r]] = (uint16_t)j;
+        }
+        __syncthreads();
+        // every pair ranks itself among the members of its bin (independent reads, evenly spread over the
+        // threads whatever the bin sizes are) and takes the slot of that rank
+        uint16_t* const Q = perm(1);
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t j = (uint32_t)r * kT + tid;
+            if (j < n) {
+                const uint32_t b = bin[r];
+                const uint32_t lo_slot = count[b];
+                const uint32_t hi_slot = b + 1 < (uint32_t)kT ? count[b + 1] : n;
+                const uint32_t md = depth[j], mi = index[j];
+                uint32_t rank = 0;
+                for (uint32_t q = lo_slot; q < hi_slot; ++q) {
+                    const uint32_t e = P[q];
+                    const uint32_t ed = depth[e], ei = index[e];
+                    rank += (ed < md || (ed == md && ei < mi)) ? 1u : 0u;
+                }
+                Q[lo_slot + rank] = (uint16_t)j;
+            }
+        }
+        __syncthreads();
+        return 1;
+    }
+
     __device__ void run(uint32_t tile, const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ buckets,
                         uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals) const
     {
         const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
         if (n == 0 || n > (uint32_t)kCap) return;  // uniform over the workgroup
-        if (threadIdx.x == 0) flags[11] = 0;
+        if (threadIdx.x == 0) {
+            flags[11] = 0;
+            flags[12] = 0xFFFFFFFFu;
+            flags[13] = 0;
+        }
         __syncthreads();
         const uint32_t d0 = (uint32_t)(buckets[lo] >> 32);
-        uint32_t diff = 0;
+        uint32_t diff = 0, dmin = 0xFFFFFFFFu, dmax = 0;
         for (uint32_t j = threadIdx.x; j < n; j += kT) {
             const uint64_t v = buckets[lo + j];
-            depth[j] = (uint32_t)(v >> 32);
+            const uint32_t dj = (uint32_t)(v >> 32);
+            depth[j] = dj;
             index[j] = (uint32_t)v;
-            diff |= depth[j] ^ d0;
+            diff |= dj ^ d0;
+            dmin = min(dmin, dj);
+            dmax = max(dmax, dj);
         }
 #pragma unroll
-        for (int d = 32; d > 0; d >>= 1) diff |= __shfl_xor(diff, d, 64);
-        if ((threadIdx.x & 63) == 0 && diff) atomicOr(&flags[11], diff);
+        for (int d = 32; d > 0; d >>= 1) {
+            diff |= __shfl_xor(diff, d, 64);
+            dmin = min(dmin, (uint32_t)__shfl_xor(dmin, d, 64));
+            dmax = max(dmax, (uint32_t)__shfl_xor(dmax, d, 64));
+        }
+        if ((threadIdx.x & 63) == 0) {
+            if (diff) atomicOr(&flags[11], diff);
+            atomicMin(&flags[12], dmin);
+            atomicMax(&flags[13], dmax);
+        }
         __syncthreads();
-        const int cur = sort(n, flags[11]);
+        int cur = bucket_sort(n, flags[12], flags[13]);
+        if (cur == -2) cur = sort(n, flags[11]);
         for (uint32_t j = threadIdx.x; j < n; j += kT) {
             const uint32_t e = cur < 0 ? j : (uint32_t)perm(cur)[j];
             out_keys[lo + j] = ((uint64_t)tile << 32) | (uint64_t)depth[e];

@@ -351,3 +351,25 @@ def test_full_size_headline_frame_properties(gpu_device):
     for name in ("sorted_keys", "sorted_values", "ranges", "image", "depth", "alpha"):
         np.testing.assert_array_equal(got[name], again[name], err_msg=name)
     assert got["alpha"].min() >= 0.0 and got["alpha"].max() <= 1.0 and np.isfinite(got["image"]).all()
+
+
+@pytest.mark.parametrize("same,spread,label", [(1800, 0, "one depth only"), (1500, 2500, "one heavy depth among many"),
+                                                (300, 6000, "heavy depth in a class-3 bucket")])
+def test_tile_sort_fallback_on_massive_depth_ties(gpu_device, same, spread, label):
+    """Hundreds of Gaussians with identical depth bits in one tile overfill a counting bin: the sorter must fall
+    back to its radix passes and still deliver ascending index order inside the tie."""
+    P = same + spread
+    scene = scenes.config1(P=P, width=32, height=32)
+    g = torch.Generator().manual_seed(P)
+    scene.means3D[:, :2] = (torch.rand(P, 2, generator=g) - 0.5) * 0.05
+    scene.means3D[:same, 2] = 0.25  # identity camera rotation: view depth = z + 3, identical bits
+    scene.scales[:] = 0.35
+    scene.opacities[:] = 0.01
+    got = run_fast_path(scene, gpu_device)
+    ref = oracle_render(scene)
+    np.testing.assert_array_equal(got["ranges"], ref["ranges"])
+    np.testing.assert_array_equal(got["sorted_keys"], ref["sorted_keys"])
+    np.testing.assert_array_equal(got["sorted_values"], ref["sorted_values"])
+    k = got["sorted_keys"]
+    run_lengths = np.diff(np.flatnonzero(np.concatenate([[True], k[1:] != k[:-1], [True]])))
+    assert run_lengths.max() >= same, label

@@ -71,35 +71,52 @@ __device__ __forceinline__ half4_t weight_fragment(const float* __restrict__ w, 
     return to_half4(v[0], v[1], v[2], v[3]);
 }
 
-// Bias for an accumulator: register v = 4b + t holds row 8b + 4*half + t.
-__device__ __forceinline__ floatx16 bias_rows(const float* __restrict__ bias, int rows, int row0, int half)
+// Bias for an accumulator: register v = 4b + t holds row 8b + 4*half + t.  `bias` is the head's bias vector
+// staged in LDS, zero-padded to a multiple of 32 rows.
+__device__ __forceinline__ floatx16 bias_rows(const float* bias, int row0, int half)
 {
     floatx16 c;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int r = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
-        c[v] = r < rows ? bias[r] : 0.0f;
-    }
+    for (int v = 0; v < 16; ++v) c[v] = bias[row0 + 8 * (v >> 2) + 4 * half + (v & 3)];
     return c;
 }
 
-// One head for one tile of 32 anchors: returns up to kTiles accumulators of the
-// second layer (rows = outputs 32r + 8b + 4*half + t, column = this lane's anchor).
+// Weight fragments of one head, held in registers for the whole kernel.
 template <int kTiles>
-__device__ __forceinline__ void run_head(const DecodeArgs& d, int head, int outputs, const half4_t X[5], int row,
-                                         int half, floatx16 out[kTiles])
+struct HeadWeights {
+    half4_t w0[5];          // layer 1: [32 x in], k-steps 0..4
+    half4_t w1[kTiles][4];  // layer 2: [outputs x 32] in row tiles of 32
+};
+
+template <int kTiles>
+__device__ __forceinline__ void load_head(const DecodeArgs& d, int head, int outputs, int row, int half,
+                                          HeadWeights<kTiles>& w)
 {
-    // layer 1: hidden = W0 [32 x in] * X^T + b0
-    floatx16 h = bias_rows(d.b0[head], kFeat, 0, half);
     const int in = d.in_dim[head];
 #pragma unroll
     for (int s = 0; s < 5; ++s) {
         // k-step 4 carries the fp32-only inputs twice: hi parts on the low half of the lanes, lo parts on the
         // high half, both against the same weights W0[:, 32..35]
         const int k0 = s < 4 ? 8 * s + 4 * half : 32;
-        const half4_t a = weight_fragment(d.w0[head], kFeat, in, row, k0);
-        h = __builtin_amdgcn_mfma_f32_32x32x8f16(a, X[s], h, 0, 0, 0);
+        w.w0[s] = weight_fragment(d.w0[head], kFeat, in, row, k0);
     }
+#pragma unroll
+    for (int r = 0; r < kTiles; ++r)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+            w.w1[r][s] = weight_fragment(d.w1[head], outputs, kFeat, 32 * r + row, 8 * s + 4 * half);
+}
+
+// One head for one tile of 32 anchors: returns up to kTiles accumulators of the
+// second layer (rows = outputs 32r + 8b + 4*half + t, column = this lane's anchor).
+template <int kTiles>
+__device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const float* bias0, const float* bias1,
+                                         const half4_t X[5], int half, floatx16 out[kTiles])
+{
+    // layer 1: hidden = W0 [32 x in] * X^T + b0
+    floatx16 h = bias_rows(bias0, 0, half);
+#pragma unroll
+    for (int s = 0; s < 5; ++s) h = __builtin_amdgcn_mfma_f32_32x32x8f16(w.w0[s], X[s], h, 0, 0, 0);
     // ReLU, then hi/lo split: registers 4s..4s+3 are the B operand of k-step s
     half4_t hh[4], hl[4];
 #pragma unroll
@@ -117,12 +134,11 @@ __device__ __forceinline__ void run_head(const DecodeArgs& d, int head, int outp
     // layer 2: out = W1 [outputs x 32] * hidden + b1
 #pragma unroll
     for (int r = 0; r < kTiles; ++r) {
-        floatx16 c = bias_rows(d.b1[head], outputs, 32 * r, half);
+        floatx16 c = bias_rows(bias1, 32 * r, half);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const half4_t a = weight_fragment(d.w1[head], outputs, kFeat, 32 * r + row, 8 * s + 4 * half);
-            c = __builtin_amdgcn_mfma_f32_32x32x8f16(a, hh[s], c, 0, 0, 0);
-            c = __builtin_amdgcn_mfma_f32_32x32x8f16(a, hl[s], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x8f16(w.w1[r][s], hh[s], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x8f16(w.w1[r][s], hl[s], c, 0, 0, 0);
         }
         out[r] = c;
     }
@@ -150,8 +166,29 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
     constexpr int kStrideMax = kCountOnly ? 11 : 113;
     __shared__ float s_out[4][32 * kStrideMax];
 
+    // biases of the three heads, zero-padded: b0 at [head*32], b1 of opacity / cov / colour at 96 / 128 / 224
+    __shared__ float s_bias[256];
+
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
     const int n = d.n;
+    {
+        const int t = threadIdx.x;
+        float v = 0.0f;
+        if (t < 96) v = d.b0[t >> 5][t & 31];
+        else if (t < 128) v = (t - 96) < n ? d.b1[0][t - 96] : 0.0f;
+        else if (t < 224) v = (t - 128) < 7 * n ? d.b1[1][t - 128] : 0.0f;
+        else v = (t - 224) < 3 * n ? d.b1[2][t - 224] : 0.0f;
+        s_bias[t] = v;
+    }
+    __syncthreads();
+    HeadWeights<1> w_op;
+    load_head<1>(d, 0, n, col, half, w_op);
+    HeadWeights<3> w_cov;
+    HeadWeights<1> w_col;
+    if (!kCountOnly) {
+        load_head<3>(d, 1, 7 * n, col, half, w_cov);
+        load_head<1>(d, 2, 3 * n, col, half, w_col);
+    }
     const int stride = kCountOnly ? 11 : 11 * n + 3;
     const int tiles = (d.A + 31) / 32;
     float* __restrict__ mine = s_out[wave];
@@ -198,9 +235,9 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
 
         // ---- opacity head ----
         floatx16 op[1];
-        run_head<1>(d, 0, n, X, col, half, op);
-#pragma unroll
-        for (int v = 0; v < 16; ++v) op[0][v] = tanhf(op[0][v]);
+        run_head<1>(w_op, s_bias, s_bias + 96, X, half, op);
+        // the mask opacity > 0 is the sign of the pre-activation (tanh is odd, monotone and tanh(x) = x for the
+        // smallest floats), so tanh itself is only evaluated for the offsets that are kept
         store_rows(mine + col * stride, 0, n, 0, half, op[0]);
         if (kCountOnly) {
             __builtin_amdgcn_wave_barrier();
@@ -216,11 +253,11 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
 
         // ---- covariance and colour heads ----
         floatx16 cv[3];
-        run_head<3>(d, 1, 7 * n, X, col, half, cv);
+        run_head<3>(w_cov, s_bias + 32, s_bias + 128, X, half, cv);
 #pragma unroll
         for (int r = 0; r < 3; ++r) store_rows(mine + col * stride, n, 7 * n, 32 * r, half, cv[r]);
         floatx16 cl[1];
-        run_head<1>(d, 2, 3 * n, X, col, half, cl);
+        run_head<1>(w_col, s_bias + 64, s_bias + 224, X, half, cl);
         store_rows(mine + col * stride, 8 * n, 3 * n, 0, half, cl[0]);
         __builtin_amdgcn_wave_barrier();
 
@@ -231,8 +268,8 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
             const int ga = tile * 32 + al;
             if (ga >= d.A || d.visible[ga] == 0) continue;
             const float* __restrict__ o = mine + al * stride;
-            const float opac = o[m];
-            if (!(opac > 0.0f)) continue;
+            if (!(o[m] > 0.0f)) continue;
+            const float opac = tanhf(o[m]);
             uint32_t rank = 0;
             for (int mm = 0; mm < m; ++mm) rank += o[mm] > 0.0f ? 1u : 0u;
             const uint32_t pos = offsets[ga] + rank;

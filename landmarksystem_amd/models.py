@@ -13,7 +13,8 @@ They keep the reference's call sequence (visibility prefilter -> optional
 anchor decode -> settings record re-assigned on the renderer -> rasterize),
 its eval-mode gather of the visible Gaussians and its `act_cache` behaviour,
 and its parameter names so checkpoints map one to one.  Forward / eval only:
-training, densification and checkpoint I/O are not part of this package.
+training and densification are not part of this package; checkpoint I/O lives
+in `checkpoints.py`.
 Activations and gathers are a handful of torch elementwise calls, as in the
 reference; everything per-Gaussian and per-pixel runs in the HIP library.
 """
@@ -37,6 +38,24 @@ def _settings(camera, bg, scaling_modifier, sh_degree):
     )
 
 
+def _cfg(config, name, default):
+    """Field `name` of a config object (attribute- or key-addressable), else `default`."""
+    if isinstance(config, dict):
+        return config.get(name, default)
+    return getattr(config, name, default)
+
+
+def _split_prefix(state_dict, prefix):
+    """Pop the entries under `prefix` (base_model.py:363-368)."""
+    picked = {}
+    for key in list(state_dict.keys()):
+        if key.startswith(prefix):
+            picked[key[len(prefix):]] = state_dict.pop(key)
+    if not picked:
+        print("WRANING: could not found any key start with %s in provided state_dict" % prefix)
+    return picked
+
+
 def _placeholder_renderer(bg):
     # the reference builds its renderer once with empty placeholders (origin_gs/gs_model.py:82-97)
     return GaussianRasterizer(raster_settings=GaussianRasterizationSettings(
@@ -47,10 +66,24 @@ def _placeholder_renderer(bg):
 class GaussianModel(nn.Module):
     """Vanilla 3DGS: raw parameters with exp / sigmoid / normalize activations."""
 
-    def __init__(self, xyz, features_dc, features_rest, scaling, rotation, opacity, sh_degree: int = 3,
-                 white_bkgd: bool = False, act_cache: bool = False, compute_cov3D_python: bool = False,
-                 convert_SHs_python: bool = False, fuse_prefilter: bool = False):
+    def __init__(self, xyz=None, features_dc=None, features_rest=None, scaling=None, rotation=None, opacity=None,
+                 sh_degree: int = 3, white_bkgd: bool = False, act_cache: bool = False,
+                 compute_cov3D_python: bool = False, convert_SHs_python: bool = False, fuse_prefilter: bool = False,
+                 config=None, scene_manager=None):
         super().__init__()
+        if xyz is not None and not torch.is_tensor(xyz):  # the reference's signature: (config, scene_manager)
+            config, xyz = xyz, None
+        if config is not None:  # empty model, filled by load_from_state_dict (origin_gs/gs_model.py:62-79)
+            sh_degree = _cfg(config, "sh_degree", sh_degree)
+            white_bkgd, act_cache = _cfg(config, "white_bkgd", white_bkgd), _cfg(config, "act_cache", act_cache)
+            compute_cov3D_python = _cfg(config, "compute_cov3D_python", compute_cov3D_python)
+            convert_SHs_python = _cfg(config, "convert_SHs_python", convert_SHs_python)
+            fuse_prefilter = _cfg(config, "fuse_prefilter", fuse_prefilter)
+        if xyz is None:
+            e = torch.empty
+            xyz, features_dc, features_rest = e(0, 3), e(0, 1, 3), e(0, (sh_degree + 1) ** 2 - 1, 3)
+            scaling, rotation, opacity = e(0, 3), e(0, 4), e(0, 1)
+        self.config, self.scene_manager = config, scene_manager
         # fuse_prefilter: render all Gaussians in one pass instead of "visibility prefilter, gather the survivors,
         # render them".  The prefilter applies the same cull / radius / tile-rectangle tests as the rasterizer's own
         # preprocess with the same camera, and a boolean-mask gather keeps relative order, so image, visibility_filter
@@ -77,6 +110,51 @@ class GaussianModel(nn.Module):
         op = opacities.clamp(eps, 1 - eps)
         return cls(means3D, shs[:, :1].contiguous(), shs[:, 1:].contiguous(), torch.log(scales), rotations,
                    torch.log(op / (1 - op)), **kw)
+
+    @classmethod
+    def from_cache(cls, xyz, features, scaling, rotation, opacity, **kw):
+        """Build from stored activated values (the `cache_*` checkpoint schema, gaussian_encoding.py:226-266):
+        the raw parameters stay empty and the getters serve the cache, so the model is eval-only."""
+        kw["act_cache"] = True
+        empty = lambda *shape: torch.empty(*shape, device=xyz.device)  # noqa: E731
+        m = cls(xyz, empty(0, 1, 3), empty(0, features.shape[1] - 1, 3), empty(0, 3), empty(0, 4), empty(0, 1), **kw)
+        m._cache = {"features": features, "scaling": scaling, "rotation": rotation, "opacity": opacity}
+        return m.eval()
+
+    def get_state_dict_from_ckpt(self, file_path, map_location="cpu"):
+        """PLY columns under `gaussian_encoding.` merged with `state_dict.th` (base_model.py:308-342)."""
+        from . import checkpoints
+        return checkpoints.merged_state_dict(file_path, "gaussian", map_location, max_sh_degree=self.max_sh_degree)
+
+    def load_from_state_dict(self, state_dict, strict: bool = True):
+        """base_model.py:344-372 + gaussian_encoding.py:273-338: raw parameters, or the activation cache."""
+        gs = _split_prefix(dict(state_dict), "gaussian_encoding.")
+        raw = ("_xyz", "_features_dc", "_features_rest", "_opacity", "_scaling", "_rotation")
+        cache = ("_xyz", "_cache_features", "_cache_opacity", "_cache_scaling", "_cache_rotation")
+        if "_opacity" in gs or "_features_dc" in gs:
+            found = set(gs) & set(raw)
+            if strict and len(found) != len(raw):
+                raise ValueError("only found keys %s in state dict" % (found,))
+            for name in found:
+                setattr(self, name, nn.Parameter(gs[name].detach().to(self._xyz.device).float().contiguous(),
+                                                 requires_grad=False))
+            self._cache = {}
+        elif set(gs) & set(cache[1:]):
+            found = set(gs) & set(cache)
+            if strict and len(found) != len(cache):
+                raise ValueError("only found keys %s in state dict" % (found,))
+            dev = self._xyz.device
+            self._xyz = nn.Parameter(gs["_xyz"].detach().to(dev).float().contiguous(), requires_grad=False)
+            self.act_cache = True
+            self._cache = {k[len("_cache_"):]: gs[k].detach().to(dev).float().contiguous() for k in found if k != "_xyz"}
+        elif strict:
+            raise ValueError("not found any param keys in state dict, state dict keys: %s" % (list(gs),))
+        self.active_sh_degree = self.max_sh_degree
+
+    def _apply(self, fn, *args, **kwargs):
+        out = super()._apply(fn, *args, **kwargs)  # .to()/.cuda(): the activation cache follows the parameters
+        self._cache = {k: fn(v) for k, v in self._cache.items()}
+        return out
 
     def _cached(self, name, fn):
         if self.act_cache and not self.training:
@@ -174,10 +252,34 @@ class GaussianModel(nn.Module):
 class ScaffoldGS(nn.Module):
     """Scaffold-GS: anchors decoded into neural Gaussians per frame."""
 
-    def __init__(self, anchor, anchor_feat, offset, scaling, rotation, n_offsets: int = 10, feat_dim: int = 32,
-                 add_opacity_dist: bool = True, add_cov_dist: bool = True, add_color_dist: bool = True,
-                 white_bkgd: bool = False, act_cache: bool = False):
+    _ckpt_kind = "scaffold"
+
+    def __init__(self, anchor=None, anchor_feat=None, offset=None, scaling=None, rotation=None, n_offsets: int = 10,
+                 feat_dim: int = 32, add_opacity_dist: bool = True, add_cov_dist: bool = True,
+                 add_color_dist: bool = True, white_bkgd: bool = False, act_cache: bool = False, opacity=None,
+                 config=None, scene_manager=None):
         super().__init__()
+        if anchor is not None and not torch.is_tensor(anchor):  # the reference's signature: (config, scene_manager)
+            config, anchor = anchor, None
+        if config is not None:  # empty model, filled by load_from_state_dict (scaffold_gs/gs_model.py:104-140)
+            n_offsets, feat_dim = _cfg(config, "n_offsets", n_offsets), _cfg(config, "feat_dim", feat_dim)
+            add_opacity_dist = _cfg(config, "add_opacity_dist", add_opacity_dist)
+            add_cov_dist = _cfg(config, "add_cov_dist", add_cov_dist)
+            add_color_dist = _cfg(config, "add_color_dist", add_color_dist)
+            white_bkgd, act_cache = _cfg(config, "white_bkgd", white_bkgd), _cfg(config, "act_cache", act_cache)
+            for name, allowed in (("use_feat_bank", False), ("appearance_dim", 0), ("add_level", False),
+                                  ("view_dim", 3)):
+                if _cfg(config, name, allowed) != allowed:
+                    raise NotImplementedError("%s=%r: the fused anchor decode supports %s=%r only"
+                                              % (name, _cfg(config, name, allowed), name, allowed))
+        if anchor is None:
+            e = torch.empty
+            anchor, anchor_feat, offset = e(0, 3), e(0, feat_dim), e(0, n_offsets, 3)
+            scaling, rotation = e(0, 6), e(0, 4)
+        self.config, self.scene_manager = config, scene_manager
+        # per-anchor opacity is carried by checkpoints but never read by the forward pass (scaffoldgs_encoding.py:88)
+        self._opacity = nn.Parameter(torch.zeros(anchor.shape[0], 1, device=anchor.device) if opacity is None
+                                     else opacity, requires_grad=False)  # [A,1] logit
         self._anchor = nn.Parameter(anchor, requires_grad=False)  # [A,3]
         self._anchor_feat = nn.Parameter(anchor_feat, requires_grad=False)  # [A,32]
         self._offset = nn.Parameter(offset, requires_grad=False)  # [A,n,3]
@@ -230,6 +332,39 @@ class ScaffoldGS(nn.Module):
     def get_rotation(self):
         return self._cached("rotation", lambda: torch.nn.functional.normalize(self._rotation))
 
+    def get_state_dict_from_ckpt(self, file_path, map_location="cpu"):
+        """PLY columns under `gaussian_encoding.` merged with `state_dict.th` (base_model.py:308-342)."""
+        from . import checkpoints
+        return checkpoints.merged_state_dict(file_path, self._ckpt_kind, map_location)
+
+    _encoding_keys = ("_anchor_feat", "_offset", "_anchor", "_opacity", "_scaling", "_rotation")
+
+    def load_from_state_dict(self, state_dict, strict: bool = True):
+        """base_model.py:344-372 + scaffoldgs_encoding.py:236-281; the rest (`anchor_decoder.*`) loads as an
+        ordinary module state dict."""
+        state_dict = dict(state_dict)
+        gs = _split_prefix(state_dict, "gaussian_encoding.")
+        found = set(gs) & set(self._encoding_keys)
+        if strict and len(found) != len(self._encoding_keys):
+            raise ValueError("only found keys %s in state dict" % (found,))
+        dev = self._anchor.device
+        for name in found:
+            value = gs[name].detach().to(dev)
+            if isinstance(getattr(self, name), nn.Parameter):
+                setattr(self, name, nn.Parameter(value.float().contiguous(), requires_grad=False))
+            else:
+                self._load_buffer(name, value)
+        self._cache = {}
+        decoder = _split_prefix(state_dict, "anchor_decoder.") if any(
+            k.startswith("anchor_decoder.") for k in state_dict) else {}
+        if decoder or strict:
+            self.anchor_decoder.load_state_dict(decoder, strict=strict)
+        if strict and state_dict:
+            raise ValueError("unexpected keys in state dict: %s" % (sorted(state_dict),))
+
+    def _load_buffer(self, name, value):
+        raise KeyError(name)
+
     def _anchor_subset(self):
         return None  # Scaffold-GS filters all anchors
 
@@ -272,9 +407,24 @@ class ScaffoldGS(nn.Module):
 class OctreeGS(ScaffoldGS):
     """Octree-GS: Scaffold-GS plus a per-frame level-of-detail mask over the anchors."""
 
-    def __init__(self, anchor, anchor_feat, offset, scaling, rotation, level, voxel_size: float, standard_dist: float,
-                 fork: int = 2, extra_level=None, enable_lod: bool = True, dist2level: str = "round", **kw):
-        super().__init__(anchor, anchor_feat, offset, scaling, rotation, **kw)
+    _ckpt_kind = "octree"
+    _encoding_keys = ScaffoldGS._encoding_keys + ("_level", "_extra_level")
+
+    def __init__(self, anchor=None, anchor_feat=None, offset=None, scaling=None, rotation=None, level=None,
+                 voxel_size: float = 0.0, standard_dist: float = 1.0, fork: int = 2, extra_level=None,
+                 enable_lod: bool = True, dist2level: str = "round", config=None, scene_manager=None, **kw):
+        if anchor is not None and not torch.is_tensor(anchor):  # the reference's signature: (config, scene_manager)
+            config, anchor = anchor, None
+        if config is not None:  # octree_gs/gs_model.py:139-177; Octree-GS defaults to no distance inputs (:44-46)
+            fork, dist2level = _cfg(config, "fork", fork), _cfg(config, "dist2level", dist2level)
+            enable_lod = _cfg(config, "enable_lod", enable_lod)
+            for name in ("add_opacity_dist", "add_cov_dist", "add_color_dist"):
+                kw.setdefault(name, _cfg(config, name, False))
+        super().__init__(anchor, anchor_feat, offset, scaling, rotation, config=config, scene_manager=scene_manager,
+                         **kw)
+        if level is None:
+            level = torch.zeros(self._anchor.shape[0])
+        anchor = self._anchor
         if dist2level not in ("floor", "round", "ceil"):
             raise NotImplementedError("dist2level=%r (the progressive mode is dead code from the reference's model, "
                                       "octree_gs/gs_model.py:247)" % dist2level)
@@ -302,6 +452,27 @@ class OctreeGS(ScaffoldGS):
             int_level = torch.ceil(pred_level).int()
         int_level = torch.clamp(int_level, min=0, max=int(cur_level.item()))
         self._anchor_mask = self._level.squeeze(dim=1) <= int_level
+
+    def get_state_dict_from_ckpt(self, file_path, map_location="cpu"):
+        """As Scaffold-GS; reading the PLY also sets `voxel_size` and `standard_dist` from its `info` column
+        (octreegs_encoding.py:323-324)."""
+        from . import checkpoints
+        _, self.voxel_size, self.standard_dist = checkpoints.octree_state_dict(file_path, "cpu")
+        return super().get_state_dict_from_ckpt(file_path, map_location)
+
+    def _load_buffer(self, name, value):
+        if name == "_level":
+            self._level = value.reshape(-1, 1).float()
+        elif name == "_extra_level":
+            self._extra_level = value.reshape(-1).float()
+        else:
+            raise KeyError(name)
+
+    def forward(self, viewpoint_camera, scaling_modifier=1.0, retain_grad=False, render_exclude_filter=None,
+                ape_code=-1):
+        # ape_code selects an appearance embedding in the reference (octree_gs/gs_model.py:254-260); without
+        # appearance inputs (appearance_dim = 0, all this decode supports) it has no effect
+        return super().forward(viewpoint_camera, scaling_modifier, retain_grad, render_exclude_filter)
 
     def _before_prefilter(self, viewpoint_camera):
         if not self.training:

@@ -1,0 +1,266 @@
+"""Checkpoint reader / writer against PLY files built here byte by byte.
+
+The files are assembled with `struct.pack` from the published PLY layout
+(ascii header, then rows of the declared scalars in declaration order), not
+with the package's own writer, and the expected tensors are spelled out from
+the reference's column conventions (gaussian_encoding.py:185-222,
+scaffoldgs_encoding.py:193-223, octreegs_encoding.py:321-353), so a transposed
+reshape, a mis-sorted numbered column (f_rest_10 before f_rest_2) or a wrong
+endianness fails here.
+"""
+import os
+import struct
+
+import numpy as np
+import pytest
+import torch
+
+from landmarksystem_amd import checkpoints as ck
+from landmarksystem_amd.models import GaussianModel, OctreeGS, ScaffoldGS
+
+_CODES = {"float": "f", "double": "d", "int": "i", "uchar": "B", "short": "h"}
+
+
+def _raw_ply(path, props, rows, fmt="binary_little_endian", extra_header=(), trailing_element=False):
+    head = ["ply", "format %s 1.0" % fmt, "comment written by the test"]
+    head += list(extra_header)
+    head.append("element vertex %d" % len(rows))
+    head += ["property %s %s" % (t, n) for n, t in props]
+    if trailing_element:
+        head += ["element face 1", "property list uchar int vertex_indices"]
+    head.append("end_header")
+    with open(path, "wb") as fh:
+        fh.write(("\n".join(head) + "\n").encode())
+        for row in rows:
+            if fmt == "ascii":
+                fh.write((" ".join(repr(float(x)) if t in ("float", "double") else str(int(x))
+                                   for x, (_, t) in zip(row, props)) + "\n").encode())
+            else:
+                order = "<" if fmt == "binary_little_endian" else ">"
+                for x, (_, t) in zip(row, props):
+                    fh.write(struct.pack(order + _CODES[t], x if t in ("float", "double") else int(x)))
+        if trailing_element:
+            fh.write(b"3 0 1 2\n" if fmt == "ascii" else struct.pack("<Biii", 3, 0, 1, 2))
+
+
+def _vanilla_props(deg, shuffled=False):
+    k = (deg + 1) ** 2 - 1
+    rest = ["f_rest_%d" % i for i in range(3 * k)]
+    if shuffled:
+        rest = rest[::-1]  # numbered columns must be found by their index, not their position
+    names = (["x", "y", "z", "nx", "ny", "nz", "f_dc_0", "f_dc_1", "f_dc_2"] + rest + ["opacity"]
+             + ["scale_0", "scale_1", "scale_2", "rot_0", "rot_1", "rot_2", "rot_3"])
+    return names, k
+
+
+def _value(name, p):
+    # every (column, row) gets a distinct float32-exact value derived from the column NAME
+    return float(np.float32((sum(name.encode()) % 97) + 0.001 * len(name) + 100.0 * p + (hash_tail(name))))
+
+
+def hash_tail(name):
+    tail = name.split("_")[-1]
+    return 0.25 * int(tail) if tail.isdigit() else 0.0
+
+
+@pytest.mark.parametrize("fmt", ["binary_little_endian", "binary_big_endian", "ascii"])
+@pytest.mark.parametrize("deg", [0, 1, 3])
+def test_vanilla_ply_columns(tmp_path, fmt, deg):
+    names, k = _vanilla_props(deg, shuffled=True)
+    P = 5
+    rows = [[_value(n, p) for n in names] for p in range(P)]
+    assert len({v for row in rows for v in row}) == P * len(names)  # no two cells share a value
+    path = tmp_path / "point_cloud.ply"
+    _raw_ply(path, [(n, "float") for n in names], rows, fmt, trailing_element=(fmt != "ascii"))
+    s = ck.gaussian_state_dict(path, max_sh_degree=deg, prefix="gaussian_encoding.")
+    g = lambda key: s["gaussian_encoding." + key]  # noqa: E731
+    assert g("_xyz").shape == (P, 3) and g("_features_dc").shape == (P, 1, 3)
+    assert g("_features_rest").shape == (P, k, 3) and g("_opacity").shape == (P, 1)
+    assert all(t.dtype == torch.float32 and t.is_contiguous() for t in s.values())
+    for p in range(P):
+        assert g("_xyz")[p].tolist() == [_value(n, p) for n in "xyz"]
+        assert g("_opacity")[p, 0].item() == _value("opacity", p)
+        for c in range(3):
+            assert g("_features_dc")[p, 0, c].item() == _value("f_dc_%d" % c, p)
+            assert g("_scaling")[p, c].item() == _value("scale_%d" % c, p)
+            for j in range(k):  # channel-major storage: column c*k + j holds coefficient j of channel c
+                assert g("_features_rest")[p, j, c].item() == _value("f_rest_%d" % (c * k + j), p)
+        for c in range(4):
+            assert g("_rotation")[p, c].item() == _value("rot_%d" % c, p)
+
+
+def test_vanilla_ply_mixed_types_round_to_float32(tmp_path):
+    names, _ = _vanilla_props(0)
+    props = [(n, "double" if n in ("x", "opacity") else "float") for n in names]
+    rows = [[0.1 + p if n == "x" else _value(n, p) for n in names] for p in range(3)]
+    path = tmp_path / "d.ply"
+    _raw_ply(path, props, rows)
+    s = ck.gaussian_state_dict(path, max_sh_degree=0)
+    assert s["_xyz"][:, 0].tolist() == [float(np.float32(0.1 + p)) for p in range(3)]
+    assert s["_xyz"][:, 1].tolist() == [_value("y", p) for p in range(3)]
+
+
+def test_vanilla_cache_schema(tmp_path):
+    names = (["x", "y", "z", "nx", "ny", "nz"] + ["cache_f_%d" % i for i in range(12)] + ["cache_opacity"]
+             + ["cache_scale_%d" % i for i in range(3)] + ["cache_rot_%d" % i for i in range(4)])
+    rows = [[_value(n, p) for n in names] for p in range(4)]
+    path = tmp_path / "c.ply"
+    _raw_ply(path, [(n, "float") for n in names], rows)
+    s = ck.gaussian_state_dict(path, max_sh_degree=1)
+    assert set(s) == {"_xyz", "_cache_features", "_cache_opacity", "_cache_scaling", "_cache_rotation"}
+    assert s["_cache_features"].shape == (4, 4, 3)
+    assert s["_cache_features"][2, 3, 1].item() == _value("cache_f_%d" % (1 * 4 + 3), 2)
+    m = ck.load_gaussian_model(path, sh_degree=1, device="cpu")
+    assert m.get_opacity is s["_cache_opacity"] or torch.equal(m.get_opacity, s["_cache_opacity"])
+    assert torch.equal(m.get_features, s["_cache_features"]) and torch.equal(m.get_scaling, s["_cache_scaling"])
+    out = tmp_path / "resaved"
+    ck.save_model(m, out)
+    s2 = ck.gaussian_state_dict(out / "point_cloud.ply", max_sh_degree=1)
+    assert all(torch.equal(s[k], s2[k]) for k in s)
+
+
+def test_vanilla_errors(tmp_path):
+    names, _ = _vanilla_props(1)
+    path = tmp_path / "p.ply"
+    _raw_ply(path, [(n, "float") for n in names], [[0.0] * len(names)])
+    with pytest.raises(ck.PlyError, match="f_rest"):
+        ck.gaussian_state_dict(path, max_sh_degree=3)  # the reference asserts the same count
+    only_xyz = tmp_path / "xyz.ply"
+    _raw_ply(only_xyz, [(n, "float") for n in "xyz"], [[1.0, 2.0, 3.0]])
+    with pytest.raises(NotImplementedError, match="unsupport keys"):
+        ck.gaussian_state_dict(only_xyz)
+    bad = tmp_path / "bad.ply"
+    bad.write_bytes(b"plx\nformat ascii 1.0\nend_header\n")
+    with pytest.raises(ck.PlyError):
+        ck.read_ply(bad)
+    short = tmp_path / "short.ply"
+    _raw_ply(short, [(n, "float") for n in "xyz"], [[1.0, 2.0, 3.0]])
+    data = short.read_bytes()
+    short.write_bytes(data[:-4])
+    with pytest.raises(ck.PlyError, match="shorter"):
+        ck.read_ply(short)
+    lst = tmp_path / "list.ply"
+    lst.write_bytes(b"ply\nformat ascii 1.0\nelement vertex 1\nproperty list uchar int v\nend_header\n1 5\n")
+    with pytest.raises(ck.PlyError, match="list"):
+        ck.read_ply(lst)
+
+
+def _anchor_props(n_off, feat, octree):
+    head = ["x", "y", "z"] + (["level", "extra_level", "info"] if octree else ["nx", "ny", "nz"])
+    return (head + ["f_offset_%d" % i for i in range(3 * n_off)] + ["f_anchor_feat_%d" % i for i in range(feat)]
+            + ["opacity"] + ["scale_%d" % i for i in range(6)] + ["rot_%d" % i for i in range(4)])
+
+
+@pytest.mark.parametrize("n_off", [10, 4])
+def test_scaffold_ply_columns(tmp_path, n_off):
+    names = _anchor_props(n_off, 32, octree=False)
+    A = 3
+    rows = [[_value(n, a) for n in names] for a in range(A)]
+    path = tmp_path / "point_cloud.ply"
+    _raw_ply(path, [(n, "float") for n in names], rows)
+    s = ck.scaffold_state_dict(path)
+    assert s["_offset"].shape == (A, n_off, 3) and s["_anchor_feat"].shape == (A, 32)
+    assert s["_scaling"].shape == (A, 6) and s["_rotation"].shape == (A, 4) and s["_opacity"].shape == (A, 1)
+    for a in range(A):
+        assert s["_anchor"][a].tolist() == [_value(n, a) for n in "xyz"]
+        for j in range(n_off):
+            for axis in range(3):  # axis-major storage: column axis*n + j is component `axis` of offset j
+                assert s["_offset"][a, j, axis].item() == _value("f_offset_%d" % (axis * n_off + j), a)
+        assert s["_anchor_feat"][a].tolist() == [_value("f_anchor_feat_%d" % i, a) for i in range(32)]
+        assert s["_scaling"][a].tolist() == [_value("scale_%d" % i, a) for i in range(6)]
+
+
+def test_octree_ply_columns(tmp_path):
+    names = _anchor_props(10, 32, octree=True)
+    A = 4
+    rows = []
+    for a in range(A):
+        row = {n: _value(n, a) for n in names}
+        row["level"], row["extra_level"] = float(a % 3), 0.125 * a
+        row["info"] = [0.37, 12.5, 0.0, 0.0][a]
+        rows.append([row[n] for n in names])
+    path = tmp_path / "point_cloud.ply"
+    _raw_ply(path, [(n, "float") for n in names], rows)
+    s, voxel_size, standard_dist = ck.octree_state_dict(path)
+    assert voxel_size == float(np.float32(0.37)) and standard_dist == 12.5
+    assert s["_level"].dtype == torch.int32 and s["_level"].shape == (A, 1)
+    assert s["_level"][:, 0].tolist() == [0, 1, 2, 0]
+    assert s["_extra_level"].shape == (A,) and s["_extra_level"].tolist() == [0.0, 0.125, 0.25, 0.375]
+    assert s["_offset"][2, 7, 1].item() == _value("f_offset_%d" % (1 * 10 + 7), 2)
+    with pytest.raises(ck.PlyError, match="two rows"):
+        one = tmp_path / "one.ply"
+        _raw_ply(one, [(n, "float") for n in names], rows[:1])
+        ck.octree_state_dict(one)
+
+
+def _random_anchor_args(A, n_off, g):
+    r = lambda *s: torch.randn(*s, generator=g)  # noqa: E731
+    return r(A, 3), r(A, 32), r(A, n_off, 3), r(A, 6), r(A, 4)
+
+
+def _randomise_decoder(m, g):
+    for p in m.anchor_decoder.parameters():
+        p.data = torch.randn(p.shape, generator=g)
+
+
+def test_writer_header_and_layout(tmp_path):
+    g = torch.Generator().manual_seed(1)
+    m = GaussianModel(torch.randn(6, 3, generator=g), torch.randn(6, 1, 3, generator=g),
+                      torch.randn(6, 15, 3, generator=g), torch.randn(6, 3, generator=g),
+                      torch.randn(6, 4, generator=g), torch.randn(6, 1, generator=g))
+    ck.save_model(m, tmp_path)
+    raw = (tmp_path / "point_cloud.ply").read_bytes()
+    head, body = raw.split(b"end_header\n", 1)
+    lines = head.decode().splitlines()
+    names, _ = _vanilla_props(3)
+    assert lines[:3] == ["ply", "format binary_little_endian 1.0", "element vertex 6"]
+    assert lines[3:] == ["property float %s" % n for n in names]  # the reference's column order
+    table = np.frombuffer(body, dtype="<f4").reshape(6, len(names))
+    assert not os.path.exists(tmp_path / "state_dict.th")  # vanilla 3DGS has no MLP state
+    assert np.array_equal(table[:, 3:6], np.zeros((6, 3), np.float32))
+    # f_rest column c*15+j holds _features_rest[:, j, c]
+    assert np.array_equal(table[:, names.index("f_rest_%d" % (2 * 15 + 4))], m._features_rest[:, 4, 2].numpy())
+    assert np.array_equal(table[:, names.index("f_dc_1")], m._features_dc[:, 0, 1].numpy())
+
+
+def test_round_trip_all_models(tmp_path):
+    g = torch.Generator().manual_seed(3)
+    v = GaussianModel(torch.randn(9, 3, generator=g), torch.randn(9, 1, 3, generator=g),
+                      torch.randn(9, 15, 3, generator=g), torch.randn(9, 3, generator=g),
+                      torch.randn(9, 4, generator=g), torch.randn(9, 1, generator=g))
+    ck.save_model(v, tmp_path / "v")
+    v2 = ck.load_gaussian_model(tmp_path / "v", device="cpu")
+    assert all(torch.equal(a, b) for a, b in zip(v.parameters(), v2.parameters()))
+
+    s = ScaffoldGS(*_random_anchor_args(7, 10, g), opacity=torch.randn(7, 1, generator=g), add_cov_dist=False)
+    _randomise_decoder(s, g)
+    ck.save_model(s, tmp_path / "s")
+    keys = set(torch.load(tmp_path / "s" / "state_dict.th", weights_only=True))
+    assert keys == {"anchor_decoder.mlp_%s.%d.%s" % (h, i, w) for h in ("opacity", "cov", "color") for i in (0, 2)
+                    for w in ("weight", "bias")}
+    s2 = ck.load_scaffold_gs(tmp_path / "s", device="cpu")
+    assert s2.anchor_decoder.mlp_cov[0].weight.shape[1] == 35 and s2.anchor_decoder.mlp_color[0].weight.shape[1] == 36
+    assert [n for n, _ in s.named_parameters()] == [n for n, _ in s2.named_parameters()]
+    assert all(torch.equal(a, b) for a, b in zip(s.parameters(), s2.parameters()))
+
+    level = torch.tensor([0, 1, 2, 1, 0, 2, 1])
+    o = OctreeGS(*_random_anchor_args(7, 10, g), level, 0.37, 12.5, extra_level=torch.randn(7, generator=g))
+    _randomise_decoder(o, g)
+    ck.save_model(o, tmp_path / "o", rank=3)
+    assert os.path.exists(tmp_path / "o" / "point_cloud-sub3.ply") and os.path.exists(tmp_path / "o" / "state_dict-sub3.th")
+    ck.save_model(o, tmp_path / "o")
+    o2 = ck.load_octree_gs(tmp_path / "o", device="cpu")
+    assert o2.voxel_size == float(np.float32(0.37)) and o2.standard_dist == 12.5
+    assert torch.equal(o._level, o2._level) and torch.equal(o._extra_level, o2._extra_level)
+    assert all(torch.equal(a, b) for a, b in zip(o.parameters(), o2.parameters()))
+
+
+def test_merged_state_dict_rejects_duplicates(tmp_path):
+    g = torch.Generator().manual_seed(4)
+    s = ScaffoldGS(*_random_anchor_args(3, 10, g))
+    ck.save_model(s, tmp_path)
+    merged = ck.merged_state_dict(tmp_path / "point_cloud.ply", "scaffold")
+    assert "gaussian_encoding._anchor" in merged and "anchor_decoder.mlp_cov.2.bias" in merged
+    torch.save({"gaussian_encoding._anchor": torch.zeros(1)}, tmp_path / "state_dict.th")
+    with pytest.raises(ValueError, match="Duplicate keys found"):
+        ck.merged_state_dict(tmp_path / "point_cloud.ply", "scaffold")

@@ -123,3 +123,31 @@ def test_fused_prefilter_gives_the_same_frame(gpu_device):
     keep[::2] = False
     assert torch.equal(plain(scene.camera, render_exclude_filter=keep), fused(scene.camera, render_exclude_filter=keep))
     assert torch.equal(plain(scene.camera, scaling_modifier=0.7), fused(scene.camera, scaling_modifier=0.7))
+
+
+def test_checkpoint_round_trip_renders_the_same_frame(gpu_device, tmp_path):
+    """point_cloud.ply + state_dict.th written in the reference's layout, read back, rendered: identical frames."""
+    from landmarksystem_amd import checkpoints as ck
+    scene = scenes.config2(P=30_000, width=480, height=270)
+    vanilla = GaussianModel.from_activated(scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs,
+                                           sh_degree=3).to(gpu_device).eval()
+    ck.save_model(vanilla, tmp_path / "v")
+    loaded = ck.load_gaussian_model(tmp_path / "v", device=gpu_device).eval()
+    assert torch.equal(vanilla(scene.camera), loaded(scene.camera))
+    assert float(loaded(scene.camera).max()) > 0.0
+
+    anchors = scenes.config5(A=20_000, width=480, height=270)
+    scaffold = ScaffoldGS.from_scene(anchors).to(gpu_device).eval()
+    ck.save_model(scaffold, tmp_path / "s")
+    loaded = ck.load_scaffold_gs(tmp_path / "s", device=gpu_device).eval()
+    assert torch.equal(scaffold(anchors.camera), loaded(anchors.camera))
+
+    level = torch.randint(0, 5, (20_000,), generator=torch.Generator().manual_seed(5))
+    octree = OctreeGS(anchors.anchor, anchors.anchor_feat, anchors.offset, torch.log(anchors.scaling),
+                      anchors.rotation, level, voxel_size=0.5, standard_dist=250.0, n_offsets=anchors.n_offsets)
+    octree.anchor_decoder.load_state_dict(scaffold.anchor_decoder.state_dict())
+    octree = octree.to(gpu_device).eval()
+    ck.save_model(octree, tmp_path / "o")
+    loaded = ck.load_octree_gs(tmp_path / "o", device=gpu_device).eval()
+    assert torch.equal(octree(anchors.camera), loaded(anchors.camera))
+    assert torch.equal(octree._anchor_mask, loaded._anchor_mask) and 0 < int(loaded._anchor_mask.sum()) < 20_000

@@ -46,40 +46,113 @@ __device__ __forceinline__ void covariance3d(const float* __restrict__ scale, fl
     cov[5] = (l20 * l20 + l21 * l21) + l22 * l22;
 }
 
-// SH degree 0..3 -> RGB for one Gaussian; `sh` points at its [M,3] block
-// (coefficient-major, RGB innermost) in global memory or in LDS.
-__device__ __forceinline__ void sh_to_rgb(int degree, const float* sh, float dx, float dy, float dz, float out[3])
+// Real SH basis of degree 0..3 at the unit direction (dx, dy, dz), with the
+// sign of each term folded in, so that colour = sum_k basis[k] * sh[k].
+// Each value is the product the closed-form expression multiplies the
+// coefficient by, associated the same way ((C * a) * b).
+__device__ __forceinline__ void sh_basis(int degree, float dx, float dy, float dz, float b[16])
 {
     const float len = sqrtf((dx * dx + dy * dy) + dz * dz);
     dx = dx / len;
     dy = dy / len;
     dz = dz / len;
-#pragma unroll
-    for (int c = 0; c < 3; ++c) {
-        float res = kShC0 * sh[c];
-        if (degree > 0) {
-            res = res - kShC1 * dy * sh[3 + c] + kShC1 * dz * sh[6 + c] - kShC1 * dx * sh[9 + c];
-            if (degree > 1) {
-                const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
-                const float xy = dx * dy, yz = dy * dz, xz = dx * dz;
-                res = res + kShC2[0] * xy * sh[12 + c] + kShC2[1] * yz * sh[15 + c] +
-                      kShC2[2] * (2.0f * zz - xx - yy) * sh[18 + c] + kShC2[3] * xz * sh[21 + c] +
-                      kShC2[4] * (xx - yy) * sh[24 + c];
-                if (degree > 2) {
-                    res = res + kShC3[0] * dy * (3.0f * xx - yy) * sh[27 + c] + kShC3[1] * xy * dz * sh[30 + c] +
-                          kShC3[2] * dy * (4.0f * zz - xx - yy) * sh[33 + c] +
-                          kShC3[3] * dz * (2.0f * zz - 3.0f * xx - 3.0f * yy) * sh[36 + c] +
-                          kShC3[4] * dx * (4.0f * zz - xx - yy) * sh[39 + c] + kShC3[5] * dz * (xx - yy) * sh[42 + c] +
-                          kShC3[6] * dx * (xx - 3.0f * yy) * sh[45 + c];
-                }
+    b[0] = kShC0;
+    if (degree > 0) {
+        b[1] = -(kShC1 * dy);
+        b[2] = kShC1 * dz;
+        b[3] = -(kShC1 * dx);
+        if (degree > 1) {
+            const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
+            const float xy = dx * dy, yz = dy * dz, xz = dx * dz;
+            b[4] = kShC2[0] * xy;
+            b[5] = kShC2[1] * yz;
+            b[6] = kShC2[2] * (2.0f * zz - xx - yy);
+            b[7] = kShC2[3] * xz;
+            b[8] = kShC2[4] * (xx - yy);
+            if (degree > 2) {
+                b[9] = kShC3[0] * dy * (3.0f * xx - yy);
+                b[10] = kShC3[1] * xy * dz;
+                b[11] = kShC3[2] * dy * (4.0f * zz - xx - yy);
+                b[12] = kShC3[3] * dz * (2.0f * zz - 3.0f * xx - 3.0f * yy);
+                b[13] = kShC3[4] * dx * (4.0f * zz - xx - yy);
+                b[14] = kShC3[5] * dz * (xx - yy);
+                b[15] = kShC3[6] * dx * (xx - 3.0f * yy);
             }
         }
-        res += 0.5f;
-        out[c] = res < 0.0f ? 0.0f : res;
     }
 }
 
-constexpr int kShStride = 52;  // floats per Gaussian in the LDS staging area: 48 + 4 keeps 16-B reads conflict-free
+// res[c] += sum over coefficients k in [kFirst, kFirst + kCount) below
+// `terms` of basis[k] * sh[3 * (k - kFirst) + c], added one by one in
+// ascending k: `sh` points at coefficient kFirst of a [M,3] block
+// (coefficient-major, RGB innermost) in global memory or in LDS.
+template <int kFirst, int kCount>
+__device__ __forceinline__ void sh_accumulate(int terms, const float* sh, const float b[16], float res[3])
+{
+#pragma unroll
+    for (int k = 0; k < kCount; ++k) {
+        if (kFirst + k < terms) {
+#pragma unroll
+            for (int c = 0; c < 3; ++c) res[c] = res[c] + b[kFirst + k] * sh[3 * k + c];
+        }
+    }
+}
+
+__device__ __forceinline__ void sh_finish(float res[3])
+{
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+        const float v = res[c] + 0.5f;
+        res[c] = v < 0.0f ? 0.0f : v;
+    }
+}
+
+// SH blocks are staged through LDS in kShRounds rounds of kShChunk
+// coefficients; the stride keeps the 16-B reads of the 64 lanes on distinct
+// banks (stride = 4 mod 8 floats).
+constexpr int kShRounds = 1;
+constexpr int kShChunk = 16 / kShRounds;                                   // coefficients per round
+constexpr int kShChunk4 = kShChunk * 3 / 4;                                // float4s per Gaussian per round
+constexpr int kShStride = kShChunk * 3 + ((kShChunk * 3) % 8 == 0 ? 4 : 0);  // floats per Gaussian in LDS
+
+// Orders one wavefront's LDS writes before its later LDS reads (and the reverse): the hardware executes a
+// wavefront's LDS instructions in order, this keeps the compiler from moving them across.
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int kRound>
+__device__ __forceinline__ void sh_staged_rounds(float4* __restrict__ mine, const float4* __restrict__ src, int count,
+                                                 int lane, bool alive, int terms, const float b[16], float res[3])
+{
+    if constexpr (kRound < kShRounds) {
+        if (kRound * kShChunk < terms) {  // uniform: lower degrees stop early
+            if (kRound > 0) wave_lds_sync();
+            // all loads of the round are issued before the first LDS write, so they are in flight together;
+            // slots past a partial wavefront's last Gaussian re-read that Gaussian (same value, same address)
+            float4 v[kShChunk4];
+            int dst[kShChunk4];
+#pragma unroll
+            for (int it = 0; it < kShChunk4; ++it) {
+                const int q4 = it * 64 + lane;
+                const int gq = min(q4 / kShChunk4, count - 1), m = q4 % kShChunk4;
+                v[it] = src[gq * 12 + kRound * kShChunk4 + m];
+                dst[it] = gq * (kShStride / 4) + m;
+            }
+#pragma unroll
+            for (int it = 0; it < kShChunk4; ++it) mine[dst[it]] = v[it];
+            wave_lds_sync();
+            if (alive)
+                sh_accumulate<kRound * kShChunk, kShChunk>(terms, reinterpret_cast<const float*>(mine) + lane * kShStride,
+                                                           b, res);
+            sh_staged_rounds<kRound + 1>(mine, src, count, lane, alive, terms, b, res);
+        }
+    }
+}
+
 
 template <bool kRadiiOnly>
 __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaussians g,
@@ -102,10 +175,27 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
     uint32_t touched = 0;
     uint64_t rect_packed = 0;  // x0 | y0 << 16 | x1 << 32 | y1 << 48, zero when culled
     float x = 0.f, y = 0.f, z = 0.f, vz = 0.f, px = 0.f, py = 0.f, ca = 0.f, cc = 0.f, qx = 0.f, qy = 0.f, qz = 0.f;
-    if (valid) do {
+    // Every per-Gaussian geometry input is requested up front, before the cull
+    // decides whether it is needed: one memory latency instead of a chain of
+    // dependent ones (culled Gaussians cost 28 to 32 B of extra reads).
+    float cov[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, scale[3] = {0.f, 0.f, 0.f}, quat[4] = {0.f, 0.f, 0.f, 0.f};
+    float opacity = 0.f;
+    if (valid) {
         x = g.means3D[3 * (size_t)i];
         y = g.means3D[3 * (size_t)i + 1];
         z = g.means3D[3 * (size_t)i + 2];
+        if (g.cov3D_precomp) {
+#pragma unroll
+            for (int k = 0; k < 6; ++k) cov[k] = g.cov3D_precomp[6 * (size_t)i + k];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 3; ++k) scale[k] = g.scales[3 * (size_t)i + k];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) quat[k] = g.rotations[4 * (size_t)i + k];
+        }
+        if (!kRadiiOnly) opacity = g.opacities[i];
+    }
+    if (valid) do {
         const float vx = ((V[0] * x + V[4] * y) + V[8] * z) + V[12];
         const float vy = ((V[1] * x + V[5] * y) + V[9] * z) + V[13];
         vz = ((V[2] * x + V[6] * y) + V[10] * z) + V[14];
@@ -117,13 +207,7 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
         const float inv_w = 1.0f / (hw + 0.0000001f);
         const float ndc_x = hx * inv_w, ndc_y = hy * inv_w;
 
-        float cov[6];
-        if (g.cov3D_precomp) {
-#pragma unroll
-            for (int k = 0; k < 6; ++k) cov[k] = g.cov3D_precomp[6 * (size_t)i + k];
-        } else {
-            covariance3d(g.scales + 3 * (size_t)i, f.scale_modifier, g.rotations + 4 * (size_t)i, cov);
-        }
+        if (!g.cov3D_precomp) covariance3d(scale, f.scale_modifier, quat, cov);
 
         // EWA splatting: Jacobian of the perspective projection at the
         // (frustum-clamped) view-space mean, times the world->view rotation.
@@ -189,29 +273,26 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
             rgb[2] = g.colors_precomp[3 * (size_t)i + 2];
         }
     } else {
-        const float dx = x - f.campos[0], dy = y - f.campos[1], dz = z - f.campos[2];
         // When most of the wavefront survived and the blocks are the full 192 B,
-        // the 12 KB of SH of its 64 Gaussians are fetched with fully coalesced
-        // 16-B loads into LDS and each lane reads its own block back from there;
-        // otherwise every survivor fetches its own block.  Same values either way.
+        // the SH of its 64 Gaussians is fetched with coalesced 16-B loads into
+        // LDS, a chunk of coefficients at a time, and each lane reads its own
+        // chunk back from there; otherwise every survivor fetches its own
+        // block.  Same values and the same order of additions either way.
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
         const int wave_first = blockIdx.x * blockDim.x + wave * 64;
         const bool staged = f.sh_coeffs == 16 && (reinterpret_cast<uintptr_t>(g.shs) & 15u) == 0 &&
                             __popcll(__ballot(alive)) >= 32;  // uniform per wavefront
+        const int terms = (f.sh_degree + 1) * (f.sh_degree + 1);
+        float b[16];
+        if (alive) sh_basis(f.sh_degree, x - f.campos[0], y - f.campos[1], z - f.campos[2], b);
         if (staged) {
-            float4* __restrict__ mine = s_sh + wave * (64 * kShStride / 4);
-            const float4* __restrict__ src = reinterpret_cast<const float4*>(g.shs + (size_t)wave_first * 48);
-            const int count4 = min(64, g.P - wave_first) * 12;
-#pragma unroll
-            for (int it = 0; it < 12; ++it) {
-                const int q4 = it * 64 + lane;
-                if (q4 < count4) mine[(q4 / 12) * (kShStride / 4) + q4 % 12] = src[q4];
-            }
-            __builtin_amdgcn_wave_barrier();
-            if (alive) sh_to_rgb(f.sh_degree, reinterpret_cast<const float*>(mine) + lane * kShStride, dx, dy, dz, rgb);
+            sh_staged_rounds<0>(s_sh + wave * (64 * kShStride / 4),
+                                reinterpret_cast<const float4*>(g.shs + (size_t)wave_first * 48),
+                                min(64, g.P - wave_first), lane, alive, terms, b, rgb);
         } else if (alive) {
-            sh_to_rgb(f.sh_degree, g.shs + (size_t)i * f.sh_coeffs * 3, dx, dy, dz, rgb);
+            sh_accumulate<0, 16>(terms, g.shs + (size_t)i * f.sh_coeffs * 3, b, rgb);
         }
+        if (alive) sh_finish(rgb);
     }
     if (!alive) return;
 
@@ -222,7 +303,6 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
     // exponent (bounded below by `noise`), so a quadrant outside the box is
     // certain to take the blend's `alpha < 1/255` branch on all of its pixels.
     // +inf = never cull (large or ill-conditioned splats), -inf = never visible.
-    const float opacity = g.opacities[i];
     float ex, ey;
     {
         const float reach = (float)radius + 24.0f;  // |d| over every pixel of every touched tile

@@ -65,9 +65,14 @@ __device__ __forceinline__ half4_t to_half4(float a, float b, float c, float d)
 // lane (row = lane % 32, half = lane / 32) holds W[row0 + row][8s + 4*half + 0..3].
 __device__ __forceinline__ half4_t weight_fragment(const float* __restrict__ w, int rows, int cols, int row, int k0)
 {
+    // loads are unconditional at clamped (in-range) positions and masked afterwards, so that none of them
+    // waits for another: the fragments of a head are fetched with all loads in flight together
     float v[4];
+    const int r = min(row, rows - 1);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) v[t] = (row < rows && k0 + t < cols) ? w[(size_t)row * cols + k0 + t] : 0.0f;
+    for (int t = 0; t < 4; ++t) v[t] = w[(size_t)r * cols + min(k0 + t, cols - 1)];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) v[t] = (row < rows && k0 + t < cols) ? v[t] : 0.0f;
     return to_half4(v[0], v[1], v[2], v[3]);
 }
 
@@ -155,6 +160,16 @@ __device__ __forceinline__ void store_rows(float* __restrict__ dst_anchor, int b
     }
 }
 
+// Per-lane inputs of one tile of 32 anchors.
+template <bool kCountOnly>
+struct TileInputs {
+    float4 f[4] = {};          // features 8s + 4*half .. +3, s = 0..3
+    float pos[3] = {0.f, 0.f, 0.f};
+    float sc3[3] = {0.f, 0.f, 0.f};
+    uint32_t first_slot = 0;
+    float ofv[kCountOnly ? 1 : 5][3] = {};
+};
+
 template <bool kCountOnly>
 __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
                                                      const uint32_t* __restrict__ offsets, uint32_t capacity,
@@ -162,9 +177,11 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
                                                      float* __restrict__ opacity, float* __restrict__ scaling_out,
                                                      float* __restrict__ rot)
 {
-    // per wavefront: [32 anchors][stride] floats; stride odd -> conflict-free column access
-    constexpr int kStrideMax = kCountOnly ? 11 : 113;
-    __shared__ float s_out[4][32 * kStrideMax];
+    // per wavefront: [32 anchors][stride] floats; stride odd -> conflict-free column access.  Emit pass: the
+    // 11n head outputs of an anchor, then its scaling (6), position (3) and first output slot (1).
+    constexpr int kStrideMax = kCountOnly ? 11 : 123;
+    constexpr int kListFloats = kCountOnly ? 0 : 160;  // 320 16-bit item numbers after the anchors' rows
+    __shared__ float s_out[4][32 * kStrideMax + kListFloats];
 
     // biases of the three heads, zero-padded: b0 at [head*32], b1 of opacity / cov / colour at 96 / 128 / 224
     __shared__ float s_bias[256];
@@ -189,7 +206,10 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         load_head<3>(d, 1, 7 * n, col, half, w_cov);
         load_head<1>(d, 2, 3 * n, col, half, w_col);
     }
-    const int stride = kCountOnly ? 11 : 11 * n + 3;
+    const int stride = kCountOnly ? 11 : 11 * n + 13;
+    const int items = 32 * n;  // (anchor, offset) pairs of a tile: item = anchor_in_tile * n + offset
+    const int inv_n = (65536 + n - 1) / n;  // item / n == (item * inv_n) >> 16 for item < 32 n, n <= 10
+    const uint64_t lanes_below = (1ull << lane) - 1ull;
     const int tiles = (d.A + 31) / 32;
     float* __restrict__ mine = s_out[wave];
     const float cx = d.campos[0], cy = d.campos[1], cz = d.campos[2];
@@ -197,24 +217,44 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
     for (int tile = blockIdx.x * 4 + wave; tile < tiles; tile += gridDim.x * 4) {
         const int a = tile * 32 + col;  // this lane's anchor (lanes l and l+32 share it)
         const bool vis = a < d.A && d.visible[a] != 0;
-        const uint64_t any = __ballot(vis);
+        const uint64_t any = __ballot(vis);  // bits l and l + 32 belong to anchor l of the tile
         if (any == 0ull) {  // nothing visible in these 32 anchors
             if (kCountOnly && half == 0 && a < d.A) counts[a] = 0;
             continue;
         }
-        // B operand: X^T, column = anchor, k = 8s + 4*half + t
-        half4_t X[5];
-        float ax = 0.f, ay = 0.f, az = 0.f;
+        // Everything the tile needs from global memory is requested here, before the first use.
+        TileInputs<kCountOnly> in;
         if (vis) {
             const float4* __restrict__ f4 = reinterpret_cast<const float4*>(d.feat + (size_t)a * kFeat);
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const float4 v = f4[2 * s + half];
-                X[s] = to_half4(v.x, v.y, v.z, v.w);
+            for (int s = 0; s < 4; ++s) in.f[s] = f4[2 * s + half];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) in.pos[k] = d.anchor[3 * (size_t)a + k];
+        }
+        if constexpr (!kCountOnly) {
+            // half 0: scaling[0..2] (offset scale), half 1: scaling[3..5] (Gaussian scale)
+            if (vis) {
+#pragma unroll
+                for (int k = 0; k < 3; ++k) in.sc3[k] = d.scaling[6 * (size_t)a + 3 * half + k];
             }
-            ax = d.anchor[3 * (size_t)a];
-            ay = d.anchor[3 * (size_t)a + 1];
-            az = d.anchor[3 * (size_t)a + 2];
+            if (a < d.A) in.first_slot = offsets[a];  // lane 0's value is the tile's first output slot
+            // the learned offsets of the items this lane's position covers (contiguous over the lanes),
+            // for visible anchors only
+#pragma unroll
+            for (int r = 0; r < 5; ++r) {
+                const int it = r * 64 + lane;
+                const bool want = it < items && ((any >> ((it * inv_n) >> 16)) & 1ull);
+                const float* __restrict__ of = d.offset + ((size_t)tile * 32 * n + (want ? it : 0)) * 3;
+#pragma unroll
+                for (int k = 0; k < 3; ++k) in.ofv[r][k] = want ? of[k] : 0.0f;
+            }
+        }
+        // B operand: X^T, column = anchor, k = 8s + 4*half + t
+        half4_t X[5];
+        const float ax = in.pos[0], ay = in.pos[1], az = in.pos[2];
+        if (vis) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) X[s] = to_half4(in.f[s].x, in.f[s].y, in.f[s].z, in.f[s].w);
             float vx = ax - cx, vy = ay - cy, vz = az - cz;
             const float dist = sqrtf(vx * vx + vy * vy + vz * vz);
             vx /= dist;
@@ -259,32 +299,69 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         floatx16 cl[1];
         run_head<1>(w_col, s_bias + 64, s_bias + 224, X, half, cl);
         store_rows(mine + col * stride, 8 * n, 3 * n, 0, half, cl[0]);
+        {
+            float* __restrict__ extra = mine + col * stride + 11 * n;
+#pragma unroll
+            for (int k = 0; k < 3; ++k) extra[3 * half + k] = in.sc3[k];
+            if (half == 0) {
+                extra[6] = ax;
+                extra[7] = ay;
+                extra[8] = az;
+                reinterpret_cast<uint32_t*>(extra)[9] = in.first_slot;
+            }
+        }
         __builtin_amdgcn_wave_barrier();
 
-        // ---- per (anchor, offset): mask, post-process, write at its slot ----
-        const int items = 32 * n;
-        for (int it = lane; it < items; it += 64) {
-            const int al = it / n, m = it - al * n;
-            const int ga = tile * 32 + al;
-            if (ga >= d.A || d.visible[ga] == 0) continue;
+        // ---- compact the kept (anchor, offset) items of the tile: about one in five survives the mask, and the
+        // activations below are the expensive part, so they run on dense wavefronts of survivors only ----
+        uint16_t* __restrict__ list = reinterpret_cast<uint16_t*>(mine + 32 * stride);  // [32 n] item numbers
+        uint32_t total = 0;
+#pragma unroll
+        for (int r = 0; r < 5; ++r) {
+            if (r * 64 >= items) break;  // uniform
+            const int it = r * 64 + lane;
+            bool kept = false;
+            if (it < items) {
+                const int al = (it * inv_n) >> 16, m = it - al * n;
+                kept = ((any >> al) & 1ull) && mine[al * stride + m] > 0.0f;
+            }
+            const uint64_t b = __ballot(kept);
+            if (kept) list[total + (uint32_t)__popcll(b & lanes_below)] = (uint16_t)it;
+            total += (uint32_t)__popcll(b);
+        }
+        __builtin_amdgcn_wave_barrier();
+
+        // Items are numbered anchor-major and the slots come from an exclusive scan of the per-anchor counts, so
+        // the survivors of a tile occupy consecutive output slots from the slot of its first anchor: lanes write
+        // consecutive addresses.  No global reads in here: the learned offsets sit in registers of the lane that
+        // requested them (item = round * 64 + lane) and are fetched across lanes.
+        const uint32_t tile_slot = reinterpret_cast<const uint32_t*>(mine)[11 * n + 9];
+        for (uint32_t s0 = 0; s0 < total; s0 += 64) {  // uniform
+            const uint32_t s = s0 + lane;
+            const bool live = s < total;
+            const int it = live ? (int)list[s] : 0;
+            float off3[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+            for (int r = 0; r < 5; ++r) {
+#pragma unroll
+                for (int k = 0; k < 3; ++k) {
+                    const float got = __shfl(in.ofv[r][k], it & 63, 64);
+                    if ((it >> 6) == r) off3[k] = got;
+                }
+            }
+            const uint32_t pos = tile_slot + s;
+            if (!live || pos >= capacity) continue;  // the second cannot happen when capacity comes from the count pass
+            const int al = (it * inv_n) >> 16, m = it - al * n;
             const float* __restrict__ o = mine + al * stride;
-            if (!(o[m] > 0.0f)) continue;
-            const float opac = tanhf(o[m]);
-            uint32_t rank = 0;
-            for (int mm = 0; mm < m; ++mm) rank += o[mm] > 0.0f ? 1u : 0u;
-            const uint32_t pos = offsets[ga] + rank;
-            if (pos >= capacity) continue;  // cannot happen when capacity comes from the count pass
+            const float* __restrict__ extra = o + 11 * n;
             const float* __restrict__ c7 = o + n + 7 * m;
             const float* __restrict__ c3 = o + 8 * n + 3 * m;
-            const float* __restrict__ sc = d.scaling + 6 * (size_t)ga;
-            const float* __restrict__ of = d.offset + (size_t)ga * n * 3 + 3 * m;
-            const float* __restrict__ an = d.anchor + 3 * (size_t)ga;
-            opacity[pos] = opac;
+            opacity[pos] = tanhf(o[m]);
 #pragma unroll
             for (int k = 0; k < 3; ++k) {
                 color[3 * (size_t)pos + k] = 1.0f / (1.0f + expf(-c3[k]));
-                scaling_out[3 * (size_t)pos + k] = sc[3 + k] * (1.0f / (1.0f + expf(-c7[k])));
-                xyz[3 * (size_t)pos + k] = an[k] + of[k] * sc[k];
+                scaling_out[3 * (size_t)pos + k] = extra[3 + k] * (1.0f / (1.0f + expf(-c7[k])));
+                xyz[3 * (size_t)pos + k] = extra[6 + k] + off3[k] * extra[k];
             }
             const float q0 = c7[3], q1 = c7[4], q2 = c7[5], q3 = c7[6];
             const float norm = fmaxf(sqrtf(q0 * q0 + q1 * q1 + q2 * q2 + q3 * q3), 1e-12f);
@@ -341,11 +418,13 @@ static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, DecodeAr
     return GS355_OK;
 }
 
-static dim3 decode_grid(int A)
+// Persistent workgroups (4 wavefronts, each walking tiles of 32 anchors): at most `cap` of them, about what
+// the chip holds at once, so the weight fragments are fetched once per resident workgroup.
+static dim3 decode_grid(int A, int cap)
 {
     const int tiles = (A + 31) / 32;
     int blocks = (tiles + 3) / 4;
-    if (blocks > 2048) blocks = 2048;
+    if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
     return dim3(blocks);
 }
@@ -377,7 +456,7 @@ int gs355_decode_count(const gs355_decoder* dec, const gs355_anchors* an, uint32
     if (scratch_bytes < need)
         return set_error(GS355_ENOSPC, "decode scratch has %zu bytes, %zu needed", scratch_bytes, need);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(decode_kernel<true>, decode_grid(a.A), dim3(256), 0, s, a, counts, (const uint32_t*)nullptr, 0u,
+    hipLaunchKernelGGL(decode_kernel<true>, decode_grid(a.A, 1024), dim3(256), 0, s, a, counts, (const uint32_t*)nullptr, 0u,
                        (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr);
     GS355_CHECK_LAUNCH("decode: count");
     return launch_exclusive_scan(counts, offsets, (size_t)a.A, static_cast<uint32_t*>(scratch), s);
@@ -396,7 +475,7 @@ int gs355_decode_emit(const gs355_decoder* dec, const gs355_anchors* an, const u
     if (!out || !out->xyz || !out->color || !out->opacity || !out->scaling || !out->rot)
         return set_error(GS355_EINVAL, "decoded outputs must all be non-NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(decode_kernel<false>, decode_grid(a.A), dim3(256), 0, s, a, (uint32_t*)nullptr, offsets,
+    hipLaunchKernelGGL(decode_kernel<false>, decode_grid(a.A, 512), dim3(256), 0, s, a, (uint32_t*)nullptr, offsets,
                        (uint32_t)capacity, out->xyz, out->color, out->opacity, out->scaling, out->rot);
     GS355_CHECK_LAUNCH("decode: emit");
     return GS355_OK;

@@ -4,10 +4,14 @@
 // [3,H,W] image at tests/test_inference_framework/test_inference.py:195-197).
 //
 // Blending: one 256-thread workgroup per 16x16 pixel tile, each of its four
-// wavefronts owning an 8x8 pixel quadrant.  The tile's depth-sorted Gaussians
-// are staged through LDS in batches of 256 records (48 B each); a wavefront
-// stops reading as soon as a ballot shows all of its 64 pixels finished, and
-// the workgroup stops fetching batches once all four wavefronts have.
+// wavefronts owning an 8x8 pixel quadrant, each group of 16 lanes a 4x4 block
+// of it.  The tile's depth-sorted Gaussians are staged through LDS in batches
+// of 256 records (48 B each); every 4x4 block gets its own list of the staged
+// Gaussians that can reach it, and the four lane groups of a wavefront walk
+// their lists side by side, so one pass of the pixel arithmetic serves four
+// different Gaussians.  A wavefront stops as soon as a ballot shows all of
+// its 64 pixels finished, and the workgroup stops fetching batches once all
+// four wavefronts have.
 #include "gs355_internal.h"
 
 namespace gs355 {
@@ -84,11 +88,13 @@ __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, c
     }
 }
 
-// kCull: each wavefront first tests the staged Gaussians against its own 8x8
-// quadrant (one Gaussian per lane, bounding box of the alpha >= 1/255 region
-// from the record) and then visits only the ballot's set bits.  A skipped
-// (quadrant, Gaussian) pair is one whose 64 pixels would all have taken the
-// `alpha < 1/255` branch, so both variants produce identical images.
+// kCull: each wavefront first tests the staged Gaussians (one per lane) against
+// the four 4x4 blocks of its quadrant, using the bounding box of the
+// alpha >= 1/255 region from the record, and appends the survivors, in depth
+// order, to the list of each block they can reach.  A (block, Gaussian) pair
+// that is left out is one whose 16 pixels would all have taken the
+// `alpha < 1/255` branch, and every pixel still sees its Gaussians front to
+// back with the same arithmetic, so both variants produce identical images.
 template <bool kCull>
 __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_header* __restrict__ header,
                                                     const uint32_t* __restrict__ ranges,
@@ -100,17 +106,22 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
     __shared__ float4 s_b[256];  // conic_z, opacity, r, g
     __shared__ float4 s_c[256];  // b, depth, reach_x, reach_y
     __shared__ uint32_t s_wave_done[4];
+    // per wavefront and 4x4 block: staged-record numbers of the Gaussians that can reach the block
+    __shared__ uint8_t s_list[kCull ? 4 : 1][4][256 + 4];
 
     if (header->overflow) return;
     const int tile = blockIdx.x;
     const int tile_x = tile % f.grid_x, tile_y = tile / f.grid_x;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int group = lane >> 4, sub = lane & 15;  // 4x4 block within the quadrant, pixel within the block
     const int qx0 = tile_x * kTile + (wave & 1) * 8, qy0 = tile_y * kTile + (wave >> 1) * 8;
-    const int px = qx0 + (lane & 7), py = qy0 + (lane >> 3);
+    const int px = qx0 + (group & 1) * 4 + (sub & 3), py = qy0 + (group >> 1) * 4 + (sub >> 2);
     const bool inside = px < f.W && py < f.H;
     const float pxf = (float)px, pyf = (float)py;
-    // pixel-centre bounds of this wavefront's quadrant
-    const float qx_lo = (float)qx0, qx_hi = (float)(qx0 + 7), qy_lo = (float)qy0, qy_hi = (float)(qy0 + 7);
+    // pixel-centre bounds of the quadrant's two block columns and two block rows
+    const float x_lo0 = (float)qx0, x_hi0 = (float)(qx0 + 3), x_lo1 = (float)(qx0 + 4), x_hi1 = (float)(qx0 + 7);
+    const float y_lo0 = (float)qy0, y_hi0 = (float)(qy0 + 3), y_lo1 = (float)(qy0 + 4), y_hi1 = (float)(qy0 + 7);
+    const uint64_t lanes_below = (1ull << lane) - 1ull;
 
     const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
     PixelState p = {inside ? 1.0f : -1.0f, 0.0f, 0.0f, 0.0f, 0.0f};
@@ -131,26 +142,42 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
         const int count = (int)min(256u, hi - base);
         if (!wave_done) {
             if (kCull) {
-                bool finished = false;
-                for (int chunk = 0; chunk < count && !finished; chunk += 64) {
+                // ---- lists: which staged Gaussians reach which 4x4 block (lane = Gaussian) ----
+                uint32_t len[4] = {0u, 0u, 0u, 0u};  // uniform over the wavefront
+                for (int chunk = 0; chunk < count; chunk += 64) {
                     const int k = chunk + lane;
-                    bool hit = false;
+                    bool in_x0 = false, in_x1 = false, in_y0 = false, in_y1 = false;
                     if (k < count) {
                         const float4 a = s_a[k];
                         const float4 c = s_c[k];
-                        hit = (a.x + c.z >= qx_lo) && (a.x - c.z <= qx_hi) && (a.y + c.w >= qy_lo) &&
-                              (a.y - c.w <= qy_hi);
+                        const float bx_lo = a.x - c.z, bx_hi = a.x + c.z, by_lo = a.y - c.w, by_hi = a.y + c.w;
+                        in_x0 = bx_hi >= x_lo0 && bx_lo <= x_hi0;
+                        in_x1 = bx_hi >= x_lo1 && bx_lo <= x_hi1;
+                        in_y0 = by_hi >= y_lo0 && by_lo <= y_hi0;
+                        in_y1 = by_hi >= y_lo1 && by_lo <= y_hi1;
                     }
-                    uint64_t todo = __ballot(hit);
-                    while (todo != 0ull) {
-                        const int kk = chunk + (int)__builtin_ctzll(todo);
-                        todo &= todo - 1ull;
-                        blend_one(p, pxf, pyf, s_a[kk], s_b[kk], s_c[kk]);
-                        if (__ballot(p.T > 0.0f) == 0ull) {
-                            finished = true;
-                            break;
-                        }
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const bool hit = ((b & 1) ? in_x1 : in_x0) && ((b >> 1) ? in_y1 : in_y0);
+                        const uint64_t m = __ballot(hit);
+                        if (hit) s_list[wave][b][len[b] + (uint32_t)__popcll(m & lanes_below)] = (uint8_t)k;
+                        len[b] += (uint32_t)__popcll(m);
                     }
+                }
+                // a wavefront's LDS operations execute in order: its list writes precede the reads below
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                // ---- the four lane groups walk their lists side by side ----
+                const uint32_t my_len = group == 0 ? len[0] : group == 1 ? len[1] : group == 2 ? len[2] : len[3];
+                const uint32_t longest = max(max(len[0], len[1]), max(len[2], len[3]));
+                const uint8_t* __restrict__ mine = s_list[wave][group];
+                uint32_t k_next = mine[0];  // read ahead by one entry (entries past the end are never used)
+                for (uint32_t i = 0; i < longest; ++i) {
+                    const uint32_t kk = k_next;
+                    k_next = mine[i + 1];
+                    if (i < my_len) blend_one(p, pxf, pyf, s_a[kk], s_b[kk], s_c[kk]);
+                    if (__ballot(p.T > 0.0f) == 0ull) break;
                 }
             } else {
                 for (int k = 0; k < count; ++k) {

@@ -27,7 +27,14 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of the heaviest kernels on the default workload (6M Gaussians, 1080p), from two
 # `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what
 # the same counter reads for the 1 GiB copy of --calibration-copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
-MEASURED_TRAFFIC_BYTES = {"blend": 1849.0e6, "preprocess": 1727.6e6}
+# "keys_sort_ranges" is the sum over the kernels of the tile count, scatter and tile sort stages.
+MEASURED_TRAFFIC_BYTES = {"blend": 1848.7e6, "preprocess": 1722.7e6, "keys_sort_ranges": 831.2e6}
+# (pixel, Gaussian) pairs of the default workload's blend, counted by the CPU checker (`python -m oracle.workload_stats 3`):
+# every list entry a pixel visits before it terminates / the pairs applied to a pixel (alpha >= 1/255).  Properties
+# of the seeded scene, not of a kernel; 25 flop per evaluated pair is the blend's algorithmic work.
+BLEND_PAIRS = {"evaluated": 1.612e9, "accepted": 1.001e8}
+# fp32 flops the blend kernel issues per launch on that workload (64 x (2 FMA + MUL + ADD) from a `rocprofv3 --pmc` run)
+BLEND_ISSUED_FLOPS = 11.12e9
 FP32_PEAK_TFLOPS = 157.3  # MI355X fp32 vector peak (packed FMA); this build issues unpacked FP32 only
 
 
@@ -45,6 +52,8 @@ def parse_args():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--two-in-flight", action="store_true",
+                    help="also time the frames with two in flight on alternating streams (reported beside `value`)")
     return ap.parse_args()
 
 
@@ -236,6 +245,23 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     fps = args.steps / elapsed
 
+    # the same frames with two in flight (alternating HIP streams, one workspace each): the next frame's
+    # HBM-bound preprocess overlaps the current frame's VALU-bound blend.  Reported beside `value`, never as it.
+    # Opt-in (--two-in-flight): overlapping kernels would distort the per-kernel durations of a profiler trace.
+    fps_two_in_flight = None
+    if args.two_in_flight:
+        streams = [torch.cuda.Stream(device=dev) for _ in range(2)]
+        for k in range(4):
+            with torch.cuda.stream(streams[k % 2]):
+                rast(**kwargs)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            with torch.cuda.stream(streams[k % 2]):
+                rast(**kwargs)
+        torch.cuda.synchronize()
+        fps_two_in_flight = round(args.steps / (time.perf_counter() - t0), 2)
+
     # model-level frame rate: the reference's forward sequence (visibility prefilter, gather of the survivors,
     # rasterize) and the fused single-pass variant that produces the same frame
     from landmarksystem_amd.models import GaussianModel
@@ -291,9 +317,18 @@ def main():
                                   "ranges_ms": round(stage_ms["ranges"], 4),
                                   "sort_GBps": round(work["sort"] / stage_ms["sort"] / 1e6, 1)}
     ms = stage_ms["blend"]
+    default_workload = args.config == 3 and not args.gaussians
     stages["blend"] = {"ms": round(ms, 4), "flops_upper": work["blend_flops"],
                        "TFLOPs_upper": round(work["blend_flops"] / ms / 1e9, 2),
                        "frac_fp32_upper": round(work["blend_flops"] / ms / 1e9 / FP32_PEAK_TFLOPS, 4)}
+    if default_workload:
+        flops = 25 * BLEND_PAIRS["evaluated"]
+        stages["blend"].update({
+            "pairs_evaluated": BLEND_PAIRS["evaluated"], "pairs_accepted": BLEND_PAIRS["accepted"],
+            "flops_algorithmic": flops, "TFLOPs_algorithmic": round(flops / ms / 1e9, 2),
+            "frac_fp32_algorithmic": round(flops / ms / 1e9 / FP32_PEAK_TFLOPS, 4),
+            "TFLOPs_issued": round(BLEND_ISSUED_FLOPS / ms / 1e9, 2),
+            "frac_fp32_issued": round(BLEND_ISSUED_FLOPS / ms / 1e9 / FP32_PEAK_TFLOPS, 4)})
     pre_sort_bytes = work["preprocess"] + sort_bytes
     pre_sort_ms = stage_ms["preprocess"] + sort_ms
     stages["preprocess_plus_sort"] = hbm("preprocess_plus_sort", pre_sort_ms, pre_sort_bytes)
@@ -302,16 +337,21 @@ def main():
                        "blend_frames_per_s": round(1e3 / stage_ms["blend"], 1)}
 
     # counter-measured traffic only applies to the workload it was measured on
-    traffic = MEASURED_TRAFFIC_BYTES if (args.config == 3 and not args.gaussians) else {}
+    traffic = MEASURED_TRAFFIC_BYTES if default_workload else {}
     shipped = {"preprocess": stage_ms["preprocess"], "keys_sort_ranges": sort_ms,
                "blend": stage_ms["blend"]}
     dominant = max(shipped, key=lambda n: shipped[n])
     if dominant == "blend":
-        roofline = {"bound": "mfma", "kernel": "blend_kernel", "achieved": stages["blend"]["TFLOPs_upper"],
-                    "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": stages["blend"]["frac_fp32_upper"],
+        kind = "algorithmic" if default_workload else "upper"
+        roofline = {"bound": "mfma", "kernel": "blend_kernel", "achieved": stages["blend"]["TFLOPs_" + kind],
+                    "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": stages["blend"]["frac_fp32_" + kind],
                     "traffic": traffic.get("blend"),
-                    "note": "FP32 VALU kernel (no MFMA); peak is the MI355X fp32 figure; flops = 25 x 256 x sum of "
-                            "tile range lengths (upper bound on evaluated pixel-Gaussian pairs)"}
+                    "note": "FP32 VALU kernel (no MFMA); peak is the MI355X fp32 vector figure (packed FMA; this build "
+                            "issues unpacked fp32, half of it).  flops = 25 x the (pixel, Gaussian) pairs the per-pixel "
+                            "loop evaluates" + (" (counted by the CPU checker for this seeded scene); the kernel skips "
+                            "pairs whose alpha is provably < 1/255, so it issues fewer flops than that: see "
+                            "stages.blend.TFLOPs_issued" if default_workload else
+                            ", bounded above by 256 x sum of tile range lengths")}
     else:
         roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": traffic.get(dominant)}
@@ -335,6 +375,7 @@ def main():
         "roofline": roofline,
         "stages": stages,
         "model_forward_frames_per_s": model_fps,
+        "two_frames_in_flight_frames_per_s": fps_two_in_flight,
     }
     if not args.no_cpu_baseline:
         try:

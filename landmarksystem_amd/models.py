@@ -101,7 +101,31 @@ class GaussianModel(nn.Module):
         self.register_buffer("background", torch.tensor([1.0, 1.0, 1.0] if white_bkgd else [0.0, 0.0, 0.0]))
         self.renderer = _placeholder_renderer(self.background)
         self._cache = {}
-        self.radii = self.visibility_filter = None
+        self._radii = self._visibility_filter = self._radii_all = None
+
+    # `visibility_filter` (bool[P]) and `radii` (int32 of the visible Gaussians) are by-products the reference
+    # leaves on the model for its training loop.  The fused single-pass frame derives them from the rasterizer's
+    # radii only when they are read, so a render loop that never looks at them pays nothing (the boolean-mask
+    # gather waits for the device).
+    @property
+    def visibility_filter(self):
+        if self._visibility_filter is None and self._radii_all is not None:
+            self._visibility_filter = self._radii_all > 0
+        return self._visibility_filter
+
+    @visibility_filter.setter
+    def visibility_filter(self, value):
+        self._visibility_filter = value
+
+    @property
+    def radii(self):
+        if self._radii is None and self._radii_all is not None:
+            self._radii = self._radii_all[self.visibility_filter]
+        return self._radii
+
+    @radii.setter
+    def radii(self, value):
+        self._radii = value
 
     @classmethod
     def from_activated(cls, means3D, scales, rotations, opacities, shs, **kw):
@@ -234,8 +258,7 @@ class GaussianModel(nn.Module):
             rendered_image, radii, _ = self.renderer(
                 means3D=means3D, means2D=None, shs=shs, colors_precomp=colors_precomp, opacities=opacity,
                 scales=scales, rotations=rotations, cov3D_precomp=cov3D_precomp)
-            self.visibility_filter = radii > 0
-            self.radii = radii[self.visibility_filter]
+            self._radii_all, self._radii, self._visibility_filter = radii, None, None
             return rendered_image
         if not self.training:  # the reference renders only what its prefilter kept (origin_gs/gs_model.py:199-208)
             mask = voxel_visible_mask.nonzero().squeeze(-1)
@@ -245,7 +268,7 @@ class GaussianModel(nn.Module):
         rendered_image, radii, _ = self.renderer(
             means3D=means3D, means2D=None, shs=shs, colors_precomp=colors_precomp, opacities=opacity, scales=scales,
             rotations=rotations, cov3D_precomp=cov3D_precomp)
-        self.visibility_filter, self.radii = voxel_visible_mask, radii
+        self._radii_all, self.visibility_filter, self.radii = None, voxel_visible_mask, radii
         return rendered_image
 
 
@@ -433,6 +456,7 @@ class OctreeGS(ScaffoldGS):
         self.voxel_size, self.standard_dist, self.fork = float(voxel_size), float(standard_dist), int(fork)
         self.enable_lod, self.dist2level = enable_lod, dist2level
         self._anchor_mask: Optional[torch.Tensor] = None
+        self._level_span = None  # (the level tensor it was computed from, max level - min level)
 
     def set_anchor_mask(self, cam_center, iteration, resolution_scale):
         """octreegs_encoding.py:238-264 in eval mode: keep anchors whose level does not exceed the level
@@ -443,14 +467,16 @@ class OctreeGS(ScaffoldGS):
         anchor_pos = self._anchor + (self.voxel_size / 2) / (float(self.fork) ** self._level)
         dist = torch.sqrt(torch.sum((anchor_pos - cam_center) ** 2, dim=1)) * resolution_scale
         pred_level = torch.log2(self.standard_dist / dist) / math.log2(self.fork) + self._extra_level
-        cur_level = torch.max(self._level) - torch.min(self._level)
+        if self._level_span is None or self._level_span[0] is not self._level:
+            # the span of the levels is a constant of the loaded model: read it back once, not per frame
+            self._level_span = (self._level, int((torch.max(self._level) - torch.min(self._level)).item()))
         if self.dist2level == "floor":
             int_level = torch.floor(pred_level).int()
         elif self.dist2level == "round":
             int_level = torch.round(pred_level).int()
         else:
             int_level = torch.ceil(pred_level).int()
-        int_level = torch.clamp(int_level, min=0, max=int(cur_level.item()))
+        int_level = torch.clamp(int_level, min=0, max=self._level_span[1])
         self._anchor_mask = self._level.squeeze(dim=1) <= int_level
 
     def get_state_dict_from_ckpt(self, file_path, map_location="cpu"):

@@ -12,9 +12,12 @@
 //
 // Everything is computed transposed so that the two layers chain without any
 // data movement: weights are the A operand (rows = output units), 32 anchors
-// are the columns of one v_mfma_f32_32x32x8_f16 tile, and the accumulator
-// layout of layer 1 (lane = anchor, registers = hidden units 8b+4*half+t) is
-// exactly the B-operand layout layer 2 needs.
+// are the columns of one v_mfma_f32_32x32x16_f16 tile (the gfx950 form: 16
+// k values per instruction, 8 per lane), and the accumulator layout of layer 1
+// (lane = anchor, registers = hidden units 8b+4*half+t) feeds layer 2's B
+// operand directly: which k value sits in which of a lane's 8 slots is free
+// as long as both operands agree, so the weights of layer 2 are simply loaded
+// in the order the accumulator registers come in.
 //
 // Precision: weights and anchor features are rounded to fp16 (exact for fp16
 // checkpoints); the four fp32-only inputs (view direction, distance) and the
@@ -31,7 +34,7 @@ namespace gs355 {
 
 namespace {
 
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kFeat = 32;
@@ -51,29 +54,28 @@ struct DecodeArgs {
     const float* b1[3];
 };
 
-__device__ __forceinline__ half4_t to_half4(float a, float b, float c, float d)
+__device__ __forceinline__ half8_t to_half8(const float v[8])
 {
-    half4_t h;
-    h[0] = (_Float16)a;
-    h[1] = (_Float16)b;
-    h[2] = (_Float16)c;
-    h[3] = (_Float16)d;
+    half8_t h;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) h[j] = (_Float16)v[j];
     return h;
 }
 
-// A fragment of a [rows x cols] row-major fp32 weight matrix for k-step s:
-// lane (row = lane % 32, half = lane / 32) holds W[row0 + row][8s + 4*half + 0..3].
-__device__ __forceinline__ half4_t weight_fragment(const float* __restrict__ w, int rows, int cols, int row, int k0)
+// Eight entries of row `row` of a [rows x cols] row-major fp32 weight matrix, as one lane's share of an A
+// operand: slots 0..3 hold columns ka..ka+3, slots 4..7 columns kb..kb+3 (zero outside the matrix).  Loads are
+// unconditional at clamped (in-range) positions and masked afterwards, so that none of them waits for another:
+// the fragments of a head are fetched with all loads in flight together.
+__device__ __forceinline__ half8_t weight_fragment(const float* __restrict__ w, int rows, int cols, int row, int ka,
+                                                   int kb, bool enable = true)
 {
-    // loads are unconditional at clamped (in-range) positions and masked afterwards, so that none of them
-    // waits for another: the fragments of a head are fetched with all loads in flight together
-    float v[4];
+    float v[8];
     const int r = min(row, rows - 1);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) v[t] = w[(size_t)r * cols + min(k0 + t, cols - 1)];
+    for (int j = 0; j < 8; ++j) v[j] = w[(size_t)r * cols + min((j < 4 ? ka : kb - 4) + j, cols - 1)];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) v[t] = (row < rows && k0 + t < cols) ? v[t] : 0.0f;
-    return to_half4(v[0], v[1], v[2], v[3]);
+    for (int j = 0; j < 8; ++j) v[j] = (enable && row < rows && (j < 4 ? ka : kb - 4) + j < cols) ? v[j] : 0.0f;
+    return to_half8(v);
 }
 
 // Bias for an accumulator: register v = 4b + t holds row 8b + 4*half + t.  `bias` is the head's bias vector
@@ -87,10 +89,15 @@ __device__ __forceinline__ floatx16 bias_rows(const float* bias, int row0, int h
 }
 
 // Weight fragments of one head, held in registers for the whole kernel.
+//   layer 1, k-steps 0 and 1: the 32 anchor features, slot j of half h <-> feature 16s + 8h + j
+//   layer 1, k-step 2:        the four fp32-only inputs twice on half 0 (slots 0..3 meet their hi parts, slots
+//                             4..7 their lo parts, both against W0[:, 32..35]); half 1 is zero
+//   layer 2, k-step s:        slot j of half h <-> hidden unit 16s + 4h + j (j < 4) or 16s + 8 + 4h + (j - 4),
+//                             the units held by accumulator registers 8s..8s+7 of that lane
 template <int kTiles>
 struct HeadWeights {
-    half4_t w0[5];          // layer 1: [32 x in], k-steps 0..4
-    half4_t w1[kTiles][4];  // layer 2: [outputs x 32] in row tiles of 32
+    half8_t w0[3];          // layer 1: [32 x in]
+    half8_t w1[kTiles][2];  // layer 2: [outputs x 32] in row tiles of 32
 };
 
 template <int kTiles>
@@ -99,51 +106,48 @@ __device__ __forceinline__ void load_head(const DecodeArgs& d, int head, int out
 {
     const int in = d.in_dim[head];
 #pragma unroll
-    for (int s = 0; s < 5; ++s) {
-        // k-step 4 carries the fp32-only inputs twice: hi parts on the low half of the lanes, lo parts on the
-        // high half, both against the same weights W0[:, 32..35]
-        const int k0 = s < 4 ? 8 * s + 4 * half : 32;
-        w.w0[s] = weight_fragment(d.w0[head], kFeat, in, row, k0);
-    }
+    for (int s = 0; s < 2; ++s) w.w0[s] = weight_fragment(d.w0[head], kFeat, in, row, 16 * s + 8 * half, 16 * s + 8 * half + 4);
+    w.w0[2] = weight_fragment(d.w0[head], kFeat, in, row, 32, 32, half == 0);
 #pragma unroll
     for (int r = 0; r < kTiles; ++r)
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
-            w.w1[r][s] = weight_fragment(d.w1[head], outputs, kFeat, 32 * r + row, 8 * s + 4 * half);
+        for (int s = 0; s < 2; ++s)
+            w.w1[r][s] = weight_fragment(d.w1[head], outputs, kFeat, 32 * r + row, 16 * s + 4 * half,
+                                         16 * s + 8 + 4 * half);
 }
 
 // One head for one tile of 32 anchors: returns up to kTiles accumulators of the
 // second layer (rows = outputs 32r + 8b + 4*half + t, column = this lane's anchor).
 template <int kTiles>
 __device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const float* bias0, const float* bias1,
-                                         const half4_t X[5], int half, floatx16 out[kTiles])
+                                         const half8_t X[3], int half, floatx16 out[kTiles])
 {
     // layer 1: hidden = W0 [32 x in] * X^T + b0
     floatx16 h = bias_rows(bias0, 0, half);
 #pragma unroll
-    for (int s = 0; s < 5; ++s) h = __builtin_amdgcn_mfma_f32_32x32x8f16(w.w0[s], X[s], h, 0, 0, 0);
-    // ReLU, then hi/lo split: registers 4s..4s+3 are the B operand of k-step s
-    half4_t hh[4], hl[4];
+    for (int s = 0; s < 3; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w0[s], X[s], h, 0, 0, 0);
+    // ReLU, then hi/lo split: registers 8s..8s+7 are the B operand of k-step s
+    half8_t hh[2], hl[2];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-        float r[4], lo[4];
+    for (int s = 0; s < 2; ++s) {
+        float r[8], lo[8];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            r[t] = fmaxf(h[4 * s + t], 0.0f);
-            const _Float16 top = (_Float16)r[t];
-            lo[t] = r[t] - (float)top;
+        for (int j = 0; j < 8; ++j) {
+            r[j] = fmaxf(h[8 * s + j], 0.0f);
+            const _Float16 top = (_Float16)r[j];
+            lo[j] = r[j] - (float)top;
         }
-        hh[s] = to_half4(r[0], r[1], r[2], r[3]);
-        hl[s] = to_half4(lo[0], lo[1], lo[2], lo[3]);
+        hh[s] = to_half8(r);
+        hl[s] = to_half8(lo);
     }
     // layer 2: out = W1 [outputs x 32] * hidden + b1
 #pragma unroll
     for (int r = 0; r < kTiles; ++r) {
         floatx16 c = bias_rows(bias1, 32 * r, half);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            c = __builtin_amdgcn_mfma_f32_32x32x8f16(w.w1[r][s], hh[s], c, 0, 0, 0);
-            c = __builtin_amdgcn_mfma_f32_32x32x8f16(w.w1[r][s], hl[s], c, 0, 0, 0);
+        for (int s = 0; s < 2; ++s) {
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w1[r][s], hh[s], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w1[r][s], hl[s], c, 0, 0, 0);
         }
         out[r] = c;
     }
@@ -163,7 +167,7 @@ __device__ __forceinline__ void store_rows(float* __restrict__ dst_anchor, int b
 // Per-lane inputs of one tile of 32 anchors.
 template <bool kCountOnly>
 struct TileInputs {
-    float4 f[4] = {};          // features 8s + 4*half .. +3, s = 0..3
+    float4 f[4] = {};          // features 16s + 8*half .. +7 in f[2s], f[2s+1], s = 0..1
     float pos[3] = {0.f, 0.f, 0.f};
     float sc3[3] = {0.f, 0.f, 0.f};
     uint32_t first_slot = 0;
@@ -227,7 +231,10 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         if (vis) {
             const float4* __restrict__ f4 = reinterpret_cast<const float4*>(d.feat + (size_t)a * kFeat);
 #pragma unroll
-            for (int s = 0; s < 4; ++s) in.f[s] = f4[2 * s + half];
+            for (int s = 0; s < 2; ++s) {  // features 16s + 8*half .. +7
+                in.f[2 * s] = f4[4 * s + 2 * half];
+                in.f[2 * s + 1] = f4[4 * s + 2 * half + 1];
+            }
 #pragma unroll
             for (int k = 0; k < 3; ++k) in.pos[k] = d.anchor[3 * (size_t)a + k];
         }
@@ -249,28 +256,34 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
                 for (int k = 0; k < 3; ++k) in.ofv[r][k] = want ? of[k] : 0.0f;
             }
         }
-        // B operand: X^T, column = anchor, k = 8s + 4*half + t
-        half4_t X[5];
+        // B operand: X^T, column = anchor; slots as described at HeadWeights
+        half8_t X[3];
         const float ax = in.pos[0], ay = in.pos[1], az = in.pos[2];
-        if (vis) {
+        {
+            float x8[8];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) X[s] = to_half4(in.f[s].x, in.f[s].y, in.f[s].z, in.f[s].w);
-            float vx = ax - cx, vy = ay - cy, vz = az - cz;
-            const float dist = sqrtf(vx * vx + vy * vy + vz * vz);
-            vx /= dist;
-            vy /= dist;
-            vz /= dist;
-            const float in4[4] = {vx, vy, vz, dist};
-            float part[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const _Float16 top = (_Float16)in4[t];
-                part[t] = half ? in4[t] - (float)top : (float)top;
+            for (int s = 0; s < 2; ++s) {
+                x8[0] = in.f[2 * s].x, x8[1] = in.f[2 * s].y, x8[2] = in.f[2 * s].z, x8[3] = in.f[2 * s].w;
+                x8[4] = in.f[2 * s + 1].x, x8[5] = in.f[2 * s + 1].y, x8[6] = in.f[2 * s + 1].z, x8[7] = in.f[2 * s + 1].w;
+                X[s] = to_half8(x8);  // all zero for an invisible anchor
             }
-            X[4] = to_half4(part[0], part[1], part[2], part[3]);
-        } else {
 #pragma unroll
-            for (int s = 0; s < 5; ++s) X[s] = to_half4(0.f, 0.f, 0.f, 0.f);
+            for (int j = 0; j < 8; ++j) x8[j] = 0.0f;
+            if (vis && half == 0) {
+                float vx = ax - cx, vy = ay - cy, vz = az - cz;
+                const float dist = sqrtf(vx * vx + vy * vy + vz * vz);
+                vx /= dist;
+                vy /= dist;
+                vz /= dist;
+                const float in4[4] = {vx, vy, vz, dist};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const _Float16 top = (_Float16)in4[t];
+                    x8[t] = (float)top;
+                    x8[4 + t] = in4[t] - (float)top;
+                }
+            }
+            X[2] = to_half8(x8);
         }
 
         // ---- opacity head ----

@@ -264,17 +264,21 @@ def main():
 
     # model-level frame rate: the reference's forward sequence (visibility prefilter, gather of the survivors,
     # rasterize) and the fused single-pass variant that produces the same frame
-    from landmarksystem_amd.models import GaussianModel
+    # (third variant: the same scene stored along a Morton curve, a load-time option of the checkpoint loaders)
+    from landmarksystem_amd.models import GaussianModel, morton_order
     model_fps = {}
-    for name, fuse in (("reference_sequence", False), ("fused_prefilter", True)):
-        model = GaussianModel(d.means3D, d.shs[:, :1].contiguous(), d.shs[:, 1:].contiguous(), torch.log(d.scales),
-                              d.rotations, torch.logit(d.opacities.clamp(1e-6, 1 - 1e-6)), sh_degree=scene.sh_degree,
+    for name, fuse, ordered in (("reference_sequence", False, False), ("fused_prefilter", True, False),
+                                ("fused_prefilter_spatial_order", True, True)):
+        pick = morton_order(d.means3D) if ordered else slice(None)
+        model = GaussianModel(d.means3D[pick], d.shs[pick][:, :1].contiguous(), d.shs[pick][:, 1:].contiguous(),
+                              torch.log(d.scales[pick]), d.rotations[pick],
+                              torch.logit(d.opacities[pick].clamp(1e-6, 1 - 1e-6)), sh_degree=scene.sh_degree,
                               act_cache=True, fuse_prefilter=fuse).eval()
         for _ in range(5):
             model(scene.camera)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        n_model = max(10, args.steps // 4)
+        n_model = max(20, args.steps // 2)
         for _ in range(n_model):
             model(scene.camera)
         torch.cuda.synchronize()

@@ -286,10 +286,24 @@ def _decoder_kwargs(dec: Mapping[str, torch.Tensor], n_offsets: int, feat_dim: i
     return out
 
 
-def load_gaussian_model(path, sh_degree: int = 3, device="cuda", **kw):
-    """`GaussianModel` from a checkpoint directory or a PLY file."""
+def _reorder(state: Dict[str, torch.Tensor], positions: str) -> None:
+    """Store the per-Gaussian / per-anchor tensors along a Morton curve of their positions (see
+    `models.morton_order`): same scene, memory-coherent frames.  Indices of by-products then refer to this order."""
+    from .models import morton_order
+    order = morton_order(state[positions])
+    n = order.shape[0]
+    for k, v in state.items():
+        if torch.is_tensor(v) and v.dim() >= 1 and v.shape[0] == n:
+            state[k] = v[order].contiguous()
+
+
+def load_gaussian_model(path, sh_degree: int = 3, device="cuda", spatial_order: bool = False, **kw):
+    """`GaussianModel` from a checkpoint directory or a PLY file.  `spatial_order` stores the Gaussians along a
+    Morton curve instead of in file order."""
     from .models import GaussianModel
     s = gaussian_state_dict(_ply_in(path), sh_degree, device)
+    if spatial_order:
+        _reorder(s, "_xyz")
     if "_cache_opacity" in s:
         return GaussianModel.from_cache(s["_xyz"], s["_cache_features"], s["_cache_scaling"], s["_cache_rotation"],
                                         s["_cache_opacity"], sh_degree=sh_degree, **kw)
@@ -297,11 +311,13 @@ def load_gaussian_model(path, sh_degree: int = 3, device="cuda", **kw):
                          s["_opacity"], sh_degree=sh_degree, **kw)
 
 
-def load_scaffold_gs(path, device="cuda", **kw):
+def load_scaffold_gs(path, device="cuda", spatial_order: bool = False, **kw):
     """`ScaffoldGS` from a checkpoint directory (`point_cloud.ply` + `state_dict.th`)."""
     from .models import ScaffoldGS
     ply = _ply_in(path)
     s = scaffold_state_dict(ply, device)
+    if spatial_order:
+        _reorder(s, "_anchor")
     dec = _decoder_state(load_mlp_state(os.path.dirname(os.path.abspath(ply)), device))
     n_offsets, feat_dim = s["_offset"].shape[1], s["_anchor_feat"].shape[1]
     kw = {**_decoder_kwargs(dec, n_offsets, feat_dim), **kw}
@@ -312,11 +328,13 @@ def load_scaffold_gs(path, device="cuda", **kw):
     return m.to(device)
 
 
-def load_octree_gs(path, device="cuda", **kw):
+def load_octree_gs(path, device="cuda", spatial_order: bool = False, **kw):
     """`OctreeGS` from a checkpoint directory (`point_cloud.ply` + `state_dict.th`)."""
     from .models import OctreeGS
     ply = _ply_in(path)
     s, voxel_size, standard_dist = octree_state_dict(ply, device)
+    if spatial_order:
+        _reorder(s, "_anchor")
     dec = _decoder_state(load_mlp_state(os.path.dirname(os.path.abspath(ply)), device))
     n_offsets, feat_dim = s["_offset"].shape[1], s["_anchor_feat"].shape[1]
     kw = {**_decoder_kwargs(dec, n_offsets, feat_dim), **kw}

@@ -56,6 +56,33 @@ def _split_prefix(state_dict, prefix):
     return picked
 
 
+def morton_order(xyz: torch.Tensor) -> torch.Tensor:
+    """Permutation that sorts points along a 3-D Morton (Z-order) curve: 21 bits per axis on a common scale,
+    interleaved x, y, z from the most significant bit down.
+
+    Storing a scene in this order is a load-time choice.  The rasterizer orders by depth, so a frame changes only
+    where two Gaussians of exactly equal fp32 depth share a pixel (ties blend in index order, as in the reference;
+    the effect is of the order of 1e-4 on isolated pixels).  It makes the memory traffic of a frame coherent:
+    Gaussians that land in the same screen tile sit near each other in memory, so culled stretches skip whole
+    wavefronts, bucket writes of one slice of the scene fall into few tiles, and the blend's record gathers hit
+    lines that are already in cache."""
+    p = xyz.detach().double()
+    lo = p.min(dim=0).values
+    span = float((p.max(dim=0).values - lo).max())
+    q = ((p - lo) / (span if span > 0 else 1.0) * float((1 << 21) - 1)).long().clamp_(0, (1 << 21) - 1)
+
+    def spread(v):  # 21 bits -> every third bit of 63
+        v = (v | (v << 32)) & 0x1F00000000FFFF
+        v = (v | (v << 16)) & 0x1F0000FF0000FF
+        v = (v | (v << 8)) & 0x100F00F00F00F00F
+        v = (v | (v << 4)) & 0x10C30C30C30C30C3
+        v = (v | (v << 2)) & 0x1249249249249249
+        return v
+
+    code = (spread(q[:, 0]) << 2) | (spread(q[:, 1]) << 1) | spread(q[:, 2])
+    return torch.sort(code, stable=True).indices
+
+
 def _placeholder_renderer(bg):
     # the reference builds its renderer once with empty placeholders (origin_gs/gs_model.py:82-97)
     return GaussianRasterizer(raster_settings=GaussianRasterizationSettings(

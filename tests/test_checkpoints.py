@@ -264,3 +264,47 @@ def test_merged_state_dict_rejects_duplicates(tmp_path):
     torch.save({"gaussian_encoding._anchor": torch.zeros(1)}, tmp_path / "state_dict.th")
     with pytest.raises(ValueError, match="Duplicate keys found"):
         ck.merged_state_dict(tmp_path / "point_cloud.ply", "scaffold")
+
+
+def test_morton_order_against_bitwise_interleaving():
+    from landmarksystem_amd.models import morton_order
+    g = torch.Generator().manual_seed(0)
+    p = torch.rand(1500, 3, generator=g) * torch.tensor([10.0, 4.0, 1.0]) - 3.0
+    order = morton_order(p)
+    assert sorted(order.tolist()) == list(range(1500))
+    lo = p.double().min(0).values
+    span = float((p.double().max(0).values - lo).max())
+    q = ((p.double() - lo) / span * ((1 << 21) - 1)).long()
+
+    def interleave(x, y, z):  # bit b of x, y, z -> bits 3b+2, 3b+1, 3b
+        c = 0
+        for b in range(21):
+            c |= ((x >> b) & 1) << (3 * b + 2) | ((y >> b) & 1) << (3 * b + 1) | ((z >> b) & 1) << (3 * b)
+        return c
+
+    codes = np.array([interleave(*map(int, q[i])) for i in range(1500)], dtype=np.uint64)
+    assert np.array_equal(np.argsort(codes, kind="stable"), order.numpy())
+    assert morton_order(torch.zeros(5, 3)).tolist() == [0, 1, 2, 3, 4]  # degenerate extent: stable identity
+
+
+def test_spatial_order_loads_the_same_scene_in_another_order(tmp_path):
+    g = torch.Generator().manual_seed(8)
+    v = GaussianModel(torch.randn(40, 3, generator=g), torch.randn(40, 1, 3, generator=g),
+                      torch.randn(40, 15, 3, generator=g), torch.randn(40, 3, generator=g),
+                      torch.randn(40, 4, generator=g), torch.randn(40, 1, generator=g))
+    ck.save_model(v, tmp_path / "v")
+    a = ck.load_gaussian_model(tmp_path / "v", device="cpu")
+    b = ck.load_gaussian_model(tmp_path / "v", device="cpu", spatial_order=True)
+    from landmarksystem_amd.models import morton_order
+    order = morton_order(a._xyz)
+    assert not torch.equal(order, torch.arange(40))
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        assert torch.equal(pa[order], pb)
+    level = torch.arange(12) % 3
+    o = OctreeGS(*_random_anchor_args(12, 10, g), level, 0.3, 9.0, extra_level=torch.randn(12, generator=g))
+    ck.save_model(o, tmp_path / "o")
+    oa = ck.load_octree_gs(tmp_path / "o", device="cpu")
+    ob = ck.load_octree_gs(tmp_path / "o", device="cpu", spatial_order=True)
+    order = morton_order(oa._anchor)
+    assert torch.equal(oa._level[order], ob._level) and torch.equal(oa._extra_level[order], ob._extra_level)
+    assert torch.equal(oa._offset[order], ob._offset) and torch.equal(oa._anchor[order], ob._anchor)

@@ -106,19 +106,19 @@ __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P
 
 // Thread per tile: exclusive prefix of the tile's counts over the slices (in
 // place) and the tile's total.
-__global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict__ matrix, int groups, int tiles,
+__global__ __launch_bounds__(64) void slice_prefix_kernel(uint32_t* __restrict__ matrix, int groups, int tiles,
                                                            uint32_t* __restrict__ totals)
 {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= tiles) return;
     uint32_t run = 0;
     int c = 0;
-    for (; c + 8 <= groups; c += 8) {
-        uint32_t v[8];
+    for (; c + 32 <= groups; c += 32) {  // 32 independent loads in flight per thread
+        uint32_t v[32];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) v[k] = matrix[(size_t)(c + k) * tiles + t];
+        for (int k = 0; k < 32; ++k) v[k] = matrix[(size_t)(c + k) * tiles + t];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < 32; ++k) {
             matrix[(size_t)(c + k) * tiles + t] = run;
             run += v[k];
         }
@@ -141,71 +141,67 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
                                                            uint32_t* __restrict__ lists)
 {
     __shared__ uint64_t s_wave[16];
-    __shared__ uint64_t s_carry;
     __shared__ uint32_t s_nlist[4], s_vis;
     if (threadIdx.x == 0) {
-        s_carry = 0;
         s_nlist[0] = s_nlist[1] = s_nlist[2] = s_nlist[3] = 0;
         s_vis = 0;
     }
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    // pass 1: grand total (decides overflow before any range is published)
+    // Every thread owns a run of consecutive tiles, so one scan over the 1024 run sums (one barrier) places
+    // them all.  The grand total decides overflow before any range is published.
+    const uint32_t per = (tiles + 1023u) / 1024u;
+    const uint32_t t0 = min(threadIdx.x * per, tiles), t1 = min(t0 + per, tiles);
     uint64_t mine = 0;
-    for (uint32_t t = threadIdx.x; t < tiles; t += 1024) mine += totals[t];
+    for (uint32_t t = t0; t < t1; t += 8) {  // 8 loads in flight (the last batch re-reads the run's last tile)
+        uint32_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = totals[min(t + k, t1 - 1)];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) mine += t + k < t1 ? v[k] : 0u;
+    }
     uint32_t vis = 0;
     for (int c = threadIdx.x; c < groups; c += 1024) vis += group_visible[c];
+    uint64_t inc = mine;
 #pragma unroll
-    for (int d = 32; d > 0; d >>= 1) {
-        mine += __shfl_down(mine, d, 64);
-        vis += __shfl_down(vis, d, 64);
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint64_t up = __shfl_up(inc, d, 64);
+        if (lane >= d) inc += up;
     }
-    if (lane == 0) {
-        s_wave[wave] = mine;
-        if (vis) atomicAdd(&s_vis, vis);
-    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) vis += __shfl_down(vis, d, 64);
+    if (lane == 63) s_wave[wave] = inc;
+    if (lane == 0 && vis) atomicAdd(&s_vis, vis);
     __syncthreads();
-    uint64_t total = 0;
-    for (int w = 0; w < 16; ++w) total += s_wave[w];
+    uint64_t total = 0, before = 0;
+    for (int w = 0; w < 16; ++w) {
+        if (w < wave) before += s_wave[w];
+        total += s_wave[w];
+    }
     const bool overflow = total > (uint64_t)n_cap;
-    __syncthreads();
     if (threadIdx.x == 0) {
         header->num_keys_total = total;
         header->num_keys = overflow ? n_cap : (uint32_t)total;
         header->overflow = overflow ? 1u : 0u;
         header->num_visible = s_vis;
     }
-    // pass 2: exclusive scan of the totals (skipped on overflow: later stages do nothing then)
-    for (uint32_t base = 0; base < tiles && !overflow; base += 1024) {
-        const uint32_t t = base + threadIdx.x;
-        const uint32_t v = t < tiles ? totals[t] : 0u;
-        uint64_t inc = v;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const uint64_t up = __shfl_up(inc, d, 64);
-            if (lane >= d) inc += up;
-        }
-        if (lane == 63) s_wave[wave] = inc;
-        __syncthreads();
-        uint64_t off = s_carry;
-        for (int w = 0; w < wave; ++w) off += s_wave[w];
-        const uint32_t first = (uint32_t)(off + inc - v);
-        if (t < tiles) {
-            ranges[2 * t] = v ? first : 0u;
-            ranges[2 * t + 1] = v ? first + v : 0u;
-            tile_base[t] = first;
-            // buckets beyond the smallest sorter's capacity go on the list of their size class
-            int cls = -1;
-            if (v > (uint32_t)kTileSortCap[3]) cls = 3;
-            else if (v > (uint32_t)kTileSortCap[2]) cls = 2;
-            else if (v > (uint32_t)kTileSortCap[1]) cls = 1;
-            else if (v > (uint32_t)kTileSortCap[0]) cls = 0;
-            if (cls >= 0) lists[4 + (size_t)cls * tiles + atomicAdd(&s_nlist[cls], 1u)] = t;
-        }
-        __syncthreads();
-        if (threadIdx.x == 1023) s_carry = off + inc;
-        __syncthreads();
+    // bases, ranges and size-class lists of the thread's own tiles (skipped on overflow: later stages do nothing)
+    uint32_t first = (uint32_t)(before + inc - mine);
+    for (uint32_t t = t0; t < t1 && !overflow; ++t) {
+        const uint32_t v = totals[t];  // read before tile_base[t] (possibly the same word) is written
+        ranges[2 * t] = v ? first : 0u;
+        ranges[2 * t + 1] = v ? first + v : 0u;
+        tile_base[t] = first;
+        // buckets beyond the smallest sorter's capacity go on the list of their size class
+        int cls = -1;
+        if (v > (uint32_t)kTileSortCap[3]) cls = 3;
+        else if (v > (uint32_t)kTileSortCap[2]) cls = 2;
+        else if (v > (uint32_t)kTileSortCap[1]) cls = 1;
+        else if (v > (uint32_t)kTileSortCap[0]) cls = 0;
+        if (cls >= 0) lists[4 + (size_t)cls * tiles + atomicAdd(&s_nlist[cls], 1u)] = t;
+        first += v;
     }
+    __syncthreads();
     if (threadIdx.x < 4) lists[threadIdx.x] = s_nlist[threadIdx.x];
 }
 
@@ -861,7 +857,7 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
-    hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 255) / 256), dim3(256), 0, s, matrix, groups, tiles,
+    hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(64), 0, s, matrix, groups, tiles,
                        tile_base);
     GS355_CHECK_LAUNCH("bin: slice prefix");
     hipLaunchKernelGGL(tile_layout_kernel, dim3(1), dim3(1024), 0, s, tile_base, (uint32_t)tiles, group_visible, groups,

@@ -165,9 +165,7 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
                     }
                 }
                 // a wavefront's LDS operations execute in order: its list writes precede the reads below
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                wave_lds_sync();
                 // ---- the four lane groups walk their lists side by side ----
                 const uint32_t my_len = group == 0 ? len[0] : group == 1 ? len[1] : group == 2 ? len[2] : len[3];
                 const uint32_t longest = max(max(len[0], len[1]), max(len[2], len[3]));

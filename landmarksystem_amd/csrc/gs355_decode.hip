@@ -293,14 +293,14 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         // smallest floats), so tanh itself is only evaluated for the offsets that are kept
         store_rows(mine + col * stride, 0, n, 0, half, op[0]);
         if (kCountOnly) {
-            __builtin_amdgcn_wave_barrier();
+            wave_lds_sync();
             if (half == 0 && a < d.A) {
                 uint32_t kept = 0;
                 if (vis)
                     for (int m = 0; m < n; ++m) kept += mine[col * stride + m] > 0.0f ? 1u : 0u;
                 counts[a] = kept;
             }
-            __builtin_amdgcn_wave_barrier();
+            wave_lds_sync();
             continue;
         }
 
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
                 reinterpret_cast<uint32_t*>(extra)[9] = in.first_slot;
             }
         }
-        __builtin_amdgcn_wave_barrier();
+        wave_lds_sync();
 
         // ---- compact the kept (anchor, offset) items of the tile: about one in five survives the mask, and the
         // activations below are the expensive part, so they run on dense wavefronts of survivors only ----
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
             if (kept) list[total + (uint32_t)__popcll(b & lanes_below)] = (uint16_t)it;
             total += (uint32_t)__popcll(b);
         }
-        __builtin_amdgcn_wave_barrier();
+        wave_lds_sync();
 
         // Items are numbered anchor-major and the slots come from an exclusive scan of the per-anchor counts, so
         // the survivors of a tile occupy consecutive output slots from the slot of its first anchor: lanes write
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
             rot[4 * (size_t)pos + 2] = q2 / norm;
             rot[4 * (size_t)pos + 3] = q3 / norm;
         }
-        __builtin_amdgcn_wave_barrier();
+        wave_lds_sync();
     }
 }
 

@@ -78,6 +78,16 @@ int launch_ranges(const gs355_header* header, uint32_t n_cap, const uint64_t* ke
 int launch_blend(const FrameArgs& f, const gs355_header* header, const uint32_t* ranges, const uint32_t* values, const float* records,
                  float* image, float* depth, float* alpha, bool cull, hipStream_t s);
 
+// Orders one wavefront's LDS writes before its later LDS reads (and the reverse).  The hardware executes a
+// wavefront's LDS instructions in order; the fences (wavefront scope: no instructions) and the scheduling
+// barrier keep the compiler from moving the accesses across this point.
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 int launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t s);
 
 // tile-bucketed path

@@ -115,15 +115,6 @@ constexpr int kShChunk = 16 / kShRounds;                                   // co
 constexpr int kShChunk4 = kShChunk * 3 / 4;                                // float4s per Gaussian per round
 constexpr int kShStride = kShChunk * 3 + ((kShChunk * 3) % 8 == 0 ? 4 : 0);  // floats per Gaussian in LDS
 
-// Orders one wavefront's LDS writes before its later LDS reads (and the reverse): the hardware executes a
-// wavefront's LDS instructions in order, this keeps the compiler from moving them across.
-__device__ __forceinline__ void wave_lds_sync()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 template <int kRound>
 __device__ __forceinline__ void sh_staged_rounds(float4* __restrict__ mine, const float4* __restrict__ src, int count,
                                                  int lane, bool alive, int terms, const float b[16], float res[3])

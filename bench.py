@@ -175,6 +175,32 @@ def bench_scaffold(args, torch, dev):
         model(cam)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    # the same frames with the one-kernel anchor prefilter, and an Octree-GS model over the same anchors (random
+    # levels 0..4) with the reference's level-of-detail sequence and with the fused prefilter
+    from landmarksystem_amd.models import OctreeGS
+    variants = {}
+    level = torch.randint(0, 5, (scene.anchor.shape[0],), generator=torch.Generator().manual_seed(5))
+    for name, make in (
+        ("scaffold_fused_prefilter", lambda: ScaffoldGS.from_scene(scene, act_cache=True, fuse_prefilter=True)),
+        ("octree_reference_sequence", lambda: OctreeGS(
+            scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
+            voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True)),
+        ("octree_fused_prefilter", lambda: OctreeGS(
+            scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
+            voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True, fuse_prefilter=True)),
+    ):
+        other = make()
+        other.anchor_decoder.load_state_dict(model.anchor_decoder.state_dict())
+        other = other.to(dev).eval()
+        for _ in range(5):
+            other(cam)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            other(cam)
+        torch.cuda.synchronize()
+        variants[name] = round(args.steps / (time.perf_counter() - t1), 2)
+        del other
     # decode alone, HIP events on the launch stream
     vis = model.voxel_visible_mask
     dec_args = dict(camera_center=cam.camera_center, anchor=model.get_anchor, anchor_feat=model.get_anchor_feat,
@@ -196,6 +222,7 @@ def bench_scaffold(args, torch, dev):
         "vs_baseline": None, "dtype": "f16 matrix inputs (hi+lo pairs), f32 accumulate", "data": "synthetic",
         "config": {"workload": "configs[4]: %d anchors x %d offsets, 1920x1080" % (scene.anchor.shape[0], scene.n_offsets),
                    "visible_anchors": a_vis, "decoded_gaussians": G},
+        "model_variants_frames_per_s": variants,
         "decode": {"ms": round(dec_ms, 4), "anchors_per_s": round(a_vis / dec_ms * 1e3), "flops": flops,
                    "TFLOPs": round(flops / dec_ms / 1e9, 3), "frac_mfma_f16": round(flops / dec_ms / 1e9 / 2500.0, 6),
                    "bytes": nbytes, "GBps": round(nbytes / dec_ms / 1e6, 1),

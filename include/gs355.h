@@ -15,6 +15,8 @@
  *   GaussianRasterizer.visible_filter(...)  -> gs355_visible_filter
  *       call sites: origin_gs/gs_model.py:327-329, scaffold_gs/gs_model.py:
  *                   432-434, octree_gs/gs_model.py:491-493
+ *   ScaffoldGS / OctreeGS.prefilter_voxel   -> gs355_anchor_filter (one pass for the models' own sequence)
+ *       call sites: scaffold_gs/gs_model.py:385-436, octree_gs/gs_model.py:445-497
  *   GaussianRasterizationSettings(...)      -> gs355_frame
  *       built at:   origin_gs/gs_model.py:148-161 (and the two siblings)
  *
@@ -175,6 +177,30 @@ GS355_API int gs355_render(const gs355_frame *frame, const gs355_gaussians *g, v
  * non-empty tile rectangle); needs no workspace.  shs/colors/opacities of
  * `g` are ignored and may be NULL. */
 GS355_API int gs355_visible_filter(const gs355_frame *frame, const gs355_gaussians *g, int32_t *radii, void *stream);
+
+/* Level-of-detail selection of Octree-GS anchors in eval mode (OctreeGSEncoding.set_anchor_mask,
+ * landmark/nerf_components/model_components/fields/encodings/octreegs_encoding.py:238-264): an anchor is
+ * kept when  level <= clamp(R(log2(standard_dist / dist) / log2(fork) + extra_level), 0, max_level),
+ * dist = |anchor + (voxel_size / 2) / fork^level - campos| * resolution_scale, R = floor / round-half-even / ceil. */
+typedef struct gs355_anchor_lod {
+    const float *level;       /* f32[A] */
+    const float *extra_level; /* f32[A] */
+    float voxel_size, standard_dist, fork, resolution_scale;
+    int32_t rounding;  /* 0 floor, 1 round, 2 ceil (the reference's dist2level) */
+    int32_t max_level; /* max(level) - min(level) */
+} gs355_anchor_lod;
+
+/* The anchor-level visibility prefilter of the Scaffold-GS / Octree-GS models as one pass
+ * (scaffold_gs/gs_model.py:385-436; octree_gs/gs_model.py:216-218,445-497): optional level-of-detail mask,
+ * then GaussianRasterizer.visible_filter on the anchors that passed it, thresholded (> 0).  Produces what the
+ * models' own sequence of calls produces, without gathering the selected anchors and scattering the result
+ * back.  `anchors`: P = number of anchors, means3D, rotations and scales, of which the first three columns of
+ * rows `scale_stride` floats apart are used (3 for f32[A,3], 6 for the models' f32[A,6]); cov3D_precomp instead
+ * of scales / rotations is accepted as in gs355_visible_filter.  `lod` NULL: every anchor passes (Scaffold-GS).
+ * Outputs: visible u8[A] (required); lod_mask u8[A] and radii i32[A] (0 for anchors outside the mask) optional. */
+GS355_API int gs355_anchor_filter(const gs355_frame *frame, const gs355_gaussians *anchors, int32_t scale_stride,
+                                  const gs355_anchor_lod *lod, uint8_t *lod_mask, uint8_t *visible, int32_t *radii,
+                                  void *stream);
 
 /* ---------------------------------------------------------------------------
  * Anchor decode for Scaffold-GS / Octree-GS: replaces AnchorDecoder.forward in eval mode

@@ -19,7 +19,8 @@ PIPELINE_FAST = STAGE_PREPROCESS | STAGE_TILE_COUNT | STAGE_TILE_SCATTER | STAGE
 MAX_FAST_TILES = 36000
 
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
-           "gs355_visible_filter", "gs355_decode_scratch_bytes", "gs355_decode_count", "gs355_decode_emit")
+           "gs355_visible_filter", "gs355_anchor_filter", "gs355_decode_scratch_bytes", "gs355_decode_count",
+           "gs355_decode_emit")
 
 
 class Frame(C.Structure):
@@ -119,6 +120,12 @@ class Decoded(C.Structure):
                 ("rot", C.c_void_p)]
 
 
+class AnchorLod(C.Structure):
+    _fields_ = [("level", C.c_void_p), ("extra_level", C.c_void_p), ("voxel_size", C.c_float),
+                ("standard_dist", C.c_float), ("fork", C.c_float), ("resolution_scale", C.c_float),
+                ("rounding", C.c_int32), ("max_level", C.c_int32)]
+
+
 class Gs355Error(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__("gs355 error %d: %s" % (code, message))
@@ -151,6 +158,9 @@ def load() -> C.CDLL:
     lib.gs355_render.restype = C.c_int
     lib.gs355_visible_filter.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_void_p, C.c_void_p]
     lib.gs355_visible_filter.restype = C.c_int
+    lib.gs355_anchor_filter.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_int32, C.POINTER(AnchorLod),
+                                        C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.gs355_anchor_filter.restype = C.c_int
     lib.gs355_decode_scratch_bytes.argtypes = [C.c_int32, C.POINTER(C.c_size_t)]
     lib.gs355_decode_scratch_bytes.restype = C.c_int
     lib.gs355_decode_count.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_void_p, C.c_void_p,

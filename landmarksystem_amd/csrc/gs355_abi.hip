@@ -3,6 +3,7 @@
 // call sites: benchmarks/nerf/origin_gs/gs_model.py:211-220, 327-329).
 // Validation runs before any HIP call so that error paths are testable on a
 // machine without a GPU.
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -276,6 +277,34 @@ int gs355_visible_filter(const gs355_frame* frame, const gs355_gaussians* g, int
     if (g->P > 0 && !radii) return set_error(GS355_EINVAL, "radii is NULL");
     const FrameArgs fa = make_args(frame);
     return launch_preprocess(fa, *g, true, nullptr, nullptr, nullptr, nullptr, radii, static_cast<hipStream_t>(stream));
+}
+
+int gs355_anchor_filter(const gs355_frame* frame, const gs355_gaussians* anchors, int32_t scale_stride,
+                        const gs355_anchor_lod* lod, uint8_t* lod_mask, uint8_t* visible, int32_t* radii, void* stream)
+{
+    int rc;
+    if ((rc = check_frame(frame, false))) return rc;
+    if ((rc = check_geometry_inputs(anchors))) return rc;
+    if (scale_stride < 3) return set_error(GS355_EINVAL, "scale_stride must be >= 3 (got %d)", scale_stride);
+    if (anchors->P > 0 && !visible) return set_error(GS355_EINVAL, "visible is NULL");
+    FilterArgs x;
+    x.scale_stride = scale_stride;
+    x.visible = visible;
+    if (lod) {
+        if (anchors->P > 0 && (!lod->level || !lod->extra_level))
+            return set_error(GS355_EINVAL, "lod: level / extra_level is NULL");
+        if (lod->rounding < 0 || lod->rounding > 2)
+            return set_error(GS355_EINVAL, "lod: rounding must be 0 (floor), 1 (round) or 2 (ceil), got %d", lod->rounding);
+        if (!frame->campos) return set_error(GS355_EINVAL, "lod: frame.campos must be a device pointer to 3 floats");
+        if (!(lod->fork > 1.0f) || !(lod->standard_dist > 0.0f) || lod->max_level < 0)
+            return set_error(GS355_EINVAL, "lod: fork must be > 1, standard_dist > 0, max_level >= 0");
+        x.use_lod = 1;
+        x.lod = *lod;
+        x.log2_fork = (float)std::log2((double)lod->fork);
+        x.lod_mask = lod_mask;
+    }
+    const FrameArgs fa = make_args(frame);
+    return launch_anchor_filter(fa, *anchors, x, radii, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

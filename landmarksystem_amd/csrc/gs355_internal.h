@@ -35,6 +35,16 @@ struct FrameArgs {  // by-value kernel argument
     const float* bg;
 };
 
+// Extras of the radii-only preprocess when it serves the anchor prefilter (by-value kernel argument).
+struct FilterArgs {
+    int32_t scale_stride = 3;   // floats between the scale rows
+    int32_t use_lod = 0;
+    gs355_anchor_lod lod = {};
+    float log2_fork = 1.0f;     // (float)log2((double)fork), as the reference's host-side math.log2(fork)
+    uint8_t* lod_mask = nullptr;  // optional
+    uint8_t* visible = nullptr;   // optional: radius > 0
+};
+
 int set_error(int code, const char* fmt, ...);
 
 // Tile rectangle of a splat.  Only subtractions, additions and divisions by 16:
@@ -68,6 +78,7 @@ int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_o
                       uint32_t* tiles_touched, uint64_t* rects, uint32_t* depth_bits, int32_t* radii, hipStream_t s);
 int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int32_t P, uint32_t* offsets,
                         uint32_t* scan_tmp, gs355_header* header, uint32_t n_cap, hipStream_t s);
+int launch_anchor_filter(const FrameArgs& f, const gs355_gaussians& g, const FilterArgs& x, int32_t* radii, hipStream_t s);
 int launch_duplicate(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
                      const uint32_t* offsets, const gs355_header* header, uint64_t* keys, uint32_t* values,
                      hipStream_t s);

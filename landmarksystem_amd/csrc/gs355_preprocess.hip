@@ -145,8 +145,23 @@ __device__ __forceinline__ void sh_staged_rounds(float4* __restrict__ mine, cons
 }
 
 
+// Octree-GS level-of-detail test of one anchor, in the reference's order of fp32 operations
+// (octreegs_encoding.py:251-264).
+__device__ __forceinline__ bool lod_keeps(const gs355_anchor_lod& l, float log2_fork, int i, float x, float y, float z,
+                                          const float* campos)
+{
+    const float level = l.level[i];
+    const float shift = (0.5f * l.voxel_size) / powf(l.fork, level);
+    const float dx = (x + shift) - campos[0], dy = (y + shift) - campos[1], dz = (z + shift) - campos[2];
+    const float dist = sqrtf((dx * dx + dy * dy) + dz * dz) * l.resolution_scale;
+    const float pred = log2f(l.standard_dist / dist) / log2_fork + l.extra_level[i];
+    float r = l.rounding == 0 ? floorf(pred) : l.rounding == 1 ? rintf(pred) : ceilf(pred);
+    r = fminf(fmaxf(r, 0.0f), (float)l.max_level);  // NaN -> 0
+    return level <= r;
+}
+
 template <bool kRadiiOnly>
-__global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaussians g,
+__global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaussians g, FilterArgs fx,
                                                          float* __restrict__ records,
                                                          uint32_t* __restrict__ tiles_touched,
                                                          uint64_t* __restrict__ rects,
@@ -171,22 +186,27 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
     // dependent ones (culled Gaussians cost 28 to 32 B of extra reads).
     float cov[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, scale[3] = {0.f, 0.f, 0.f}, quat[4] = {0.f, 0.f, 0.f, 0.f};
     float opacity = 0.f;
+    bool gated = false;  // anchor outside the level-of-detail mask (anchor prefilter only)
     if (valid) {
         x = g.means3D[3 * (size_t)i];
         y = g.means3D[3 * (size_t)i + 1];
         z = g.means3D[3 * (size_t)i + 2];
+        if (kRadiiOnly && fx.use_lod) {
+            gated = !lod_keeps(fx.lod, fx.log2_fork, i, x, y, z, f.campos);
+            if (fx.lod_mask) fx.lod_mask[i] = gated ? 0 : 1;
+        }
         if (g.cov3D_precomp) {
 #pragma unroll
             for (int k = 0; k < 6; ++k) cov[k] = g.cov3D_precomp[6 * (size_t)i + k];
         } else {
 #pragma unroll
-            for (int k = 0; k < 3; ++k) scale[k] = g.scales[3 * (size_t)i + k];
+            for (int k = 0; k < 3; ++k) scale[k] = g.scales[(kRadiiOnly ? fx.scale_stride : 3) * (size_t)i + k];
 #pragma unroll
             for (int k = 0; k < 4; ++k) quat[k] = g.rotations[4 * (size_t)i + k];
         }
         if (!kRadiiOnly) opacity = g.opacities[i];
     }
-    if (valid) do {
+    if (valid && !gated) do {
         const float vx = ((V[0] * x + V[4] * y) + V[8] * z) + V[12];
         const float vy = ((V[1] * x + V[5] * y) + V[9] * z) + V[13];
         vz = ((V[2] * x + V[6] * y) + V[10] * z) + V[14];
@@ -247,8 +267,11 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
         qz = ca * det_inv;
     } while (false);
 
-    if (valid) radii[i] = radius;
-    if (kRadiiOnly) return;
+    if (valid && radii) radii[i] = radius;
+    if (kRadiiOnly) {
+        if (valid && fx.visible) fx.visible[i] = radius > 0 ? 1 : 0;
+        return;
+    }
     if (valid) {
         tiles_touched[i] = touched;
         rects[i] = rect_packed;
@@ -377,13 +400,23 @@ int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_o
 {
     if (g.P == 0) return GS355_OK;
     const dim3 block(256), grid((g.P + 255) / 256);
+    const FilterArgs none;
     if (radii_only)
-        hipLaunchKernelGGL(preprocess_kernel<true>, grid, block, 0, s, f, g, records, tiles_touched, rects, depth_bits,
-                           radii);
+        hipLaunchKernelGGL(preprocess_kernel<true>, grid, block, 0, s, f, g, none, records, tiles_touched, rects,
+                           depth_bits, radii);
     else
-        hipLaunchKernelGGL(preprocess_kernel<false>, grid, block, 0, s, f, g, records, tiles_touched, rects, depth_bits,
-                           radii);
+        hipLaunchKernelGGL(preprocess_kernel<false>, grid, block, 0, s, f, g, none, records, tiles_touched, rects,
+                           depth_bits, radii);
     GS355_CHECK_LAUNCH("preprocess");
+    return GS355_OK;
+}
+
+int launch_anchor_filter(const FrameArgs& f, const gs355_gaussians& g, const FilterArgs& x, int32_t* radii, hipStream_t s)
+{
+    if (g.P == 0) return GS355_OK;
+    hipLaunchKernelGGL(preprocess_kernel<true>, dim3((g.P + 255) / 256), dim3(256), 0, s, f, g, x, (float*)nullptr,
+                       (uint32_t*)nullptr, (uint64_t*)nullptr, (uint32_t*)nullptr, radii);
+    GS355_CHECK_LAUNCH("anchor filter");
     return GS355_OK;
 }
 

@@ -307,8 +307,13 @@ class ScaffoldGS(nn.Module):
     def __init__(self, anchor=None, anchor_feat=None, offset=None, scaling=None, rotation=None, n_offsets: int = 10,
                  feat_dim: int = 32, add_opacity_dist: bool = True, add_cov_dist: bool = True,
                  add_color_dist: bool = True, white_bkgd: bool = False, act_cache: bool = False, opacity=None,
-                 config=None, scene_manager=None):
+                 config=None, scene_manager=None, fuse_prefilter: bool = False):
         super().__init__()
+        # fuse_prefilter: the anchor-level prefilter (for Octree-GS including the level-of-detail mask, its gather
+        # of the selected anchors and the scatter of the result) runs as one kernel over all anchors.  Same masks,
+        # except that an anchor whose predicted level sits within rounding of a .5 boundary may fall on the other
+        # side (the level-of-detail formula is evaluated in the kernel instead of by a chain of torch operations).
+        self.fuse_prefilter = fuse_prefilter
         if anchor is not None and not torch.is_tensor(anchor):  # the reference's signature: (config, scene_manager)
             config, anchor = anchor, None
         if config is not None:  # empty model, filled by load_from_state_dict (scaffold_gs/gs_model.py:104-140)
@@ -317,6 +322,7 @@ class ScaffoldGS(nn.Module):
             add_cov_dist = _cfg(config, "add_cov_dist", add_cov_dist)
             add_color_dist = _cfg(config, "add_color_dist", add_color_dist)
             white_bkgd, act_cache = _cfg(config, "white_bkgd", white_bkgd), _cfg(config, "act_cache", act_cache)
+            self.fuse_prefilter = _cfg(config, "fuse_prefilter", fuse_prefilter)
             for name, allowed in (("use_feat_bank", False), ("appearance_dim", 0), ("add_level", False),
                                   ("view_dim", 3)):
                 if _cfg(config, name, allowed) != allowed:
@@ -418,7 +424,18 @@ class ScaffoldGS(nn.Module):
     def _anchor_subset(self):
         return None  # Scaffold-GS filters all anchors
 
+    def _lod(self, viewpoint_camera):
+        return None  # Scaffold-GS has no level of detail
+
     def prefilter_voxel(self, viewpoint_camera, scaling_modifier=1.0):
+        if self.fuse_prefilter and not self.training:
+            from . import pipeline
+            visible, mask = pipeline.anchor_filter(
+                _settings(viewpoint_camera, self.background, scaling_modifier, 1), self.get_anchor, self.get_scaling,
+                self.get_rotation, self._lod(viewpoint_camera))
+            if mask is not None:
+                self._anchor_mask = mask
+            return visible
         rasterizer = GaussianRasterizer(raster_settings=_settings(viewpoint_camera, self.background,
                                                                   scaling_modifier, 1))
         subset = self._anchor_subset()
@@ -494,16 +511,14 @@ class OctreeGS(ScaffoldGS):
         anchor_pos = self._anchor + (self.voxel_size / 2) / (float(self.fork) ** self._level)
         dist = torch.sqrt(torch.sum((anchor_pos - cam_center) ** 2, dim=1)) * resolution_scale
         pred_level = torch.log2(self.standard_dist / dist) / math.log2(self.fork) + self._extra_level
-        if self._level_span is None or self._level_span[0] is not self._level:
-            # the span of the levels is a constant of the loaded model: read it back once, not per frame
-            self._level_span = (self._level, int((torch.max(self._level) - torch.min(self._level)).item()))
+        max_level = self._level_span_value()
         if self.dist2level == "floor":
             int_level = torch.floor(pred_level).int()
         elif self.dist2level == "round":
             int_level = torch.round(pred_level).int()
         else:
             int_level = torch.ceil(pred_level).int()
-        int_level = torch.clamp(int_level, min=0, max=self._level_span[1])
+        int_level = torch.clamp(int_level, min=0, max=max_level)
         self._anchor_mask = self._level.squeeze(dim=1) <= int_level
 
     def get_state_dict_from_ckpt(self, file_path, map_location="cpu"):
@@ -527,7 +542,25 @@ class OctreeGS(ScaffoldGS):
         # appearance inputs (appearance_dim = 0, all this decode supports) it has no effect
         return super().forward(viewpoint_camera, scaling_modifier, retain_grad, render_exclude_filter)
 
+    def _level_span_value(self) -> int:
+        if self._level_span is None or self._level_span[0] is not self._level:
+            # the span of the levels is a constant of the loaded model: read it back once, not per frame
+            self._level_span = (self._level, int((torch.max(self._level) - torch.min(self._level)).item()))
+        return self._level_span[1]
+
+    def _lod(self, viewpoint_camera):
+        if not self.enable_lod:
+            return None
+        return dict(level=self._level.reshape(-1), extra_level=self._extra_level, voxel_size=self.voxel_size,
+                    standard_dist=self.standard_dist, fork=self.fork,
+                    resolution_scale=float(getattr(viewpoint_camera, "resolution_scale", 1.0)),
+                    rounding=self.dist2level, max_level=self._level_span_value())
+
     def _before_prefilter(self, viewpoint_camera):
+        if self.fuse_prefilter and not self.training:
+            if not self.enable_lod:
+                self._anchor_mask = torch.ones(self._level.shape[0], dtype=torch.bool, device=self._level.device)
+            return  # the fused prefilter computes the level-of-detail mask itself
         if not self.training:
             self.set_anchor_mask(viewpoint_camera.camera_center, -1, viewpoint_camera.resolution_scale)
 

@@ -167,6 +167,46 @@ def visible_filter(inputs: FrameInputs) -> torch.Tensor:
     return radii
 
 
+def anchor_filter(settings, anchors: torch.Tensor, scaling: torch.Tensor, rotations: torch.Tensor, lod=None):
+    """The anchor-level visibility prefilter of Scaffold-GS / Octree-GS in one kernel (gs355_anchor_filter).
+
+    `scaling` is the models' f32[A,6] (or [A,3]); its first three columns are read in place.  `lod`: None, or a dict
+    with level f32[A], extra_level f32[A], voxel_size, standard_dist, fork, resolution_scale, rounding
+    ("floor" | "round" | "ceil") and max_level.  Returns (visible bool[A], lod_mask bool[A] or None)."""
+    if not anchors.is_cuda:
+        raise ValueError("anchors must be a tensor on the GPU (the rasterizer has no CPU path)")
+    dev, A = anchors.device, anchors.shape[0]
+    means = _dev_f32(anchors, dev, "anchors", (A, 3))
+    sc = _dev_f32(scaling, dev, "scaling")
+    if sc.dim() != 2 or sc.shape[0] != A or sc.shape[1] < 3:
+        raise ValueError("scaling must have shape [A, >=3], got %s" % (tuple(sc.shape),))
+    rot = _dev_f32(rotations, dev, "rotations", (A, 4))
+    keep = [_dev_f32(settings.viewmatrix, dev, "viewmatrix", (16,)), _dev_f32(settings.projmatrix, dev, "projmatrix", (16,)),
+            _dev_f32(settings.campos, dev, "campos", (3,))]
+    f = _lib.Frame()
+    f.image_width, f.image_height = int(settings.image_width), int(settings.image_height)
+    f.tanfovx, f.tanfovy, f.scale_modifier = float(settings.tanfovx), float(settings.tanfovy), float(settings.scale_modifier)
+    f.viewmatrix, f.projmatrix, f.campos = keep[0].data_ptr(), keep[1].data_ptr(), keep[2].data_ptr()
+    g = _lib.Gaussians()
+    g.P, g.means3D, g.scales, g.rotations = A, _ptr(means), _ptr(sc), _ptr(rot)
+    visible = torch.empty(A, dtype=torch.bool, device=dev)
+    mask, lod_c = None, None
+    if lod is not None:
+        level = _dev_f32(lod["level"], dev, "level", (A,))
+        extra = _dev_f32(lod["extra_level"], dev, "extra_level", (A,))
+        keep += [level, extra]
+        mask = torch.empty(A, dtype=torch.bool, device=dev)
+        lod_c = _lib.AnchorLod(_ptr(level), _ptr(extra), float(lod["voxel_size"]), float(lod["standard_dist"]),
+                               float(lod["fork"]), float(lod["resolution_scale"]),
+                               {"floor": 0, "round": 1, "ceil": 2}[lod["rounding"]], int(lod["max_level"]))
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    _lib.check(_lib.load().gs355_anchor_filter(C.byref(f), C.byref(g), int(sc.shape[1]),
+                                               C.byref(lod_c) if lod_c is not None else None, _ptr(mask),
+                                               _ptr(visible), None, stream))
+    del keep
+    return visible, mask
+
+
 class FrameOutputs:
     def __init__(self, inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True):
         dev, H, W = inputs.device, inputs.height, inputs.width

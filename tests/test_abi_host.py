@@ -33,6 +33,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(_lib.Gaussians) == 8 + 7 * 8
     assert C.sizeof(_lib.Outputs) == 4 * 8
     assert C.sizeof(_lib.Layout) == 18 * 8 + 4 * 4
+    assert C.sizeof(_lib.AnchorLod) == 2 * 8 + 4 * 4 + 2 * 4
 
 
 def test_workspace_layout_is_aligned_ordered_and_sized():
@@ -148,6 +149,33 @@ def test_visible_filter_validates():
     half = _gauss()
     half.rotations = None
     assert "scale/rotation" in _err(_lib.GS355_EINVAL, vf, f, half, 0x1000)
+
+
+def test_anchor_filter_validates_before_any_hip_call():
+    lib = _lib.load()
+    f, g = _frame(), _gauss(shs=False)
+
+    def af(f, g, stride, lod, visible):
+        return lib.gs355_anchor_filter(C.byref(f) if f else None, C.byref(g) if g else None, stride,
+                                       C.byref(lod) if lod else None, None, visible, None, None)
+
+    lod = _lib.AnchorLod(0x1000, 0x1000, 0.5, 250.0, 2.0, 1.0, 1, 4)
+    assert "frame is NULL" in _err(_lib.GS355_EINVAL, af, None, g, 6, None, 0x1000)
+    assert "visible is NULL" in _err(_lib.GS355_EINVAL, af, f, g, 6, None, None)
+    assert "scale_stride" in _err(_lib.GS355_EINVAL, af, f, g, 2, None, 0x1000)
+    assert "scale/rotation" in _err(_lib.GS355_EINVAL, af, f, _gauss(sr=False), 6, None, 0x1000)
+    bad = _lib.AnchorLod(0x1000, None, 0.5, 250.0, 2.0, 1.0, 1, 4)
+    assert "extra_level is NULL" in _err(_lib.GS355_EINVAL, af, f, g, 6, bad, 0x1000)
+    bad = _lib.AnchorLod(0x1000, 0x1000, 0.5, 250.0, 2.0, 1.0, 3, 4)
+    assert "rounding" in _err(_lib.GS355_EINVAL, af, f, g, 6, bad, 0x1000)
+    bad = _lib.AnchorLod(0x1000, 0x1000, 0.5, 250.0, 1.0, 1.0, 1, 4)
+    assert "fork must be > 1" in _err(_lib.GS355_EINVAL, af, f, g, 6, bad, 0x1000)
+    no_cam = _frame()
+    no_cam.campos = None
+    assert "campos" in _err(_lib.GS355_EINVAL, af, no_cam, g, 6, lod, 0x1000)
+    empty = _gauss(shs=False)
+    empty.P = 0
+    assert af(f, empty, 6, lod, None) == 0  # nothing to do, nothing launched
 
 
 def _decoder(feat=32, n=10, in_dim=(36, 36, 36), ptr=0x1000):

@@ -169,3 +169,52 @@ def test_spatial_order_renders_the_same_frame(gpu_device, tmp_path):
     diff = (a - b).abs()
     assert float(diff.max()) <= 2e-3 and float((diff > 1e-6).float().mean()) < 0.01
     assert psnr(a.cpu().numpy(), b.cpu().numpy()) >= 80.0
+
+
+def _octree_pair(scene, gpu_device, **kw):
+    level = torch.randint(0, 5, (scene.anchor.shape[0],), generator=torch.Generator().manual_seed(5))
+    extra = torch.randn(scene.anchor.shape[0], generator=torch.Generator().manual_seed(6)) * 0.3
+    models = []
+    for fuse in (False, True):
+        m = OctreeGS(scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
+                     voxel_size=0.5, standard_dist=250.0, fork=2, extra_level=extra, n_offsets=scene.n_offsets,
+                     fuse_prefilter=fuse, **kw)
+        m.anchor_decoder.load_state_dict(ScaffoldGS.from_scene(scene).anchor_decoder.state_dict())
+        models.append(m.to(gpu_device).eval())
+    return models
+
+
+@pytest.mark.parametrize("dist2level", ["round", "floor", "ceil"])
+def test_fused_anchor_prefilter_matches_the_reference_sequence(gpu_device, dist2level):
+    """One-kernel anchor prefilter (level-of-detail mask + visibility) against the models' own sequence of torch
+    operations, gathers and visible_filter call."""
+    scene = scenes.config5(A=40_000, width=640, height=360)
+    cam = scene.camera
+    plain = ScaffoldGS.from_scene(scene).to(gpu_device).eval()
+    fused = ScaffoldGS.from_scene(scene, fuse_prefilter=True).to(gpu_device).eval()
+    a, b = plain(cam), fused(cam)
+    assert torch.equal(plain.voxel_visible_mask, fused.voxel_visible_mask)
+    assert 0 < int(fused.voxel_visible_mask.sum()) < 40_000
+    assert torch.equal(a, b)
+
+    ref, one = _octree_pair(scene, gpu_device, dist2level=dist2level)
+    a, b = ref(cam), one(cam)
+    # the predicted level is the same fp32 formula evaluated by different code: anchors within rounding of a
+    # decision boundary of floor / round / ceil may differ
+    anchor_pos = scene.anchor.double() + 0.25 / (2.0 ** ref._level.cpu().double())
+    dist = (anchor_pos - cam.camera_center.double()).norm(dim=1)
+    pred = torch.log2(250.0 / dist) + ref._extra_level.cpu().double()
+    frac = pred - torch.floor(pred)
+    edge = (frac - 0.5).abs() < 1e-4 if dist2level == "round" else (frac < 1e-4) | (frac > 1 - 1e-4)
+    same = ref._anchor_mask.cpu() == one._anchor_mask.cpu()
+    assert bool(same[~edge].all()) and int((~same).sum()) <= int(edge.sum())
+    assert 0 < int(one._anchor_mask.sum()) < 40_000
+    assert not bool((one.voxel_visible_mask & ~one._anchor_mask).any())
+    if bool(same.all()):
+        assert torch.equal(ref.voxel_visible_mask, one.voxel_visible_mask) and torch.equal(a, b)
+    # closed form in float64 away from the boundaries
+    R = {"round": torch.round, "floor": torch.floor, "ceil": torch.ceil}[dist2level]
+    want = ref._level.cpu().double().squeeze(1) <= torch.clamp(R(pred), 0, 4)
+    assert torch.equal(one._anchor_mask.cpu()[~edge], want[~edge])
+    one.enable_lod = ref.enable_lod = False
+    assert torch.equal(ref(cam), one(cam)) and bool(one._anchor_mask.all())

@@ -81,3 +81,28 @@ def test_settings_on_host_and_scale_modifier(gpu_device):
     np.testing.assert_array_equal(radii.cpu().numpy(), ref["radii"])
     solid = ref["fragile"] == 0
     assert np.abs(image.cpu().numpy() - ref["image"])[:, solid].max() <= 1e-4
+
+
+def test_frames_in_flight_on_two_streams_are_independent(gpu_device):
+    """Each stream gets its own workspace, so frames of different scenes can be in flight at once (the next
+    frame's preprocess overlapping the current frame's blend) and still come out as when rendered alone."""
+    from landmarksystem_amd import GaussianRasterizer
+    a = scenes.config2(P=120_000, width=640, height=360).to(gpu_device)
+    b = scenes.config3(P=150_000, width=512, height=288).to(gpu_device)
+
+    def render(scene):
+        rast = GaussianRasterizer(settings_for(scene, gpu_device))
+        return rast(means3D=scene.means3D, means2D=None, shs=scene.shs, colors_precomp=None, opacities=scene.opacities,
+                    scales=scene.scales, rotations=scene.rotations, cov3D_precomp=None)
+
+    alone = [render(a), render(b)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=gpu_device), torch.cuda.Stream(device=gpu_device)]
+    outs = []
+    for k in range(8):
+        with torch.cuda.stream(streams[k % 2]):
+            outs.append(render(a if k % 2 == 0 else b))
+    torch.cuda.synchronize()
+    for k, (image, radii, depth) in enumerate(outs):
+        want = alone[k % 2]
+        assert torch.equal(image, want[0]) and torch.equal(radii, want[1]) and torch.equal(depth, want[2])

@@ -24,6 +24,10 @@
 // hidden activations enter the matrix cores as hi + lo fp16 pairs, so the
 // result carries fp32-level accuracy with fp32 accumulation.
 //
+// Work follows the visible anchors: a wavefront takes runs of 128 consecutive
+// anchors, packs the visible ones (in order) into dense tiles of 32 and decodes
+// those only.
+//
 // Output order is the reference's boolean-mask order: row-major over (visible
 // anchor, offset).  Two launches: count kept offsets per anchor (opacity head
 // only) -> exclusive scan -> emit (all heads; the opacity head is recomputed
@@ -174,6 +178,10 @@ struct TileInputs {
     float ofv[kCountOnly ? 1 : 5][3] = {};
 };
 
+// A wavefront takes runs of kRun consecutive anchors, packs the visible ones (in order) into dense tiles of 32
+// and runs the MLPs on those only: the work follows the number of visible anchors, not of anchors.
+constexpr int kRun = 128;
+
 template <bool kCountOnly>
 __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
                                                      const uint32_t* __restrict__ offsets, uint32_t capacity,
@@ -185,7 +193,8 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
     // 11n head outputs of an anchor, then its scaling (6), position (3) and first output slot (1).
     constexpr int kStrideMax = kCountOnly ? 11 : 123;
     constexpr int kListFloats = kCountOnly ? 0 : 160;  // 320 16-bit item numbers after the anchors' rows
-    __shared__ float s_out[4][32 * kStrideMax + kListFloats];
+    constexpr int kRunFloats = kRun / 4;                // kRun 8-bit positions of the run's visible anchors
+    __shared__ float s_out[4][32 * kStrideMax + kListFloats + kRunFloats];
 
     // biases of the three heads, zero-padded: b0 at [head*32], b1 of opacity / cov / colour at 96 / 128 / 224
     __shared__ float s_bias[256];
@@ -214,18 +223,30 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
     const int items = 32 * n;  // (anchor, offset) pairs of a tile: item = anchor_in_tile * n + offset
     const int inv_n = (65536 + n - 1) / n;  // item / n == (item * inv_n) >> 16 for item < 32 n, n <= 10
     const uint64_t lanes_below = (1ull << lane) - 1ull;
-    const int tiles = (d.A + 31) / 32;
+    const int runs = (d.A + kRun - 1) / kRun;
     float* __restrict__ mine = s_out[wave];
+    uint8_t* __restrict__ run_list = reinterpret_cast<uint8_t*>(mine + 32 * kStrideMax + kListFloats);
     const float cx = d.campos[0], cy = d.campos[1], cz = d.campos[2];
 
-    for (int tile = blockIdx.x * 4 + wave; tile < tiles; tile += gridDim.x * 4) {
-        const int a = tile * 32 + col;  // this lane's anchor (lanes l and l+32 share it)
-        const bool vis = a < d.A && d.visible[a] != 0;
-        const uint64_t any = __ballot(vis);  // bits l and l + 32 belong to anchor l of the tile
-        if (any == 0ull) {  // nothing visible in these 32 anchors
-            if (kCountOnly && half == 0 && a < d.A) counts[a] = 0;
-            continue;
-        }
+    for (int run = blockIdx.x * 4 + wave; run < runs; run += gridDim.x * 4) {
+      // positions (within the run) of its visible anchors, in order: lane covers anchors lane and 64 + lane
+      const int base = run * kRun;
+      const int a0 = base + lane, a1 = base + 64 + lane;
+      const bool v0 = a0 < d.A && d.visible[a0] != 0, v1 = a1 < d.A && d.visible[a1] != 0;
+      const uint64_t m0 = __ballot(v0), m1 = __ballot(v1);
+      const int n0 = __popcll(m0), nvis = n0 + __popcll(m1);
+      if (kCountOnly) {  // anchors that are not decoded keep nothing
+          if (!v0 && a0 < d.A) counts[a0] = 0;
+          if (!v1 && a1 < d.A) counts[a1] = 0;
+      }
+      if (nvis == 0) continue;  // uniform
+      if (v0) run_list[__popcll(m0 & lanes_below)] = (uint8_t)lane;
+      if (v1) run_list[n0 + __popcll(m1 & lanes_below)] = (uint8_t)(64 + lane);
+      wave_lds_sync();
+      for (int first = 0; first < nvis; first += 32) {  // dense tiles of the run
+        const bool vis = first + col < nvis;  // lanes l and l+32 share entry first + l
+        const int a = vis ? base + (int)run_list[first + col] : 0;
+        const uint64_t any = __ballot(vis);  // bits l and l + 32 belong to entry l of the tile
         // Everything the tile needs from global memory is requested here, before the first use.
         TileInputs<kCountOnly> in;
         if (vis) {
@@ -244,14 +265,15 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
 #pragma unroll
                 for (int k = 0; k < 3; ++k) in.sc3[k] = d.scaling[6 * (size_t)a + 3 * half + k];
             }
-            if (a < d.A) in.first_slot = offsets[a];  // lane 0's value is the tile's first output slot
-            // the learned offsets of the items this lane's position covers (contiguous over the lanes),
-            // for visible anchors only
+            if (vis) in.first_slot = offsets[a];  // entry 0's value is the tile's first output slot
+            // the learned offsets of the items this lane's position covers (item = entry * n + offset)
 #pragma unroll
             for (int r = 0; r < 5; ++r) {
                 const int it = r * 64 + lane;
-                const bool want = it < items && ((any >> ((it * inv_n) >> 16)) & 1ull);
-                const float* __restrict__ of = d.offset + ((size_t)tile * 32 * n + (want ? it : 0)) * 3;
+                const int al = (it * inv_n) >> 16;
+                const bool want = it < items && ((any >> al) & 1ull);
+                const int ai = want ? base + (int)run_list[first + al] : 0;
+                const float* __restrict__ of = d.offset + ((size_t)ai * n + (want ? it - al * n : 0)) * 3;
 #pragma unroll
                 for (int k = 0; k < 3; ++k) in.ofv[r][k] = want ? of[k] : 0.0f;
             }
@@ -294,10 +316,9 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         store_rows(mine + col * stride, 0, n, 0, half, op[0]);
         if (kCountOnly) {
             wave_lds_sync();
-            if (half == 0 && a < d.A) {
+            if (half == 0 && vis) {
                 uint32_t kept = 0;
-                if (vis)
-                    for (int m = 0; m < n; ++m) kept += mine[col * stride + m] > 0.0f ? 1u : 0u;
+                for (int m = 0; m < n; ++m) kept += mine[col * stride + m] > 0.0f ? 1u : 0u;
                 counts[a] = kept;
             }
             wave_lds_sync();
@@ -384,6 +405,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
             rot[4 * (size_t)pos + 3] = q3 / norm;
         }
         wave_lds_sync();
+      }
     }
 }
 
@@ -431,12 +453,12 @@ static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, DecodeAr
     return GS355_OK;
 }
 
-// Persistent workgroups (4 wavefronts, each walking tiles of 32 anchors): at most `cap` of them, about what
+// Persistent workgroups (4 wavefronts, each walking runs of kRun anchors): at most `cap` of them, about what
 // the chip holds at once, so the weight fragments are fetched once per resident workgroup.
 static dim3 decode_grid(int A, int cap)
 {
-    const int tiles = (A + 31) / 32;
-    int blocks = (tiles + 3) / 4;
+    const int runs = (A + kRun - 1) / kRun;
+    int blocks = (runs + 3) / 4;
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
     return dim3(blocks);

@@ -104,31 +104,52 @@ __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P
     }
 }
 
-// Thread per tile: exclusive prefix of the tile's counts over the slices (in
-// place) and the tile's total.
-__global__ __launch_bounds__(64) void slice_prefix_kernel(uint32_t* __restrict__ matrix, int groups, int tiles,
+// Exclusive prefix of every tile's counts over the slices (in place) and the
+// tile's total.  A workgroup covers 64 tiles; its four wavefronts take a
+// quarter of the slices each (loads of a thread are issued in batches, so many
+// are in flight), exchange their quarter sums through LDS and write the
+// prefixes shifted by the quarters before them.
+__global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict__ matrix, int groups, int tiles,
                                                            uint32_t* __restrict__ totals)
 {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= tiles) return;
-    uint32_t run = 0;
-    int c = 0;
-    for (; c + 32 <= groups; c += 32) {  // 32 independent loads in flight per thread
-        uint32_t v[32];
+    __shared__ uint32_t s_part[4][64];
+    const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
+    const int t = blockIdx.x * 64 + lane;
+    const int per = (groups + 3) / 4;
+    const int c0 = min(part * per, groups), c1 = min(c0 + per, groups);
+    const bool live = t < tiles;
+    // pass 1: sum of this thread's quarter
+    uint32_t sum = 0;
+    for (int c = c0; c < c1 && live; c += 16) {
+        uint32_t v[16];
 #pragma unroll
-        for (int k = 0; k < 32; ++k) v[k] = matrix[(size_t)(c + k) * tiles + t];
+        for (int k = 0; k < 16; ++k) v[k] = matrix[(size_t)min(c + k, c1 - 1) * tiles + t];
 #pragma unroll
-        for (int k = 0; k < 32; ++k) {
-            matrix[(size_t)(c + k) * tiles + t] = run;
-            run += v[k];
+        for (int k = 0; k < 16; ++k) sum += c + k < c1 ? v[k] : 0u;
+    }
+    s_part[part][lane] = sum;
+    __syncthreads();
+    uint32_t run = 0, total = 0;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t v = s_part[p][lane];
+        if (p < part) run += v;
+        total += v;
+    }
+    // pass 2: the quarter's values again (now cached), replaced by the running sum before them
+    for (int c = c0; c < c1 && live; c += 16) {
+        uint32_t v[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) v[k] = matrix[(size_t)min(c + k, c1 - 1) * tiles + t];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            if (c + k < c1) {
+                matrix[(size_t)(c + k) * tiles + t] = run;
+                run += v[k];
+            }
         }
     }
-    for (; c < groups; ++c) {
-        const uint32_t v = matrix[(size_t)c * tiles + t];
-        matrix[(size_t)c * tiles + t] = run;
-        run += v;
-    }
-    totals[t] = run;
+    if (live && part == 0) totals[t] = total;
 }
 
 // One workgroup: tile totals -> tile bases, ranges, the frame header and the
@@ -187,8 +208,15 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
     }
     // bases, ranges and size-class lists of the thread's own tiles (skipped on overflow: later stages do nothing)
     uint32_t first = (uint32_t)(before + inc - mine);
-    for (uint32_t t = t0; t < t1 && !overflow; ++t) {
-        const uint32_t v = totals[t];  // read before tile_base[t] (possibly the same word) is written
+    for (uint32_t tb = t0; tb < t1 && !overflow; tb += 8) {
+      // the batch's totals are read before any of its tile_base words (possibly the same words) is written
+      uint32_t batch[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) batch[k] = totals[min(tb + k, t1 - 1)];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const uint32_t t = tb + k, v = batch[k];
+        if (t >= t1) break;
         ranges[2 * t] = v ? first : 0u;
         ranges[2 * t + 1] = v ? first + v : 0u;
         tile_base[t] = first;
@@ -200,6 +228,7 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
         else if (v > (uint32_t)kTileSortCap[0]) cls = 0;
         if (cls >= 0) lists[4 + (size_t)cls * tiles + atomicAdd(&s_nlist[cls], 1u)] = t;
         first += v;
+      }
     }
     __syncthreads();
     if (threadIdx.x < 4) lists[threadIdx.x] = s_nlist[threadIdx.x];
@@ -857,7 +886,7 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
-    hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(64), 0, s, matrix, groups, tiles,
+    hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(256), 0, s, matrix, groups, tiles,
                        tile_base);
     GS355_CHECK_LAUNCH("bin: slice prefix");
     hipLaunchKernelGGL(tile_layout_kernel, dim3(1), dim3(1024), 0, s, tile_base, (uint32_t)tiles, group_visible, groups,

@@ -709,54 +709,33 @@ struct LdsSorter {
             flags[11] = 0;
             flags[12] = 0xFFFFFFFFu;
             flags[13] = 0;
-            flags[14] = 0xFFFFFFFFu;
         }
         __syncthreads();
-        // The whole bucket is requested before the first value is used, so a thread's loads are in flight
-        // together (rounds past the end of the bucket are skipped, uniformly over the workgroup).
-        // (batches of at most 5 rounds bound the registers that hold them)
-        constexpr int kBatch = kR < 5 ? kR : 5;
-        // bits in which the depths differ = OR of all & ~AND of all
-        uint32_t all_or = 0, all_and = 0xFFFFFFFFu, dmin = 0xFFFFFFFFu, dmax = 0;
-#pragma unroll
-        for (int r0 = 0; r0 < kR; r0 += kBatch) {
-            uint64_t v[kBatch];
-#pragma unroll
-            for (int r = 0; r < kBatch; ++r) {
-                v[r] = 0;
-                if ((uint32_t)((r0 + r) * kT) < n)
-                    v[r] = buckets[lo + min((uint32_t)((r0 + r) * kT) + threadIdx.x, n - 1)];
-            }
-#pragma unroll
-            for (int r = 0; r < kBatch; ++r) {
-                const uint32_t j = (uint32_t)((r0 + r) * kT) + threadIdx.x;
-                if (j < n) {
-                    const uint32_t dj = (uint32_t)(v[r] >> 32);
-                    depth[j] = dj;
-                    index[j] = (uint32_t)v[r];
-                    all_or |= dj;
-                    all_and &= dj;
-                    dmin = min(dmin, dj);
-                    dmax = max(dmax, dj);
-                }
-            }
+        const uint32_t d0 = (uint32_t)(buckets[lo] >> 32);
+        uint32_t diff = 0, dmin = 0xFFFFFFFFu, dmax = 0;
+        for (uint32_t j = threadIdx.x; j < n; j += kT) {
+            const uint64_t v = buckets[lo + j];
+            const uint32_t dj = (uint32_t)(v >> 32);
+            depth[j] = dj;
+            index[j] = (uint32_t)v;
+            diff |= dj ^ d0;
+            dmin = min(dmin, dj);
+            dmax = max(dmax, dj);
         }
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) {
-            all_or |= __shfl_xor(all_or, d, 64);
-            all_and &= __shfl_xor(all_and, d, 64);
+            diff |= __shfl_xor(diff, d, 64);
             dmin = min(dmin, (uint32_t)__shfl_xor(dmin, d, 64));
             dmax = max(dmax, (uint32_t)__shfl_xor(dmax, d, 64));
         }
         if ((threadIdx.x & 63) == 0) {
-            atomicOr(&flags[11], all_or);
-            atomicAnd(&flags[14], all_and);
+            if (diff) atomicOr(&flags[11], diff);
             atomicMin(&flags[12], dmin);
             atomicMax(&flags[13], dmax);
         }
         __syncthreads();
         int cur = bucket_sort(n, flags[12], flags[13]);
-        if (cur == -2) cur = sort(n, flags[11] & ~flags[14]);
+        if (cur == -2) cur = sort(n, flags[11]);
         for (uint32_t j = threadIdx.x; j < n; j += kT) {
             const uint32_t e = cur < 0 ? j : (uint32_t)perm(cur)[j];
             out_keys[lo + j] = ((uint64_t)tile << 32) | (uint64_t)depth[e];

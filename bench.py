@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what
 # the same counter reads for the 1 GiB copy of --calibration-copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
 # "keys_sort_ranges" is the sum over the kernels of the tile count, scatter and tile sort stages.
-MEASURED_TRAFFIC_BYTES = {"blend": 1848.7e6, "preprocess": 1722.7e6, "keys_sort_ranges": 831.2e6}
+MEASURED_TRAFFIC_BYTES = {"blend": 1849.7e6, "preprocess": 1799.6e6, "keys_sort_ranges": 838.8e6}
 # (pixel, Gaussian) pairs of the default workload's blend, counted by the CPU checker (`python -m oracle.workload_stats 3`):
 # every list entry a pixel visits before it terminates / the pairs applied to a pixel (alpha >= 1/255).  Properties
 # of the seeded scene, not of a kernel; 25 flop per evaluated pair is the blend's algorithmic work.
@@ -52,6 +52,9 @@ def parse_args():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--no-model-level", action="store_true",
+                    help="skip the model-level variants (their launches of the same kernels on other inputs would "
+                         "mix into the per-kernel averages of a profiler run)")
     ap.add_argument("--two-in-flight", action="store_true",
                     help="also time the frames with two in flight on alternating streams (reported beside `value`)")
     return ap.parse_args()
@@ -180,7 +183,7 @@ def bench_scaffold(args, torch, dev):
     from landmarksystem_amd.models import OctreeGS
     variants = {}
     level = torch.randint(0, 5, (scene.anchor.shape[0],), generator=torch.Generator().manual_seed(5))
-    for name, make in (
+    for name, make in () if args.no_model_level else (
         ("scaffold_fused_prefilter", lambda: ScaffoldGS.from_scene(scene, act_cache=True, fuse_prefilter=True)),
         ("octree_reference_sequence", lambda: OctreeGS(
             scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
@@ -294,8 +297,9 @@ def main():
     # (third variant: the same scene stored along a Morton curve, a load-time option of the checkpoint loaders)
     from landmarksystem_amd.models import GaussianModel, morton_order
     model_fps = {}
-    for name, fuse, ordered in (("reference_sequence", False, False), ("fused_prefilter", True, False),
-                                ("fused_prefilter_spatial_order", True, True)):
+    for name, fuse, ordered in (() if args.no_model_level else (
+            ("reference_sequence", False, False), ("fused_prefilter", True, False),
+            ("fused_prefilter_spatial_order", True, True))):
         pick = morton_order(d.means3D) if ordered else slice(None)
         model = GaussianModel(d.means3D[pick], d.shs[pick][:, :1].contiguous(), d.shs[pick][:, 1:].contiguous(),
                               torch.log(d.scales[pick]), d.rotations[pick],

@@ -138,7 +138,7 @@ enum {
     GS355_STAGE_BLEND = 32,     /* front-to-back alpha blending per 16x16 tile */
     GS355_STAGE_ALL = 63, /* the six stages above: the classic pipeline */
     /* Verification variant of the blend stage: every staged Gaussian is evaluated on every pixel of the tile
-     * (no per-quadrant culling).  Produces the same image as GS355_STAGE_BLEND; not part of GS355_STAGE_ALL. */
+     * (no per-block culling).  Produces the same image as GS355_STAGE_BLEND; not part of GS355_STAGE_ALL. */
     GS355_STAGE_BLEND_PLAIN = 64,
     /* Tile-bucketed equivalent of SCAN + DUPLICATE + SORT + RANGES: same sorted keys, values, ranges and
      * header, far less memory traffic, no global atomics.

@@ -310,11 +310,11 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
     }
     if (!alive) return;
 
-    // Reach of the splat for the blend stage's quadrant culling: half-extents
+    // Reach of the splat for the blend stage's per-block culling: half-extents
     // (ex, ey) of the axis-aligned box around the region where alpha can reach
     // 1/255, i.e. where 0.5 d^T Q d <= ln(255 * opacity).  The box is enlarged
     // by more than the rounding error of the blend's fp32 evaluation of the
-    // exponent (bounded below by `noise`), so a quadrant outside the box is
+    // exponent (bounded below by `noise`), so a pixel block outside the box is
     // certain to take the blend's `alpha < 1/255` branch on all of its pixels.
     // +inf = never cull (large or ill-conditioned splats), -inf = never visible.
     float ex, ey;

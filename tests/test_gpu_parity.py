@@ -218,9 +218,9 @@ def test_rerun_is_bit_identical(gpu_device):
 @pytest.mark.parametrize("make", [lambda: scenes.config3(P=400_000), lambda: scenes.config2(P=80_000),
                                   lambda: scenes.tiny_scene(P=3000, width=333, height=211, sh_degree=1, seed=2,
                                                             log_scale_mean=-1.0)])
-def test_quadrant_culling_is_result_neutral(gpu_device, make):
-    """The blend stage skips (8x8 quadrant, Gaussian) pairs whose bounding box
-    shows alpha < 1/255 on all 64 pixels; the verification variant evaluates
+def test_block_culling_is_result_neutral(gpu_device, make):
+    """The blend stage skips (4x4 pixel block, Gaussian) pairs whose bounding box
+    shows alpha < 1/255 on all 16 pixels; the verification variant evaluates
     every pair.  Both must give identical bits."""
     scene = make()
     s = settings_for(scene, gpu_device)

@@ -217,3 +217,29 @@ def test_decode_validates_before_any_hip_call():
     assert "capacity" in _err(_lib.GS355_EINVAL, emit, _decoder(), _anchors(), 0x1000, -1, out)
     need = C.c_size_t()
     assert lib.gs355_decode_scratch_bytes(1000, C.byref(need)) == 0 and need.value >= 256
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/gs355.h must compile as C99 (the boundary carries no C++ or torch types), and a C caller's view of the
+    struct sizes must match what the Python binding assumes."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "probe.c"
+    src.write_text(
+        '#include <stdio.h>\n#include "gs355.h"\n'
+        "int main(void) {\n"
+        '  printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(gs355_header), sizeof(gs355_frame),\n'
+        "         sizeof(gs355_gaussians), sizeof(gs355_outputs), sizeof(gs355_layout), sizeof(gs355_anchor_lod),\n"
+        "         sizeof(gs355_decoder), sizeof(gs355_anchors), sizeof(gs355_decoded));\n"
+        "  return GS355_PIPELINE_FAST == (GS355_STAGE_PREPROCESS | GS355_STAGE_TILE_COUNT | GS355_STAGE_TILE_SCATTER |\n"
+        "                                 GS355_STAGE_TILESORT | GS355_STAGE_BLEND) ? 0 : 1;\n}\n")
+    exe = tmp_path / "probe"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(root, "include"), str(src),
+                    "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    want = [C.sizeof(t) for t in (_lib.Header, _lib.Frame, _lib.Gaussians, _lib.Outputs, _lib.Layout, _lib.AnchorLod,
+                                  _lib.Decoder, _lib.Anchors, _lib.Decoded)]
+    assert [int(v) for v in out] == want

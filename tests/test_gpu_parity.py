@@ -373,3 +373,25 @@ def test_tile_sort_fallback_on_massive_depth_ties(gpu_device, same, spread, labe
     k = got["sorted_keys"]
     run_lengths = np.diff(np.flatnonzero(np.concatenate([[True], k[1:] != k[:-1], [True]])))
     assert run_lengths.max() >= same, label
+
+
+def test_images_beyond_the_tile_bucket_limit(gpu_device):
+    """More than 36000 tiles: the per-tile counters of the bucketed stages no longer fit in LDS.  The C entry point
+    says so; the Python driver renders such frames through the classic stages, with the same result contract."""
+    scene = scenes.config2(P=20_000, width=4000, height=2400)  # 250 x 150 = 37500 tiles
+    s = settings_for(scene, gpu_device)
+    d = scene.to(gpu_device)
+    inp = pipeline.FrameInputs(s, d.means3D, opacities=d.opacities, shs=d.shs, scales=d.scales, rotations=d.rotations)
+    assert inp.tiles > _lib.MAX_FAST_TILES
+    out = pipeline.FrameOutputs(inp)
+    ws = pipeline.Workspace(gpu_device)
+    with pytest.raises(_lib.Gs355Error, match="tiles"):
+        pipeline.run_stages(inp, out, ws, 1 << 20, _lib.PIPELINE_FAST)
+    got = pipeline.render(inp, ws=ws)
+    torch.cuda.synchronize()
+    ref = co.render(oracle_frame(scene), oracle_gaussians(scene))
+    assert got.num_keys == ref["num_keys"]
+    np.testing.assert_array_equal(got.radii.cpu().numpy(), ref["radii"])
+    solid = ref["fragile"] == 0
+    image = got.image.cpu().numpy()
+    assert np.abs(image - ref["image"])[:, solid].max() <= 1e-4 and psnr(image, ref["image"]) >= 60.0

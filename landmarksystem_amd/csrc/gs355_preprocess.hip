@@ -107,43 +107,48 @@ __device__ __forceinline__ void sh_finish(float res[3])
     }
 }
 
-// SH blocks are staged through LDS in kShRounds rounds of kShChunk
-// coefficients; the stride keeps the 16-B reads of the 64 lanes on distinct
-// banks (stride = 4 mod 8 floats).
-constexpr int kShRounds = 1;
-constexpr int kShChunk = 16 / kShRounds;                                   // coefficients per round
-constexpr int kShChunk4 = kShChunk * 3 / 4;                                // float4s per Gaussian per round
-constexpr int kShStride = kShChunk * 3 + ((kShChunk * 3) % 8 == 0 ? 4 : 0);  // floats per Gaussian in LDS
+// SH blocks (16 coefficients, 192 B) are staged through LDS; the stride keeps the 16-B reads of the 64 lanes on
+// distinct banks (stride = 4 mod 8 floats).
+constexpr int kShStride = 52;  // floats per Gaussian in the staging area
 
-template <int kRound>
-__device__ __forceinline__ void sh_staged_rounds(float4* __restrict__ mine, const float4* __restrict__ src, int count,
-                                                 int lane, bool alive, int terms, const float b[16], float res[3])
+// One wavefront fetches the SH blocks of up to 64 Gaussians with coalesced 16-B loads (twelve lanes per block)
+// and each lane then evaluates the colour of its own entry from LDS.  `owner[e]` is the position of entry e's
+// Gaussian within the workgroup's 256 (entries are the workgroup's surviving Gaussians, packed in order), so the
+// loads touch survivors' blocks only, however few of the 256 survived.  A row of the staging area holds an
+// entry's 48 coefficients and, in its 4 floats of padding, the Gaussian's position on the way in and its colour
+// on the way out.
+template <int kLoads>  // 16-B loads per lane: 64 * kLoads >= 12 * count
+__device__ __forceinline__ void sh_colour_of_entries(float4* __restrict__ mine, const float* __restrict__ shs,
+                                                     size_t group_first, const uint8_t* __restrict__ owner,
+                                                     int first_entry, int count, int lane, int degree,
+                                                     const float* campos)
 {
-    if constexpr (kRound < kShRounds) {
-        if (kRound * kShChunk < terms) {  // uniform: lower degrees stop early
-            if (kRound > 0) wave_lds_sync();
-            // all loads of the round are issued before the first LDS write, so they are in flight together;
-            // slots past a partial wavefront's last Gaussian re-read that Gaussian (same value, same address)
-            float4 v[kShChunk4];
-            int dst[kShChunk4];
+    // all loads are issued before the first LDS write, so they are in flight together; slots past the last
+    // entry re-read that entry (same value, same address)
+    float4 v[kLoads];
+    int dst[kLoads];
 #pragma unroll
-            for (int it = 0; it < kShChunk4; ++it) {
-                const int q4 = it * 64 + lane;
-                const int gq = min(q4 / kShChunk4, count - 1), m = q4 % kShChunk4;
-                v[it] = src[gq * 12 + kRound * kShChunk4 + m];
-                dst[it] = gq * (kShStride / 4) + m;
-            }
+    for (int it = 0; it < kLoads; ++it) {
+        const int q4 = it * 64 + lane;
+        const int e = min(q4 / 12, count - 1), m = q4 % 12;
+        const float4* __restrict__ block =
+            reinterpret_cast<const float4*>(shs + (group_first + owner[first_entry + e]) * 48);
+        v[it] = block[m];
+        dst[it] = e * (kShStride / 4) + m;
+    }
 #pragma unroll
-            for (int it = 0; it < kShChunk4; ++it) mine[dst[it]] = v[it];
-            wave_lds_sync();
-            if (alive)
-                sh_accumulate<kRound * kShChunk, kShChunk>(terms, reinterpret_cast<const float*>(mine) + lane * kShStride,
-                                                           b, res);
-            sh_staged_rounds<kRound + 1>(mine, src, count, lane, alive, terms, b, res);
-        }
+    for (int it = 0; it < kLoads; ++it) mine[dst[it]] = v[it];
+    wave_lds_sync();
+    if (lane < count) {
+        float* __restrict__ row = reinterpret_cast<float*>(mine) + lane * kShStride;
+        float b[16], rgb[3] = {0.f, 0.f, 0.f};
+        sh_basis(degree, row[48] - campos[0], row[49] - campos[1], row[50] - campos[2], b);
+        sh_accumulate<0, 16>((degree + 1) * (degree + 1), row, b, rgb);
+        sh_finish(rgb);
+#pragma unroll
+        for (int c = 0; c < 3; ++c) row[48 + c] = rgb[c];
     }
 }
-
 
 // Octree-GS level-of-detail test of one anchor, in the reference's order of fp32 operations
 // (octreegs_encoding.py:251-264).
@@ -170,6 +175,9 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
 {
     // staging area for the 16-coefficient SH blocks of each wavefront's 64 Gaussians
     __shared__ float4 s_sh[kRadiiOnly ? 1 : 4 * 64 * kShStride / 4];
+    // the workgroup's surviving Gaussians, packed in order: position within the workgroup; survivors per wavefront
+    __shared__ uint8_t s_owner[kRadiiOnly ? 1 : 256];
+    __shared__ int s_alive[4];
 
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     const bool valid = i < g.P;
@@ -287,26 +295,56 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
             rgb[2] = g.colors_precomp[3 * (size_t)i + 2];
         }
     } else {
-        // When most of the wavefront survived and the blocks are the full 192 B,
-        // the SH of its 64 Gaussians is fetched with coalesced 16-B loads into
-        // LDS, a chunk of coefficients at a time, and each lane reads its own
-        // chunk back from there; otherwise every survivor fetches its own
-        // block.  Same values and the same order of additions either way.
+        // Full 192-B blocks: the survivors of the workgroup are packed (in order) and each wavefront fetches the
+        // SH blocks of 64 of them with coalesced loads through LDS, so the memory system sees dense wavefronts
+        // however many Gaussians were culled.  Other block sizes: every survivor fetches its own block.  Same
+        // values and the same order of additions either way.
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-        const int wave_first = blockIdx.x * blockDim.x + wave * 64;
-        const bool staged = f.sh_coeffs == 16 && (reinterpret_cast<uintptr_t>(g.shs) & 15u) == 0 &&
-                            __popcll(__ballot(alive)) >= 32;  // uniform per wavefront
-        const int terms = (f.sh_degree + 1) * (f.sh_degree + 1);
-        float b[16];
-        if (alive) sh_basis(f.sh_degree, x - f.campos[0], y - f.campos[1], z - f.campos[2], b);
-        if (staged) {
-            sh_staged_rounds<0>(s_sh + wave * (64 * kShStride / 4),
-                                reinterpret_cast<const float4*>(g.shs + (size_t)wave_first * 48),
-                                min(64, g.P - wave_first), lane, alive, terms, b, rgb);
+        const bool packed = f.sh_coeffs == 16 && (reinterpret_cast<uintptr_t>(g.shs) & 15u) == 0;  // uniform
+        if (packed) {
+            const uint64_t m = __ballot(alive);
+            if (lane == 0) s_alive[wave] = __popcll(m);
+            __syncthreads();
+            int before = 0, total = 0;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                before += w < wave ? s_alive[w] : 0;
+                total += s_alive[w];
+            }
+            // packed entry e lives in row e of the staging area
+            float* __restrict__ my_row = reinterpret_cast<float*>(s_sh) +
+                                         (before + __popcll(m & ((1ull << lane) - 1ull))) * kShStride;
+            if (alive) {
+                s_owner[before + __popcll(m & ((1ull << lane) - 1ull))] = (uint8_t)threadIdx.x;
+                my_row[48] = x;
+                my_row[49] = y;
+                my_row[50] = z;
+            }
+            __syncthreads();
+            // each wavefront takes a quarter of the packed survivors (entry e sits in row e of the staging area)
+            const int share = (total + 3) / 4, first_entry = wave * share;
+            if (first_entry < total) {
+                float4* __restrict__ rows = s_sh + first_entry * (kShStride / 4);
+                const size_t group_first = (size_t)blockIdx.x * blockDim.x;
+                const int count = min(share, total - first_entry);
+                if (count <= 16)  // uniform: fewer survivors, fewer load rounds
+                    sh_colour_of_entries<3>(rows, g.shs, group_first, s_owner, first_entry, count, lane, f.sh_degree, f.campos);
+                else if (count <= 32)
+                    sh_colour_of_entries<6>(rows, g.shs, group_first, s_owner, first_entry, count, lane, f.sh_degree, f.campos);
+                else
+                    sh_colour_of_entries<12>(rows, g.shs, group_first, s_owner, first_entry, count, lane, f.sh_degree, f.campos);
+            }
+            __syncthreads();
+            if (alive) {
+#pragma unroll
+                for (int c = 0; c < 3; ++c) rgb[c] = my_row[48 + c];
+            }
         } else if (alive) {
-            sh_accumulate<0, 16>(terms, g.shs + (size_t)i * f.sh_coeffs * 3, b, rgb);
+            float b[16];
+            sh_basis(f.sh_degree, x - f.campos[0], y - f.campos[1], z - f.campos[2], b);
+            sh_accumulate<0, 16>((f.sh_degree + 1) * (f.sh_degree + 1), g.shs + (size_t)i * f.sh_coeffs * 3, b, rgb);
+            sh_finish(rgb);
         }
-        if (alive) sh_finish(rgb);
     }
     if (!alive) return;
 

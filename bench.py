@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what
 # the same counter reads for the 1 GiB copy of --calibration-copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
 # "keys_sort_ranges" is the sum over the kernels of the tile count, scatter and tile sort stages.
-MEASURED_TRAFFIC_BYTES = {"blend": 1849.7e6, "preprocess": 1799.6e6, "keys_sort_ranges": 838.8e6}
+MEASURED_TRAFFIC_BYTES = {"blend": 1849.2e6, "preprocess": 1701.9e6, "keys_sort_ranges": 838.8e6}
 # (pixel, Gaussian) pairs of the default workload's blend, counted by the CPU checker (`python -m oracle.workload_stats 3`):
 # every list entry a pixel visits before it terminates / the pairs applied to a pixel (alpha >= 1/255).  Properties
 # of the seeded scene, not of a kernel; 25 flop per evaluated pair is the blend's algorithmic work.

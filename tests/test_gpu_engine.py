@@ -60,3 +60,18 @@ def test_engine_renders_checkpoints_like_the_direct_models(gpu_device, tmp_path)
     engine = init_inference(OctreeGS, InferenceOctreeGSModule, config, dict(runtime="Kernel"))
     assert engine.base_model.voxel_size == 0.5 and engine.base_model.standard_dist == 250.0
     assert torch.equal(engine(anchors.camera, 1.0, None, None), octree(anchors.camera))
+
+
+def test_render_trajectory_equals_frame_by_frame(gpu_device):
+    from landmarksystem_amd.engine import render_trajectory
+    scene = scenes.config4(P=200_000, width=640, height=360, n_poses=6)
+    model = GaussianModel.from_activated(scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs,
+                                         sh_degree=3, act_cache=True, fuse_prefilter=True).to(gpu_device).eval()
+    want = [model(cam).clone() for cam in scene.cameras]
+    for in_flight in (1, 2, 3):
+        got = list(render_trajectory(model, scene.cameras, in_flight=in_flight))
+        torch.cuda.synchronize()
+        assert len(got) == len(want)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+    assert len({float(w.sum()) for w in want}) == len(want)  # the poses really differ

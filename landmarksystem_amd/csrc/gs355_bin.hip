@@ -174,12 +174,19 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
     const uint32_t per = (tiles + 1023u) / 1024u;
     const uint32_t t0 = min(threadIdx.x * per, tiles), t1 = min(t0 + per, tiles);
     uint64_t mine = 0;
+    uint32_t head[8];  // the run's first 8 totals stay in registers for the second pass (all of them up to 8192 tiles)
+#pragma unroll
+    for (int k = 0; k < 8; ++k) head[k] = 0;
     for (uint32_t t = t0; t < t1; t += 8) {  // 8 loads in flight (the last batch re-reads the run's last tile)
         uint32_t v[8];
 #pragma unroll
         for (int k = 0; k < 8; ++k) v[k] = totals[min(t + k, t1 - 1)];
 #pragma unroll
         for (int k = 0; k < 8; ++k) mine += t + k < t1 ? v[k] : 0u;
+        if (t == t0) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) head[k] = v[k];
+        }
     }
     uint32_t vis = 0;
     for (int c = threadIdx.x; c < groups; c += 1024) vis += group_visible[c];
@@ -212,7 +219,7 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
       // the batch's totals are read before any of its tile_base words (possibly the same words) is written
       uint32_t batch[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) batch[k] = totals[min(tb + k, t1 - 1)];
+      for (int k = 0; k < 8; ++k) batch[k] = tb == t0 ? head[k] : totals[min(tb + k, t1 - 1)];
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const uint32_t t = tb + k, v = batch[k];

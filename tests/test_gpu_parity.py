@@ -255,7 +255,8 @@ def run_fast_path(scene, device):
     return dict(sorted_keys=u64(ws.view(lay, "sorted_keys", P, n, tiles)),
                 sorted_values=u32(ws.view(lay, "sorted_values", P, n, tiles)),
                 ranges=u32(ws.view(lay, "ranges", P, n, tiles)), image=out.image.cpu().numpy(),
-                depth=out.depth.cpu().numpy()[0], alpha=out.alpha.cpu().numpy()[0], num_keys=n)
+                depth=out.depth.cpu().numpy()[0], alpha=out.alpha.cpu().numpy()[0], num_keys=n,
+                radii=out.radii.cpu().numpy())
 
 
 def crowded_scene(P, width=64, height=64, duplicates=0, seed=0):
@@ -351,6 +352,22 @@ def test_full_size_headline_frame_properties(gpu_device):
     for name in ("sorted_keys", "sorted_values", "ranges", "image", "depth", "alpha"):
         np.testing.assert_array_equal(got[name], again[name], err_msg=name)
     assert got["alpha"].min() >= 0.0 and got["alpha"].max() <= 1.0 and np.isfinite(got["image"]).all()
+
+
+def test_full_size_headline_frame_equals_the_oracle(gpu_device):
+    """The whole 6M-Gaussian 1080p frame against the C oracle (a few seconds on the host's cores): radii, all
+    13.6M sorted keys and values and the ranges bit for bit, the image to the frame tolerances."""
+    scene = scenes.config3()
+    got = run_fast_path(scene, gpu_device)
+    ref = oracle_render(scene)
+    assert got["num_keys"] == ref["num_keys"] > 10_000_000
+    for name in ("radii", "ranges", "sorted_keys", "sorted_values"):
+        np.testing.assert_array_equal(got[name], ref[name], err_msg=name)
+    solid = ref["fragile"] == 0
+    assert solid.mean() > 0.98
+    assert np.abs(got["image"] - ref["image"])[:, solid].max() <= IMG_TOL
+    assert psnr(got["image"], ref["image"]) >= PSNR_MIN
+    assert np.abs(got["alpha"] - ref["alpha"])[solid].max() <= IMG_TOL
 
 
 @pytest.mark.parametrize("same,spread,label", [(1800, 0, "one depth only"), (1500, 2500, "one heavy depth among many"),

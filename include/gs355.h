@@ -17,6 +17,8 @@
  *                   432-434, octree_gs/gs_model.py:491-493
  *   ScaffoldGS / OctreeGS.prefilter_voxel   -> gs355_anchor_filter (one pass for the models' own sequence)
  *       call sites: scaffold_gs/gs_model.py:385-436, octree_gs/gs_model.py:445-497
+ *   autograd backward of forward(...)       -> gs355_render_backward
+ *       call site:  benchmarks/nerf/origin_gs/gs_trainer.py:117-124 (loss.backward())
  *   GaussianRasterizationSettings(...)      -> gs355_frame
  *       built at:   origin_gs/gs_model.py:148-161 (and the two siblings)
  *
@@ -201,6 +203,51 @@ typedef struct gs355_anchor_lod {
 GS355_API int gs355_anchor_filter(const gs355_frame *frame, const gs355_gaussians *anchors, int32_t scale_stride,
                                   const gs355_anchor_lod *lod, uint8_t *lod_mask, uint8_t *visible, int32_t *radii,
                                   void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Backward pass of GaussianRasterizer.forward: what autograd calls when the reference trains through the
+ * rasterizer (loss.backward(), benchmarks/nerf/origin_gs/gs_trainer.py:117-124; `means2D.grad` feeds
+ * densification, landmark/nerf_components/model_components/fields/encodings/gaussian_encoding.py:729-743 with
+ * origin_gs/gs_model.py:129-139,225-236).  It runs over the workspace the forward pass of the same frame left
+ * behind (records, sorted values, ranges: nothing else may have used that workspace in between) and the
+ * forward outputs. */
+#define GS355_GRAD_FLOATS 12 /* scratch floats per Gaussian */
+
+typedef struct gs355_backward_inputs {
+    const float *image;     /* [3,H,W] forward output */
+    const float *depth;     /* [H,W]   forward output; required when dL_ddepth is given */
+    const float *alpha;     /* [H,W]   forward output; required when dL_dalpha is given */
+    const int32_t *radii;   /* [P]     forward output */
+    const float *dL_dimage; /* [3,H,W] */
+    const float *dL_ddepth; /* [H,W] or NULL */
+    const float *dL_dalpha; /* [H,W] or NULL */
+} gs355_backward_inputs;
+
+/* Gradients with respect to the inputs of forward(); any pointer may be NULL (that gradient is not written).
+ * Every element is written (zeros for culled Gaussians), so the buffers need no initialisation.  means2D is
+ * the screen-space gradient in normalised device units (pixel-space gradient times W/2 and H/2, third
+ * component 0), the convention the reference's densification thresholds are tuned for.  The gradient passes
+ * through min(0.99, opacity * G) unchanged. */
+typedef struct gs355_gradients {
+    float *means3D;        /* [P,3] */
+    float *means2D;        /* [P,3] */
+    float *shs;            /* [P,M,3] */
+    float *colors_precomp; /* [P,3] */
+    float *opacities;      /* [P] */
+    float *scales;         /* [P,3] */
+    float *rotations;      /* [P,4] */
+    float *cov3D_precomp;  /* [P,6] */
+} gs355_gradients;
+
+/* Bytes of scratch gs355_render_backward needs for P Gaussians (per-Gaussian accumulators). */
+GS355_API int gs355_backward_scratch_bytes(int32_t P, size_t *bytes);
+
+/* frame, g, workspace, workspace_bytes, n_cap: exactly what the forward call (gs355_render, or gs355_run through
+ * the blend stage) was given.  The sums over pixels use floating-point atomics: results vary in the last bits
+ * from run to run. */
+GS355_API int gs355_render_backward(const gs355_frame *frame, const gs355_gaussians *g, const void *workspace,
+                                    size_t workspace_bytes, int64_t n_cap, const gs355_backward_inputs *in,
+                                    void *scratch, size_t scratch_bytes, const gs355_gradients *grads, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Anchor decode for Scaffold-GS / Octree-GS: replaces AnchorDecoder.forward in eval mode

@@ -20,7 +20,8 @@ MAX_FAST_TILES = 36000
 
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
            "gs355_visible_filter", "gs355_anchor_filter", "gs355_decode_scratch_bytes", "gs355_decode_count",
-           "gs355_decode_emit")
+           "gs355_decode_emit", "gs355_backward_scratch_bytes", "gs355_render_backward")
+GRAD_FLOATS = 12
 
 
 class Frame(C.Structure):
@@ -126,6 +127,15 @@ class AnchorLod(C.Structure):
                 ("rounding", C.c_int32), ("max_level", C.c_int32)]
 
 
+class BackwardInputs(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("image", "depth", "alpha", "radii", "dL_dimage", "dL_ddepth", "dL_dalpha")]
+
+
+class Gradients(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("means3D", "means2D", "shs", "colors_precomp", "opacities", "scales",
+                                          "rotations", "cov3D_precomp")]
+
+
 class Gs355Error(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__("gs355 error %d: %s" % (code, message))
@@ -169,6 +179,12 @@ def load() -> C.CDLL:
     lib.gs355_decode_emit.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_int64,
                                       C.POINTER(Decoded), C.c_void_p]
     lib.gs355_decode_emit.restype = C.c_int
+    lib.gs355_backward_scratch_bytes.argtypes = [C.c_int32, C.POINTER(C.c_size_t)]
+    lib.gs355_backward_scratch_bytes.restype = C.c_int
+    lib.gs355_render_backward.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_void_p, C.c_size_t, C.c_int64,
+                                          C.POINTER(BackwardInputs), C.c_void_p, C.c_size_t, C.POINTER(Gradients),
+                                          C.c_void_p]
+    lib.gs355_render_backward.restype = C.c_int
     _lib = lib
     return lib
 

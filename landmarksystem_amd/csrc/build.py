@@ -35,6 +35,7 @@ SOURCES = [
     ("gs355_bin.hip", []),
     ("gs355_decode.hip", []),
     ("gs355_blend.hip", []),
+    ("gs355_backward.hip", []),
 ]
 
 

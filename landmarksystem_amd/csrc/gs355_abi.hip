@@ -279,6 +279,52 @@ int gs355_visible_filter(const gs355_frame* frame, const gs355_gaussians* g, int
     return launch_preprocess(fa, *g, true, nullptr, nullptr, nullptr, nullptr, radii, static_cast<hipStream_t>(stream));
 }
 
+int gs355_backward_scratch_bytes(int32_t P, size_t* bytes)
+{
+    if (!bytes) return set_error(GS355_EINVAL, "bytes is NULL");
+    if (P < 0) return set_error(GS355_EINVAL, "P must be >= 0 (got %d)", P);
+    *bytes = align_up((size_t)P * GS355_GRAD_FLOATS * sizeof(float));
+    return GS355_OK;
+}
+
+int gs355_render_backward(const gs355_frame* frame, const gs355_gaussians* g, const void* workspace,
+                          size_t workspace_bytes, int64_t n_cap, const gs355_backward_inputs* in, void* scratch,
+                          size_t scratch_bytes, const gs355_gradients* grads, void* stream)
+{
+    int rc;
+    if ((rc = check_frame(frame, true))) return rc;
+    if ((rc = check_geometry_inputs(g))) return rc;
+    if ((rc = check_colour_inputs(frame, g))) return rc;
+    if (!in) return set_error(GS355_EINVAL, "backward inputs is NULL");
+    if (!grads) return set_error(GS355_EINVAL, "gradients is NULL");
+    if (!in->image || !in->dL_dimage) return set_error(GS355_EINVAL, "image / dL_dimage is NULL");
+    if (in->dL_ddepth && !in->depth) return set_error(GS355_EINVAL, "dL_ddepth is given but the forward depth is NULL");
+    if (in->dL_dalpha && !in->alpha) return set_error(GS355_EINVAL, "dL_dalpha is given but the forward alpha is NULL");
+    if (g->P > 0 && !in->radii) return set_error(GS355_EINVAL, "radii is NULL");
+    if ((grads->shs && !g->shs) || (grads->colors_precomp && !g->colors_precomp) || (grads->scales && !g->scales) ||
+        (grads->rotations && !g->rotations) || (grads->cov3D_precomp && !g->cov3D_precomp))
+        return set_error(GS355_EINVAL, "a gradient is requested for an input that was not given");
+    gs355_layout L;
+    if ((rc = make_layout(g->P, n_cap, frame->image_width, frame->image_height, &L))) return rc;
+    if (!workspace) return set_error(GS355_EINVAL, "workspace is NULL");
+    if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
+        return set_error(GS355_EINVAL, "workspace must be 256-byte aligned");
+    if (workspace_bytes < L.total_bytes)
+        return set_error(GS355_ENOSPC, "workspace has %zu bytes, %zu needed (P=%d, n_cap=%lld, %dx%d)", workspace_bytes,
+                         L.total_bytes, g->P, (long long)n_cap, frame->image_width, frame->image_height);
+    const size_t need = align_up((size_t)g->P * GS355_GRAD_FLOATS * sizeof(float));
+    if (g->P > 0 && !scratch) return set_error(GS355_EINVAL, "scratch is NULL");
+    if ((reinterpret_cast<uintptr_t>(scratch) & 15u) != 0) return set_error(GS355_EINVAL, "scratch must be 16-byte aligned");
+    if (scratch_bytes < need)
+        return set_error(GS355_ENOSPC, "scratch has %zu bytes, %zu needed (P=%d)", scratch_bytes, need, g->P);
+    const char* ws = static_cast<const char*>(workspace);
+    return launch_render_backward(make_args(frame), *g, reinterpret_cast<const gs355_header*>(ws + L.header),
+                                  reinterpret_cast<const uint32_t*>(ws + L.ranges),
+                                  reinterpret_cast<const uint32_t*>(ws + L.values[L.sorted_buffer]),
+                                  reinterpret_cast<const float*>(ws + L.records), *in, static_cast<float*>(scratch),
+                                  *grads, static_cast<hipStream_t>(stream));
+}
+
 int gs355_anchor_filter(const gs355_frame* frame, const gs355_gaussians* anchors, int32_t scale_stride,
                         const gs355_anchor_lod* lod, uint8_t* lod_mask, uint8_t* visible, int32_t* radii, void* stream)
 {

@@ -1,0 +1,479 @@
+// Backward pass of the rasterizer for gfx950: the gradients the reference's training loop pulls through
+// GaussianRasterizer.forward (loss.backward() at benchmarks/nerf/origin_gs/gs_trainer.py:117-124; the
+// screen-space gradient of `means2D` feeds densification, landmark/nerf_components/model_components/fields/
+// encodings/gaussian_encoding.py:729-743).
+//
+// Two kernels over the forward pass's workspace (records, sorted values, ranges):
+//   blend_backward   per 16x16 tile, the forward blend's walk repeated FRONT TO BACK with the same per-block
+//                    lists and the same per-pair decisions.  With f_i = colour_i . dL/dpixel, w_i = alpha_i T_i,
+//                    prefix P_i = sum_{j<=i} w_j f_j and R = out_pixel . dL/dpixel - T_final dL/dalpha_out (all
+//                    known from the forward outputs), dL/dalpha_i = T_i f_i - (R - P_i) / (1 - alpha_i): no
+//                    division by a transmittance and no second, reversed walk.  Per-pair gradients are summed
+//                    over the 16 pixels of a block with lane shuffles inside the 16-lane row, added to the staged
+//                    Gaussian's accumulators in LDS, and flushed to global memory once per batch of 256.
+//   preprocess_backward  per Gaussian: conic -> 2-D covariance -> Jacobian / 3-D covariance -> scale, rotation,
+//                    mean; pixel position -> mean; colour -> SH coefficients and view direction -> mean.
+// min(0.99, opacity * G) passes the gradient unchanged, and the `means2D` gradient is in normalised device units
+// (pixel gradient times W/2, H/2), as the published backward pass of this rasterizer family does.
+#include "gs355_internal.h"
+
+namespace gs355 {
+
+namespace {
+
+constexpr int kGradFloats = GS355_GRAD_FLOATS;  // dpx, dpy, dconic xyz, dopacity, drgb, ddepth, 2 unused
+
+__device__ __forceinline__ float splat_exponent(float dx, float dy, float qx, float qy, float qz)
+{
+#pragma clang fp contract(off)
+    const float t1 = (qx * dx) * dx;
+    const float t2 = (qz * dy) * dy;
+    const float t3 = (qy * dx) * dy;
+    return -0.5f * (t1 + t2) - t3;
+}
+
+template <int kCtrl>
+__device__ __forceinline__ float dpp(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
+}
+
+// Sum over the 16 lanes of a row (every lane gets the total).
+__device__ __forceinline__ float row_sum(float v)
+{
+    v += dpp<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp<0x141>(v);  // row_half_mirror
+    v += dpp<0x140>(v);  // row_mirror
+    return v;
+}
+
+struct PixelGrad {
+    float g0, g1, g2, g3;  // dL/d(r, g, b, depth) of this pixel
+    float R;               // out . g - T_final * dL/dalpha_out
+};
+
+// One 16-lane row evaluates staged Gaussian `a, b, c` on its 16 pixels and returns the row's summed gradient
+// contributions in v[0..9] (every lane holds the sums).  T carries the forward blend's state (sign = finished).
+__device__ __forceinline__ bool backward_one(float& T, float& prefix, const PixelGrad& pg, float pxf, float pyf,
+                                             const float4 a, const float4 b, const float4 c, bool enabled,
+                                             float v[10])
+{
+    const float dx = a.x - pxf, dy = a.y - pyf;
+    const float power = splat_exponent(dx, dy, a.z, a.w, b.x);
+    const float G = __expf(power);
+    const float alpha = fminf(0.99f, b.y * G);
+    const bool accept = enabled && !(power > 0.0f || alpha < 1.0f / 255.0f);
+    const float test_T = T * (1.0f - alpha);
+    const bool hit = accept && test_T >= 0.0001f;
+    if (accept && !hit && T > 0.0f) T = -T;
+    if (__ballot(hit) == 0ull) return false;
+    float w = 0.0f, dpow = 0.0f, dop = 0.0f;
+    if (hit) {
+        w = alpha * T;
+        const float fg = b.z * pg.g0 + b.w * pg.g1 + c.x * pg.g2 + c.y * pg.g3;
+        prefix += w * fg;
+        const float dalpha = T * fg - (pg.R - prefix) * __frcp_rn(1.0f - alpha);
+        dop = G * dalpha;
+        dpow = b.y * dop;
+        T = test_T;
+    }
+    v[0] = row_sum(dpow * (-a.z * dx - a.w * dy));
+    v[1] = row_sum(dpow * (-b.x * dy - a.w * dx));
+    v[2] = row_sum(dpow * (-0.5f * dx * dx));
+    v[3] = row_sum(dpow * (-dx * dy));
+    v[4] = row_sum(dpow * (-0.5f * dy * dy));
+    v[5] = row_sum(dop);
+    v[6] = row_sum(w * pg.g0);
+    v[7] = row_sum(w * pg.g1);
+    v[8] = row_sum(w * pg.g2);
+    v[9] = row_sum(w * pg.g3);
+    return true;
+}
+
+__global__ __launch_bounds__(256) void blend_backward_kernel(
+    FrameArgs f, const gs355_header* __restrict__ header, const uint32_t* __restrict__ ranges,
+    const uint32_t* __restrict__ values, const float* __restrict__ records, const float* __restrict__ image,
+    const float* __restrict__ out_depth, const float* __restrict__ out_alpha, const float* __restrict__ g_image,
+    const float* __restrict__ g_depth, const float* __restrict__ g_alpha, float* __restrict__ grads)
+{
+    __shared__ float4 s_a[256];  // px, py, conic_x, conic_y
+    __shared__ float4 s_b[256];  // conic_z, opacity, r, g
+    __shared__ float4 s_c[256];  // b, depth, reach_x, reach_y
+    __shared__ float s_grad[256 * kGradFloats];
+    __shared__ uint32_t s_wave_done[4];
+    __shared__ uint8_t s_list[4][4][256 + 4];
+
+    if (header->overflow) return;
+    const int tile = blockIdx.x;
+    const int tile_x = tile % f.grid_x, tile_y = tile / f.grid_x;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int group = lane >> 4, sub = lane & 15;
+    const int qx0 = tile_x * kTile + (wave & 1) * 8, qy0 = tile_y * kTile + (wave >> 1) * 8;
+    const int px = qx0 + (group & 1) * 4 + (sub & 3), py = qy0 + (group >> 1) * 4 + (sub >> 2);
+    const bool inside = px < f.W && py < f.H;
+    const float pxf = (float)px, pyf = (float)py;
+    const float x_lo0 = (float)qx0, x_hi0 = (float)(qx0 + 3), x_lo1 = (float)(qx0 + 4), x_hi1 = (float)(qx0 + 7);
+    const float y_lo0 = (float)qy0, y_hi0 = (float)(qy0 + 3), y_lo1 = (float)(qy0 + 4), y_hi1 = (float)(qy0 + 7);
+    const uint64_t lanes_below = (1ull << lane) - 1ull;
+
+    PixelGrad pg = {0.f, 0.f, 0.f, 0.f, 0.f};
+    if (inside) {
+        const size_t plane = (size_t)f.W * f.H;
+        const size_t o = (size_t)py * f.W + px;
+        pg.g0 = g_image[o];
+        pg.g1 = g_image[plane + o];
+        pg.g2 = g_image[2 * plane + o];
+        pg.R = image[o] * pg.g0 + image[plane + o] * pg.g1 + image[2 * plane + o] * pg.g2;
+        if (g_depth) {
+            pg.g3 = g_depth[o];
+            pg.R += out_depth[o] * pg.g3;
+        }
+        if (g_alpha) pg.R -= (1.0f - out_alpha[o]) * g_alpha[o];
+    }
+
+    const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
+    float T = inside ? 1.0f : -1.0f, prefix = 0.0f;
+
+    for (uint32_t base = lo; base < hi; base += 256) {
+        const bool wave_done = __ballot(T > 0.0f) == 0ull;
+        if (lane == 0) s_wave_done[wave] = wave_done ? 1u : 0u;
+        const uint32_t j = base + tid;
+        uint32_t g = 0;
+        if (j < hi) {
+            g = values[j];
+            const float4* __restrict__ rec = reinterpret_cast<const float4*>(records + (size_t)g * kRecordFloats);
+            s_a[tid] = rec[0];
+            s_b[tid] = rec[1];
+            s_c[tid] = rec[2];
+        }
+        {
+            float4* __restrict__ row = reinterpret_cast<float4*>(s_grad + tid * kGradFloats);
+            row[0] = row[1] = row[2] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        __syncthreads();
+        if ((s_wave_done[0] & s_wave_done[1] & s_wave_done[2] & s_wave_done[3]) != 0u) break;
+        const int count = (int)min(256u, hi - base);
+        if (!wave_done) {
+            // ---- lists: which staged Gaussians reach which 4x4 block (lane = Gaussian), as the forward blend ----
+            uint32_t len[4] = {0u, 0u, 0u, 0u};
+            for (int chunk = 0; chunk < count; chunk += 64) {
+                const int k = chunk + lane;
+                bool in_x0 = false, in_x1 = false, in_y0 = false, in_y1 = false;
+                if (k < count) {
+                    const float4 a = s_a[k];
+                    const float4 c = s_c[k];
+                    const float bx_lo = a.x - c.z, bx_hi = a.x + c.z, by_lo = a.y - c.w, by_hi = a.y + c.w;
+                    in_x0 = bx_hi >= x_lo0 && bx_lo <= x_hi0;
+                    in_x1 = bx_hi >= x_lo1 && bx_lo <= x_hi1;
+                    in_y0 = by_hi >= y_lo0 && by_lo <= y_hi0;
+                    in_y1 = by_hi >= y_lo1 && by_lo <= y_hi1;
+                }
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const bool reach = ((b & 1) ? in_x1 : in_x0) && ((b >> 1) ? in_y1 : in_y0);
+                    const uint64_t m = __ballot(reach);
+                    if (reach) s_list[wave][b][len[b] + (uint32_t)__popcll(m & lanes_below)] = (uint8_t)k;
+                    len[b] += (uint32_t)__popcll(m);
+                }
+            }
+            wave_lds_sync();
+            const uint32_t my_len = group == 0 ? len[0] : group == 1 ? len[1] : group == 2 ? len[2] : len[3];
+            const uint32_t longest = max(max(len[0], len[1]), max(len[2], len[3]));
+            const uint8_t* __restrict__ mine = s_list[wave][group];
+            uint32_t k_next = mine[0];
+            for (uint32_t i = 0; i < longest; ++i) {
+                const uint32_t kk = k_next;
+                k_next = mine[i + 1];
+                float v[10];
+                if (backward_one(T, prefix, pg, pxf, pyf, s_a[kk], s_b[kk], s_c[kk], i < my_len, v)) {
+                    // lane `sub` of each row adds slot `sub` of its Gaussian
+                    float mine_v = v[0];
+#pragma unroll
+                    for (int s = 1; s < 10; ++s) mine_v = sub == s ? v[s] : mine_v;
+                    if (sub < 10 && i < my_len && mine_v != 0.0f) atomicAdd(&s_grad[kk * kGradFloats + sub], mine_v);
+                }
+                if (__ballot(T > 0.0f) == 0ull) break;
+            }
+        }
+        __syncthreads();
+        // ---- flush this batch's accumulators ----
+        if (j < hi) {
+            const float* __restrict__ row = s_grad + tid * kGradFloats;
+            float* __restrict__ dst = grads + (size_t)g * kGradFloats;
+#pragma unroll
+            for (int s = 0; s < 10; ++s) {
+                const float val = row[s];
+                if (val != 0.0f) unsafeAtomicAdd(dst + s, val);
+            }
+        }
+    }
+}
+
+constexpr float kShC0 = 0.28209479177387814f;
+constexpr float kShC1 = 0.4886025119029199f;
+constexpr float kShC2[5] = {1.0925484305920792f, -1.0925484305920792f, 0.31539156525252005f, -1.0925484305920792f,
+                            0.5462742152960396f};
+constexpr float kShC3[7] = {-0.5900435899266435f, 2.890611442640554f, -0.4570457994644658f, 0.3731763325901154f,
+                            -0.4570457994644658f, 1.445305721320277f, -0.5900435899266435f};
+
+// Real SH basis (sh_utils.py:67-94) and its gradient with respect to the unit direction.
+__device__ __forceinline__ void sh_basis_grad(int deg, float x, float y, float z, float b[16], float bx[16],
+                                              float by[16], float bz[16])
+{
+#pragma unroll
+    for (int k = 0; k < 16; ++k) b[k] = bx[k] = by[k] = bz[k] = 0.0f;
+    b[0] = kShC0;
+    if (deg < 1) return;
+    b[1] = -kShC1 * y; by[1] = -kShC1;
+    b[2] = kShC1 * z;  bz[2] = kShC1;
+    b[3] = -kShC1 * x; bx[3] = -kShC1;
+    if (deg < 2) return;
+    const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+    b[4] = kShC2[0] * xy; bx[4] = kShC2[0] * y; by[4] = kShC2[0] * x;
+    b[5] = kShC2[1] * yz; by[5] = kShC2[1] * z; bz[5] = kShC2[1] * y;
+    b[6] = kShC2[2] * (2.0f * zz - xx - yy); bx[6] = kShC2[2] * -2.0f * x; by[6] = kShC2[2] * -2.0f * y;
+    bz[6] = kShC2[2] * 4.0f * z;
+    b[7] = kShC2[3] * xz; bx[7] = kShC2[3] * z; bz[7] = kShC2[3] * x;
+    b[8] = kShC2[4] * (xx - yy); bx[8] = kShC2[4] * 2.0f * x; by[8] = kShC2[4] * -2.0f * y;
+    if (deg < 3) return;
+    b[9] = kShC3[0] * y * (3.0f * xx - yy); bx[9] = kShC3[0] * 6.0f * xy; by[9] = kShC3[0] * (3.0f * xx - 3.0f * yy);
+    b[10] = kShC3[1] * xy * z; bx[10] = kShC3[1] * yz; by[10] = kShC3[1] * xz; bz[10] = kShC3[1] * xy;
+    b[11] = kShC3[2] * y * (4.0f * zz - xx - yy); bx[11] = kShC3[2] * -2.0f * xy;
+    by[11] = kShC3[2] * (4.0f * zz - xx - 3.0f * yy); bz[11] = kShC3[2] * 8.0f * yz;
+    b[12] = kShC3[3] * z * (2.0f * zz - 3.0f * xx - 3.0f * yy); bx[12] = kShC3[3] * -6.0f * xz;
+    by[12] = kShC3[3] * -6.0f * yz; bz[12] = kShC3[3] * (6.0f * zz - 3.0f * xx - 3.0f * yy);
+    b[13] = kShC3[4] * x * (4.0f * zz - xx - yy); bx[13] = kShC3[4] * (4.0f * zz - 3.0f * xx - yy);
+    by[13] = kShC3[4] * -2.0f * xy; bz[13] = kShC3[4] * 8.0f * xz;
+    b[14] = kShC3[5] * z * (xx - yy); bx[14] = kShC3[5] * 2.0f * xz; by[14] = kShC3[5] * -2.0f * yz;
+    bz[14] = kShC3[5] * (xx - yy);
+    b[15] = kShC3[6] * x * (xx - 3.0f * yy); bx[15] = kShC3[6] * (3.0f * xx - 3.0f * yy); by[15] = kShC3[6] * -6.0f * xy;
+}
+
+__global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, gs355_gaussians g,
+                                                                  const int32_t* __restrict__ radii,
+                                                                  const float* __restrict__ records,
+                                                                  const float* __restrict__ grads, gs355_gradients out)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= g.P) return;
+    const size_t si = (size_t)i;
+    const int M = f.sh_coeffs;
+    const bool alive = radii[i] > 0;
+    float dmean[3] = {0.f, 0.f, 0.f}, d2[3] = {0.f, 0.f, 0.f}, dscale[3] = {0.f, 0.f, 0.f};
+    float drot[4] = {0.f, 0.f, 0.f, 0.f}, dcov[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, dcol[3] = {0.f, 0.f, 0.f};
+    float dop = 0.f;
+    float b[16], gcol[3] = {0.f, 0.f, 0.f};
+    int K = 0;
+    if (alive) {
+        const float* __restrict__ V = f.viewmatrix;
+        const float* __restrict__ Pm = f.projmatrix;
+        const float4* __restrict__ A4 = reinterpret_cast<const float4*>(grads + si * kGradFloats);
+        const float4 A0 = A4[0], A1 = A4[1], A2 = A4[2];
+        const float g_px = A0.x, g_py = A0.y, gA = A0.z, gB = A0.w, gC = A1.x;
+        dop = A1.y;
+        dcol[0] = A1.z; dcol[1] = A1.w; dcol[2] = A2.x;
+        const float g_depth = A2.y;
+        const float x = g.means3D[3 * si], y = g.means3D[3 * si + 1], z = g.means3D[3 * si + 2];
+
+        // ---- pixel position ----
+        const float phx = Pm[0] * x + Pm[4] * y + Pm[8] * z + Pm[12];
+        const float phy = Pm[1] * x + Pm[5] * y + Pm[9] * z + Pm[13];
+        const float phw = Pm[3] * x + Pm[7] * y + Pm[11] * z + Pm[15];
+        const float pw = 1.0f / (phw + 0.0000001f);
+        d2[0] = g_px * 0.5f * (float)f.W;
+        d2[1] = g_py * 0.5f * (float)f.H;
+        const float d_phx = d2[0] * pw, d_phy = d2[1] * pw;
+        const float d_phw = -(pw * pw) * (phx * d2[0] + phy * d2[1]);
+#pragma unroll
+        for (int k = 0; k < 3; ++k) dmean[k] = Pm[4 * k] * d_phx + Pm[4 * k + 1] * d_phy + Pm[4 * k + 3] * d_phw;
+
+        // ---- 3-D covariance ----
+        float S[6], s[3] = {0.f, 0.f, 0.f}, q[4] = {0.f, 0.f, 0.f, 0.f}, R[3][3] = {};
+        if (g.cov3D_precomp) {
+#pragma unroll
+            for (int k = 0; k < 6; ++k) S[k] = g.cov3D_precomp[6 * si + k];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 3; ++k) s[k] = f.scale_modifier * g.scales[3 * si + k];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) q[k] = g.rotations[4 * si + k];
+            const float r = q[0], qx = q[1], qy = q[2], qz = q[3];
+            R[0][0] = 1.f - 2.f * (qy * qy + qz * qz); R[0][1] = 2.f * (qx * qy - r * qz); R[0][2] = 2.f * (qx * qz + r * qy);
+            R[1][0] = 2.f * (qx * qy + r * qz); R[1][1] = 1.f - 2.f * (qx * qx + qz * qz); R[1][2] = 2.f * (qy * qz - r * qx);
+            R[2][0] = 2.f * (qx * qz - r * qy); R[2][1] = 2.f * (qy * qz + r * qx); R[2][2] = 1.f - 2.f * (qx * qx + qy * qy);
+            int n = 0;
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+#pragma unroll
+                for (int c = a; c < 3; ++c)
+                    S[n++] = R[a][0] * s[0] * R[c][0] * s[0] + R[a][1] * s[1] * R[c][1] * s[1] + R[a][2] * s[2] * R[c][2] * s[2];
+        }
+        const float Sm[3][3] = {{S[0], S[1], S[2]}, {S[1], S[3], S[4]}, {S[2], S[4], S[5]}};
+
+        // ---- Jacobian of the projection, 2-D covariance, conic ----
+        const float pvx = V[0] * x + V[4] * y + V[8] * z + V[12];
+        const float pvy = V[1] * x + V[5] * y + V[9] * z + V[13];
+        const float tz = V[2] * x + V[6] * y + V[10] * z + V[14];
+        const float limx = 1.3f * f.tanfovx, limy = 1.3f * f.tanfovy;
+        const float rx = pvx / tz, ry = pvy / tz;
+        const float cx = rx > limx ? limx : rx < -limx ? -limx : 0.0f;  // non-zero: clamped to +-lim
+        const float cy = ry > limy ? limy : ry < -limy ? -limy : 0.0f;
+        const float tx = cx != 0.0f ? cx * tz : pvx, ty = cy != 0.0f ? cy * tz : pvy;
+        const float itz = 1.0f / tz, itz2 = itz * itz;
+        const float J00 = f.focal_x * itz, J02 = -(f.focal_x * tx) * itz2;
+        const float J11 = f.focal_y * itz, J12 = -(f.focal_y * ty) * itz2;
+        float a0[3], a1[3], Sa0[3], Sa1[3];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            a0[k] = J00 * V[4 * k] + J02 * V[4 * k + 2];
+            a1[k] = J11 * V[4 * k + 1] + J12 * V[4 * k + 2];
+        }
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            Sa0[k] = Sm[k][0] * a0[0] + Sm[k][1] * a0[1] + Sm[k][2] * a0[2];
+            Sa1[k] = Sm[k][0] * a1[0] + Sm[k][1] * a1[1] + Sm[k][2] * a1[2];
+        }
+        const float ca = a0[0] * Sa0[0] + a0[1] * Sa0[1] + a0[2] * Sa0[2] + 0.3f;
+        const float cb = a0[0] * Sa1[0] + a0[1] * Sa1[1] + a0[2] * Sa1[2];
+        const float cc = a1[0] * Sa1[0] + a1[1] * Sa1[1] + a1[2] * Sa1[2] + 0.3f;
+        const float D = 1.0f / (ca * cc - cb * cb), D2 = D * D;
+        const float d_ca = gA * (-cc * cc * D2) + gB * (cb * cc * D2) + gC * (D - ca * cc * D2);
+        const float d_cb = gA * (2.f * cb * cc * D2) + gB * (-D - 2.f * cb * cb * D2) + gC * (2.f * ca * cb * D2);
+        const float d_cc = gA * (D - ca * cc * D2) + gB * (ca * cb * D2) + gC * (-ca * ca * D2);
+        // symmetric gradient of the 3-D covariance, packed with the off-diagonal entries counted once each
+        float dS[3][3];
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+#pragma unroll
+            for (int l = 0; l < 3; ++l)
+                dS[k][l] = d_ca * a0[k] * a0[l] + d_cb * 0.5f * (a0[k] * a1[l] + a1[k] * a0[l]) + d_cc * a1[k] * a1[l];
+        float d_J00 = 0.f, d_J02 = 0.f, d_J11 = 0.f, d_J12 = 0.f;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const float d_a0 = 2.f * d_ca * Sa0[k] + d_cb * Sa1[k];
+            const float d_a1 = 2.f * d_cc * Sa1[k] + d_cb * Sa0[k];
+            d_J00 += d_a0 * V[4 * k];
+            d_J02 += d_a0 * V[4 * k + 2];
+            d_J11 += d_a1 * V[4 * k + 1];
+            d_J12 += d_a1 * V[4 * k + 2];
+        }
+        const float itz3 = itz2 * itz;
+        const float d_tx = d_J02 * (-f.focal_x * itz2), d_ty = d_J12 * (-f.focal_y * itz2);
+        const float d_tz = d_J00 * (-f.focal_x * itz2) + d_J11 * (-f.focal_y * itz2) +
+                           d_J02 * (2.f * f.focal_x * tx * itz3) + d_J12 * (2.f * f.focal_y * ty * itz3);
+        const float d_pvx = cx != 0.0f ? 0.0f : d_tx, d_pvy = cy != 0.0f ? 0.0f : d_ty;
+        const float d_pvz = d_tz + cx * d_tx + cy * d_ty + g_depth;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) dmean[k] += V[4 * k] * d_pvx + V[4 * k + 1] * d_pvy + V[4 * k + 2] * d_pvz;
+
+        if (g.cov3D_precomp) {
+            dcov[0] = dS[0][0]; dcov[1] = 2.f * dS[0][1]; dcov[2] = 2.f * dS[0][2];
+            dcov[3] = dS[1][1]; dcov[4] = 2.f * dS[1][2]; dcov[5] = dS[2][2];
+        } else {
+            // Sigma = L L^T with L = R diag(s): dL = 2 dS L
+            float dR[3][3];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) {
+                float ds = 0.f;
+#pragma unroll
+                for (int a = 0; a < 3; ++a) {
+                    const float dL = 2.f * (dS[a][0] * R[0][k] + dS[a][1] * R[1][k] + dS[a][2] * R[2][k]) * s[k];
+                    ds += dL * R[a][k];
+                    dR[a][k] = dL * s[k];
+                }
+                dscale[k] = ds * f.scale_modifier;
+            }
+            const float r = q[0], qx = q[1], qy = q[2], qz = q[3];
+            drot[0] = 2.f * (-qz * dR[0][1] + qy * dR[0][2] + qz * dR[1][0] - qx * dR[1][2] - qy * dR[2][0] + qx * dR[2][1]);
+            drot[1] = 2.f * (qy * dR[0][1] + qz * dR[0][2] + qy * dR[1][0] - 2.f * qx * dR[1][1] - r * dR[1][2] +
+                             qz * dR[2][0] + r * dR[2][1] - 2.f * qx * dR[2][2]);
+            drot[2] = 2.f * (-2.f * qy * dR[0][0] + qx * dR[0][1] + r * dR[0][2] + qx * dR[1][0] + qz * dR[1][2] -
+                             r * dR[2][0] + qz * dR[2][1] - 2.f * qy * dR[2][2]);
+            drot[3] = 2.f * (-2.f * qz * dR[0][0] - r * dR[0][1] + qx * dR[0][2] + r * dR[1][0] - 2.f * qz * dR[1][1] +
+                             qy * dR[1][2] + qx * dR[2][0] + qy * dR[2][1]);
+        }
+
+        // ---- colour: SH coefficients and view direction ----
+        if (g.shs) {
+            const float dirx = x - f.campos[0], diry = y - f.campos[1], dirz = z - f.campos[2];
+            const float inv_len = 1.0f / sqrtf(dirx * dirx + diry * diry + dirz * dirz);
+            const float nx = dirx * inv_len, ny = diry * inv_len, nz = dirz * inv_len;
+            float bx[16], by[16], bz[16];
+            sh_basis_grad(f.sh_degree, nx, ny, nz, b, bx, by, bz);
+            K = (f.sh_degree + 1) * (f.sh_degree + 1);
+            // the forward pass clamped the colour at zero: a zero in the record means no gradient
+            const float* __restrict__ rec = records + si * kRecordFloats;
+            gcol[0] = rec[6] > 0.0f ? dcol[0] : 0.0f;
+            gcol[1] = rec[7] > 0.0f ? dcol[1] : 0.0f;
+            gcol[2] = rec[8] > 0.0f ? dcol[2] : 0.0f;
+            if (f.sh_degree > 0) {
+                const float* __restrict__ sh = g.shs + si * M * 3;
+                float dn[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+                for (int k = 1; k < 16; ++k) {
+                    if (k < K) {
+                        const float t = gcol[0] * sh[3 * k] + gcol[1] * sh[3 * k + 1] + gcol[2] * sh[3 * k + 2];
+                        dn[0] += t * bx[k];
+                        dn[1] += t * by[k];
+                        dn[2] += t * bz[k];
+                    }
+                }
+                const float dot = nx * dn[0] + ny * dn[1] + nz * dn[2];
+                dmean[0] += (dn[0] - nx * dot) * inv_len;
+                dmean[1] += (dn[1] - ny * dot) * inv_len;
+                dmean[2] += (dn[2] - nz * dot) * inv_len;
+            }
+        }
+    }
+
+    if (out.means3D)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) out.means3D[3 * si + k] = dmean[k];
+    if (out.means2D)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) out.means2D[3 * si + k] = d2[k];
+    if (out.opacities) out.opacities[i] = dop;
+    if (out.colors_precomp)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) out.colors_precomp[3 * si + k] = dcol[k];
+    if (out.scales)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) out.scales[3 * si + k] = dscale[k];
+    if (out.rotations)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) out.rotations[4 * si + k] = drot[k];
+    if (out.cov3D_precomp)
+#pragma unroll
+        for (int k = 0; k < 6; ++k) out.cov3D_precomp[6 * si + k] = dcov[k];
+    if (out.shs) {
+        float* __restrict__ o = out.shs + si * M * 3;
+        for (int k = 0; k < M; ++k) {
+            const float bk = (alive && k < K) ? b[k < 16 ? k : 0] : 0.0f;
+            o[3 * k] = bk * gcol[0];
+            o[3 * k + 1] = bk * gcol[1];
+            o[3 * k + 2] = bk * gcol[2];
+        }
+    }
+}
+
+}  // namespace
+
+int launch_render_backward(const FrameArgs& f, const gs355_gaussians& g, const gs355_header* header,
+                           const uint32_t* ranges, const uint32_t* values, const float* records,
+                           const gs355_backward_inputs& in, float* grads, const gs355_gradients& out, hipStream_t s)
+{
+    if (g.P == 0) return GS355_OK;
+    int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(grads), (size_t)g.P * kGradFloats, 0u, s);
+    if (rc) return rc;
+    const int tiles = f.grid_x * f.grid_y;
+    hipLaunchKernelGGL(blend_backward_kernel, dim3(tiles), dim3(256), 0, s, f, header, ranges, values, records,
+                       in.image, in.depth, in.alpha, in.dL_dimage, in.dL_ddepth, in.dL_dalpha, grads);
+    GS355_CHECK_LAUNCH("blend backward");
+    hipLaunchKernelGGL(preprocess_backward_kernel, dim3((g.P + 255) / 256), dim3(256), 0, s, f, g, in.radii, records,
+                       grads, out);
+    GS355_CHECK_LAUNCH("preprocess backward");
+    return GS355_OK;
+}
+
+}  // namespace gs355

@@ -89,6 +89,10 @@ int launch_ranges(const gs355_header* header, uint32_t n_cap, const uint64_t* ke
 int launch_blend(const FrameArgs& f, const gs355_header* header, const uint32_t* ranges, const uint32_t* values, const float* records,
                  float* image, float* depth, float* alpha, bool cull, hipStream_t s);
 
+int launch_render_backward(const FrameArgs& f, const gs355_gaussians& g, const gs355_header* header,
+                           const uint32_t* ranges, const uint32_t* values, const float* records,
+                           const gs355_backward_inputs& in, float* grads, const gs355_gradients& out, hipStream_t s);
+
 // Orders one wavefront's LDS writes before its later LDS reads (and the reverse).  The hardware executes a
 // wavefront's LDS instructions in order; the fences (wavefront scope: no instructions) and the scheduling
 // barrier keep the compiler from moving the accesses across this point.

@@ -129,6 +129,7 @@ class GaussianModel(nn.Module):
         self.renderer = _placeholder_renderer(self.background)
         self._cache = {}
         self._radii = self._visibility_filter = self._radii_all = None
+        self.viewspace_points = None  # training: zero tensor whose .grad receives the screen-space gradient
 
     # `visibility_filter` (bool[P]) and `radii` (int32 of the visible Gaussians) are by-products the reference
     # leaves on the model for its training loop.  The fused single-pass frame derives them from the rasterizer's
@@ -258,8 +259,11 @@ class GaussianModel(nn.Module):
                                                rotations=rotations, cov3D_precomp=cov3D_precomp)
         return radii_pure > 0
 
-    @torch.no_grad()
     def forward(self, viewpoint_camera, scaling_modifier=1.0, override_color=None, render_exclude_filter=None):
+        """origin_gs/gs_model.py:112-228.  Under torch.no_grad() (the inference engine) this is the plain frame.
+        In training mode with gradients enabled every Gaussian is rendered (no gather), the frame is
+        differentiable with respect to the parameters, and `viewspace_points` receives the screen-space gradient
+        that the reference's densification reads (:129-139, :225-236)."""
         viewpoint_camera = viewpoint_camera.to(self._xyz.device)
         fused = (self.fuse_prefilter and not self.training and render_exclude_filter is None
                  and scaling_modifier == 1.0)  # the reference's prefilter always uses scale modifier 1
@@ -292,9 +296,14 @@ class GaussianModel(nn.Module):
             pick = lambda t: None if t is None else t[mask]  # noqa: E731
             means3D, shs, colors_precomp, opacity = pick(means3D), pick(shs), pick(colors_precomp), pick(opacity)
             scales, rotations, cov3D_precomp = pick(scales), pick(rotations), pick(cov3D_precomp)
+        screenspace_points = None
+        if self.training and torch.is_grad_enabled():
+            screenspace_points = torch.zeros_like(means3D, requires_grad=True) + 0
+            screenspace_points.retain_grad()
         rendered_image, radii, _ = self.renderer(
-            means3D=means3D, means2D=None, shs=shs, colors_precomp=colors_precomp, opacities=opacity, scales=scales,
-            rotations=rotations, cov3D_precomp=cov3D_precomp)
+            means3D=means3D, means2D=screenspace_points, shs=shs, colors_precomp=colors_precomp, opacities=opacity,
+            scales=scales, rotations=rotations, cov3D_precomp=cov3D_precomp)
+        self.viewspace_points = screenspace_points
         self._radii_all, self.visibility_filter, self.radii = None, voxel_visible_mask, radii
         return rendered_image
 

@@ -219,6 +219,7 @@ class FrameOutputs:
         self.c = o
         self.num_keys = 0
         self.num_visible = 0
+        self.key_capacity = 0  # the capacity the frame was finally rendered with (what a backward pass must pass)
 
 
 def run_stages(inputs: FrameInputs, outputs: FrameOutputs, ws: Workspace, n_cap: int, stage_mask: int):
@@ -265,7 +266,39 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
         out.num_visible = int(ws.header_host[2]) & 0xFFFFFFFF
         ws.frames += 1
         if not overflow:
+            out.key_capacity = n_cap
             return out
         ws.overflows += 1
         ws.key_capacity = int(total * _KEY_HEADROOM) + 4096
     raise RuntimeError("key capacity still insufficient after regrowing (needed %d keys)" % out.num_keys)
+
+
+GRAD_NAMES = ("means3D", "means2D", "shs", "colors_precomp", "opacities", "scales", "rotations", "cov3D_precomp")
+
+
+def render_backward(inputs: FrameInputs, out: FrameOutputs, workspace: torch.Tensor, dL_dimage: torch.Tensor,
+                    dL_ddepth: Optional[torch.Tensor] = None, dL_dalpha: Optional[torch.Tensor] = None,
+                    want=GRAD_NAMES) -> Dict[str, torch.Tensor]:
+    """Gradients of a frame rendered by `render` (gs355_render_backward).  `workspace` is the device buffer that
+    frame was rendered in, untouched since; `out` its outputs.  Returns contiguous fp32 tensors for the names in
+    `want` whose inputs were given: means3D [P,3], means2D [P,3], shs [P,M,3] / colors_precomp [P,3], opacities [P],
+    scales [P,3], rotations [P,4] / cov3D_precomp [P,6]."""
+    dev, P, H, W = inputs.device, inputs.P, inputs.height, inputs.width
+    given = {"means3D": inputs.means3D, "means2D": inputs.means3D, "shs": inputs.shs,
+             "colors_precomp": inputs.colors_precomp, "opacities": inputs.opacities, "scales": inputs.scales,
+             "rotations": inputs.rotations, "cov3D_precomp": inputs.cov3D_precomp}
+    grads = {n: torch.empty_like(given[n]) for n in want if given[n] is not None}
+    gi = _dev_f32(dL_dimage, dev, "dL_dimage", (3, H, W))
+    gd = _dev_f32(dL_ddepth, dev, "dL_ddepth", (H, W))
+    ga = _dev_f32(dL_dalpha, dev, "dL_dalpha", (H, W))
+    if gd is not None and out.depth is None or ga is not None and out.alpha is None:
+        raise ValueError("a gradient arrives for an output the forward pass did not produce")
+    b = _lib.BackwardInputs(_ptr(out.image), _ptr(out.depth), _ptr(out.alpha), _ptr(out.radii), _ptr(gi), _ptr(gd),
+                            _ptr(ga))
+    g = _lib.Gradients(*[_ptr(grads.get(n)) for n in GRAD_NAMES])
+    scratch = torch.empty(P * _lib.GRAD_FLOATS + 64, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    _lib.check(_lib.load().gs355_render_backward(C.byref(inputs.frame), C.byref(inputs.gaussians), workspace.data_ptr(),
+                                                 workspace.numel(), int(out.key_capacity), C.byref(b),
+                                                 scratch.data_ptr(), scratch.numel() * 4, C.byref(g), stream))
+    return grads

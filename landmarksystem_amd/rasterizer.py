@@ -20,11 +20,14 @@ octree_gs/gs_model.py:8) and use them as follows:
   - `rasterizer.visible_filter(means3D=..., scales=..., rotations=...,
     cov3D_precomp=...)` returns radii only (:327-329).
 
-Forward only: the returned tensors never require grad (the reference's
-inference engine calls the model under torch.no_grad(),
-landmark/render/inference_engine/inference_engine.py:89-94).
+Under torch.no_grad() (the reference's inference engine,
+landmark/render/inference_engine/inference_engine.py:89-94) the call is the
+plain forward pass.  When gradients are enabled and an input requires them
+(the reference's training loop, benchmarks/nerf/origin_gs/gs_trainer.py:
+117-124), the call goes through an autograd function whose backward is the
+library's backward pass; `means2D` then receives the screen-space gradient
+the reference's densification reads (gaussian_encoding.py:729-743).
 """
-import warnings
 from typing import NamedTuple, Optional
 
 import torch
@@ -48,20 +51,54 @@ class GaussianRasterizationSettings(NamedTuple):
     debug: bool
 
 
-_warned_grad = False
+_INPUT_NAMES = ("means3D", "means2D", "opacities", "shs", "colors_precomp", "scales", "rotations", "cov3D_precomp")
 
 
-def _note_forward_only(*tensors):
-    global _warned_grad
-    if _warned_grad or not torch.is_grad_enabled():
-        return
-    if any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors):
-        _warned_grad = True
-        warnings.warn(
-            "landmarksystem_amd.GaussianRasterizer is forward-only: outputs do not carry gradients "
-            "(call it under torch.no_grad(), as the reference's inference engine does)",
-            stacklevel=3,
-        )
+class _RasterizeGaussians(torch.autograd.Function):
+    """forward(): one frame in a workspace of its own, kept until backward() has read it."""
+
+    @staticmethod
+    def forward(ctx, settings, means3D, means2D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp):
+        inputs = pipeline.FrameInputs(settings, means3D, opacities=opacities, shs=shs, colors_precomp=colors_precomp,
+                                      scales=scales, rotations=rotations, cov3D_precomp=cov3D_precomp)
+        ws = pipeline.default_workspace(inputs.device)
+        out = pipeline.render(inputs, ws=ws)
+        # the next frame on this stream gets a fresh buffer; this one lives until the backward pass is done
+        ctx.workspace, ws.buffer = ws.buffer, None
+        ctx.settings, ctx.out = settings, out
+        ctx.set_materialize_grads(False)
+        ctx.save_for_backward(means3D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp)
+        ctx.means2D_like = None if means2D is None else (means2D.shape, means2D.dtype)
+        ctx.mark_non_differentiable(out.radii)
+        return out.image, out.radii, out.depth, out.alpha
+
+    @staticmethod
+    def backward(ctx, g_image, _g_radii, g_depth, g_alpha):
+        means3D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp = ctx.saved_tensors
+        originals = dict(means3D=means3D, opacities=opacities, shs=shs, colors_precomp=colors_precomp, scales=scales,
+                         rotations=rotations, cov3D_precomp=cov3D_precomp)
+        needs = dict(zip(_INPUT_NAMES, ctx.needs_input_grad[1:]))
+        if g_image is None and g_depth is None and g_alpha is None:
+            return (None,) * 9
+        inputs = pipeline.FrameInputs(ctx.settings, means3D, opacities=opacities, shs=shs,
+                                      colors_precomp=colors_precomp, scales=scales, rotations=rotations,
+                                      cov3D_precomp=cov3D_precomp)
+        if g_image is None:
+            g_image = torch.zeros_like(ctx.out.image)
+        want = [n for n in _INPUT_NAMES if needs[n]]
+        grads = pipeline.render_backward(inputs, ctx.out, ctx.workspace, g_image, g_depth, g_alpha, want=want)
+        ctx.workspace = None
+        result = [None]
+        for n in _INPUT_NAMES:
+            g = grads.get(n)
+            if g is not None:
+                if n == "means2D":
+                    shape, dtype = ctx.means2D_like
+                else:
+                    shape, dtype = originals[n].shape, originals[n].dtype
+                g = g.reshape(shape).to(dtype)
+            result.append(g)
+        return tuple(result)
 
 
 class GaussianRasterizer(nn.Module):
@@ -83,12 +120,17 @@ class GaussianRasterizer(nn.Module):
     def forward(self, means3D, means2D=None, opacities=None, shs=None, colors_precomp=None, scales=None,
                 rotations=None, cov3D_precomp=None):
         """Returns (image f32[3,H,W], radii i32[P], depth f32[1,H,W]).
-        `means2D` only carries screen-space gradients in the reference's
-        training loop and is ignored here.  Alpha (1 - final transmittance,
-        f32[1,H,W]) is left in `self.last_alpha`."""
-        _note_forward_only(means3D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp)
+        `means2D` takes no part in the forward pass; when it requires grad it
+        receives the screen-space gradient (normalised device units, third
+        component zero).  Alpha (1 - final transmittance, f32[1,H,W]) is left
+        in `self.last_alpha`; image, depth and alpha are all differentiable."""
         if opacities is None:
             raise ValueError("opacities is required")
+        tensors = (means3D, means2D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp)
+        if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors):
+            image, radii, depth, alpha = _RasterizeGaussians.apply(self.raster_settings, *tensors)
+            self.last_depth, self.last_alpha, self.last_num_keys = depth, alpha, 0
+            return image, radii, depth
         inputs = pipeline.FrameInputs(self.raster_settings, means3D, opacities=opacities, shs=shs,
                                       colors_precomp=colors_precomp, scales=scales, rotations=rotations,
                                       cov3D_precomp=cov3D_precomp)

@@ -1,4 +1,4 @@
-"""Compile the C oracle (oracle/gs_oracle.c) into oracle/libgs_oracle.so with gcc.
+"""Compile the C oracle (oracle/gs_oracle.c, oracle/gs_oracle_backward.c) into oracle/libgs_oracle.so with gcc.
 
 Test infrastructure only: the shipped library never links or loads this.
 There is no buildable reference source for this path (the rasterizer is an
@@ -9,7 +9,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRC = os.path.join(HERE, "gs_oracle.c")
+SRCS = [os.path.join(HERE, "gs_oracle.c"), os.path.join(HERE, "gs_oracle_backward.c")]
 OUT = os.path.join(HERE, "libgs_oracle.so")
 
 # -ffp-contract=off: the integer pipeline (depth bits, radius, tile rectangle)
@@ -18,9 +18,9 @@ FLAGS = ["-O2", "-ffp-contract=off", "-fno-fast-math", "-fopenmp", "-shared", "-
 
 
 def build(force: bool = True) -> str:
-    if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= os.path.getmtime(SRC):
+    if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= max(os.path.getmtime(s) for s in SRCS):
         return OUT
-    cmd = ["gcc", *FLAGS, "-o", OUT, SRC, "-lm"]
+    cmd = ["gcc", *FLAGS, "-o", OUT, *SRCS, "-lm"]
     subprocess.run(cmd, check=True)
     return OUT
 

@@ -238,3 +238,35 @@ def render(frame: Frame, g: Gaussians, keep_intermediates: bool = True):
         out.update(pre=pre, offsets=offsets, keys=keys, values=vals, sorted_keys=skeys, sorted_values=svals,
                    ranges=ranges)
     return out
+
+
+GRAD_SLOTS = 10  # d/dpx, d/dpy, d/dconic (x, y, z), d/dopacity, d/drgb (3), d/ddepth
+
+
+def render_backward(frame: Frame, g: Gaussians, fwd, g_image, g_depth=None, g_alpha=None):
+    """Gradients of sum(image * g_image) [+ depth * g_depth + alpha * g_alpha] with respect to every input of
+    `render`, from the intermediates `fwd` that `render` returned (oracle/gs_oracle_backward.c).  All float64."""
+    P, M = g.P, g.sh_coeffs
+    H, W = frame.image_height, frame.image_width
+    pre = fwd["pre"]
+    acc = np.zeros((P, GRAD_SLOTS), np.float64)
+    cf = frame._c(M)
+    gi = _f32(g_image, (3, H, W))
+    gd = _f32(g_depth, (H, W)) if g_depth is not None else None
+    ga = _f32(g_alpha, (H, W)) if g_alpha is not None else None
+    ranges = np.ascontiguousarray(fwd["ranges"], np.uint32)
+    vals = np.ascontiguousarray(fwd["sorted_values"], np.uint32)
+    lib().orc_blend_backward(C.byref(cf), _ptr(ranges), _ptr(vals), _ptr(pre["xy"]), _ptr(pre["conic_opacity"]),
+                             _ptr(pre["rgb"]), _ptr(pre["depth"]), _ptr(gi), _ptr(gd), _ptr(ga), _ptr(acc))
+    out = dict(acc=acc, means3D=np.zeros((P, 3)), means2D=np.zeros((P, 3)), opacities=np.zeros(P))
+    out["shs" if g.shs is not None else "colors_precomp"] = np.zeros((P, M, 3) if g.shs is not None else (P, 3))
+    if g.cov3D_precomp is not None:
+        out["cov3D_precomp"] = np.zeros((P, 6))
+    else:
+        out["scales"], out["rotations"] = np.zeros((P, 3)), np.zeros((P, 4))
+    cg = g._c()
+    lib().orc_preprocess_backward(C.byref(cf), C.byref(cg), _ptr(np.ascontiguousarray(pre["radii"], np.int32)),
+                                  _ptr(acc), *[_ptr(out.get(k)) for k in
+                                               ("means3D", "means2D", "shs", "colors_precomp", "opacities", "scales",
+                                                "rotations", "cov3D_precomp")])
+    return out

@@ -159,7 +159,7 @@ def make_keys(pre, grid_x):
     w = (rect[:, 2] - rect[:, 0])[idx]
     ty = rect[idx, 1] + local // torch.clamp_min(w, 1)
     tx = rect[idx, 0] + local % torch.clamp_min(w, 1)
-    depth_bits = pre["depth"].view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    depth_bits = pre["depth"].detach().to(torch.float32).view(torch.int32).to(torch.int64) & 0xFFFFFFFF
     keys = ((ty * grid_x + tx) << 32) | depth_bits[idx]
     return keys, idx.to(torch.int32), offsets
 
@@ -178,9 +178,14 @@ def tile_ranges(skeys, tiles):
     return torch.stack([torch.where(empty, torch.zeros_like(lo), lo), torch.where(empty, torch.zeros_like(hi), hi)], 1)
 
 
-def blend_tile(fr, t, ranges, svals, pre):
+def blend_tile(fr, t, ranges, svals, pre, straight_through=False):
     """One 16x16 tile, all its Gaussians at once: [n,256] elementwise passes
-    and a sequential cumulative product for the transmittance."""
+    and a sequential cumulative product for the transmittance.  Differentiable
+    by torch.autograd in the dtype of `pre` (fp32 or fp64); `straight_through`
+    lets the gradient through min(0.99, .) unchanged, as the published backward
+    pass of the rasterizer does (the forward value may then differ from the
+    clamp's in the last bit, so it is used for gradient checks only)."""
+    dt = pre["xy"].dtype
     W, H = fr["image_width"], fr["image_height"]
     gx = (W + 15) // 16
     lo, hi = int(ranges[t, 0]), int(ranges[t, 1])
@@ -188,35 +193,39 @@ def blend_tile(fr, t, ranges, svals, pre):
     py = (t // gx) * 16 + torch.arange(16).repeat_interleave(16)
     bg = fr["bg"]
     if hi == lo:
-        T = torch.ones(256)
-        return px, py, bg[:, None] * T[None, :], torch.zeros(256), 1.0 - T, 0
+        T = torch.ones(256, dtype=dt)
+        return px, py, bg[:, None] * T[None, :], torch.zeros(256, dtype=dt), 1.0 - T, 0
     g = svals[lo:hi].long()
     xy, co, col, dep = pre["xy"][g], pre["conic_opacity"][g], pre["rgb"][g], pre["depth"][g]
-    dx = xy[:, 0:1] - px[None, :].float()
-    dy = xy[:, 1:2] - py[None, :].float()
+    dx = xy[:, 0:1] - px[None, :].to(dt)
+    dy = xy[:, 1:2] - py[None, :].to(dt)
     power = -0.5 * (co[:, 0:1] * dx * dx + co[:, 2:3] * dy * dy) - co[:, 1:2] * dx * dy
     alpha = torch.clamp_max(co[:, 3:4] * torch.exp(power), 0.99)
+    if straight_through:
+        raw = co[:, 3:4] * torch.exp(power)
+        alpha = raw + (alpha - raw).detach()
     valid = (power <= 0) & (alpha >= 1.0 / 255.0)
     a = torch.where(valid, alpha, torch.zeros_like(alpha))
     test_T = torch.cumprod(1.0 - a, dim=0)
     stopped = torch.cumsum((valid & (test_T < 0.0001)).to(torch.int32), 0) > 0
-    T_before = torch.cat([torch.ones(1, 256), test_T[:-1]], 0)
+    T_before = torch.cat([torch.ones(1, 256, dtype=dt), test_T[:-1]], 0)
     w = torch.where(valid & ~stopped, a * T_before, torch.zeros_like(a))
     C = col.t() @ w  # [3,256]
     D = dep[None, :] @ w
     T_final = torch.where(stopped, torch.ones_like(test_T), test_T).amin(0)
-    T_final = torch.where(stopped[0], torch.ones(256), T_final)
+    T_final = torch.where(stopped[0], torch.ones(256, dtype=dt), T_final)
     return px, py, C + bg[:, None] * T_final[None, :], D[0], 1.0 - T_final, (hi - lo)
 
 
-def blend(fr, ranges, svals, pre, tiles=None):
+def blend(fr, ranges, svals, pre, tiles=None, straight_through=False):
     W, H = fr["image_width"], fr["image_height"]
     gx, gy = (W + 15) // 16, (H + 15) // 16
-    image = torch.zeros(3, H, W)
-    depth = torch.zeros(H, W)
-    alpha = torch.zeros(H, W)
+    dt = pre["xy"].dtype
+    image = torch.zeros(3, H, W, dtype=dt)
+    depth = torch.zeros(H, W, dtype=dt)
+    alpha = torch.zeros(H, W, dtype=dt)
     for t in (range(gx * gy) if tiles is None else tiles):
-        px, py, C, D, A, _ = blend_tile(fr, t, ranges, svals, pre)
+        px, py, C, D, A, _ = blend_tile(fr, t, ranges, svals, pre, straight_through)
         ok = (px < W) & (py < H)
         image[:, py[ok], px[ok]] = C[:, ok]
         depth[py[ok], px[ok]] = D[ok]
@@ -224,13 +233,13 @@ def blend(fr, ranges, svals, pre, tiles=None):
     return image, depth, alpha
 
 
-def render(fr, means3D, opacities, **kw):
+def render(fr, means3D, opacities, straight_through=False, **kw):
     pre = preprocess(fr, means3D, opacities, **kw)
     gx, gy = (fr["image_width"] + 15) // 16, (fr["image_height"] + 15) // 16
     keys, vals, offsets = make_keys(pre, gx)
     skeys, svals = sort_pairs(keys, vals)
     ranges = tile_ranges(skeys, gx * gy)
-    image, depth, alpha = blend(fr, ranges, svals, pre)
+    image, depth, alpha = blend(fr, ranges, svals, pre, straight_through=straight_through)
     return dict(image=image, depth=depth, alpha=alpha, radii=pre["radii"], pre=pre, keys=keys, values=vals,
                 offsets=offsets, sorted_keys=skeys, sorted_values=svals, ranges=ranges)
 

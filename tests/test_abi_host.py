@@ -34,6 +34,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(_lib.Outputs) == 4 * 8
     assert C.sizeof(_lib.Layout) == 18 * 8 + 4 * 4
     assert C.sizeof(_lib.AnchorLod) == 2 * 8 + 4 * 4 + 2 * 4
+    assert C.sizeof(_lib.BackwardInputs) == 7 * 8 and C.sizeof(_lib.Gradients) == 8 * 8
 
 
 def test_workspace_layout_is_aligned_ordered_and_sized():
@@ -137,6 +138,52 @@ def test_run_validates_before_any_hip_call():
     no_radii = _lib.Outputs()
     no_radii.image = 0x1000
     assert "radii is NULL" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, no_radii, _lib.STAGE_ALL)
+
+
+def test_render_backward_validates_before_any_hip_call():
+    lib = _lib.load()
+    size = C.c_size_t(0)
+    assert lib.gs355_backward_scratch_bytes(1000, C.byref(size)) == 0 and size.value >= 1000 * _lib.GRAD_FLOATS * 4
+    assert size.value % 256 == 0
+    assert "P must be" in _err(_lib.GS355_EINVAL, lib.gs355_backward_scratch_bytes, -1, C.byref(size))
+    assert _err(_lib.GS355_EINVAL, lib.gs355_backward_scratch_bytes, 10, None)
+
+    def bwd(f, g, ws, nbytes, cap, b, scratch, sbytes, grads):
+        return lib.gs355_render_backward(C.byref(f) if f else None, C.byref(g) if g else None, ws, nbytes, cap,
+                                         C.byref(b) if b else None, scratch, sbytes, C.byref(grads) if grads else None,
+                                         None)
+
+    f, g = _frame(), _gauss()
+    b = _lib.BackwardInputs(0x1000, None, None, 0x1000, 0x1000, None, None)
+    grads = _lib.Gradients()
+    grads.means3D = 0x1000
+    ok = (f, g, 0x1000, 1 << 30, 100, b, 0x1000, 1 << 20, grads)
+
+    def with_(**kw):
+        names = ("f", "g", "ws", "nbytes", "cap", "b", "scratch", "sbytes", "grads")
+        args = dict(zip(names, ok))
+        args.update(kw)
+        return [args[n] for n in names]
+
+    assert "frame is NULL" in _err(_lib.GS355_EINVAL, bwd, *with_(f=None))
+    assert "gaussians is NULL" in _err(_lib.GS355_EINVAL, bwd, *with_(g=None))
+    assert "backward inputs is NULL" in _err(_lib.GS355_EINVAL, bwd, *with_(b=None))
+    assert "gradients is NULL" in _err(_lib.GS355_EINVAL, bwd, *with_(grads=None))
+    assert "dL_dimage" in _err(_lib.GS355_EINVAL, bwd, *with_(b=_lib.BackwardInputs(0x1000, None, None, 0x1000, None, None, None)))
+    assert "forward depth" in _err(_lib.GS355_EINVAL, bwd, *with_(b=_lib.BackwardInputs(0x1000, None, None, 0x1000, 0x1000, 0x1000, None)))
+    assert "forward alpha" in _err(_lib.GS355_EINVAL, bwd, *with_(b=_lib.BackwardInputs(0x1000, None, None, 0x1000, 0x1000, None, 0x1000)))
+    assert "radii is NULL" in _err(_lib.GS355_EINVAL, bwd, *with_(b=_lib.BackwardInputs(0x1000, None, None, None, 0x1000, None, None)))
+    wrong = _lib.Gradients()
+    wrong.colors_precomp = 0x1000  # the frame was rendered from SH coefficients
+    assert "not given" in _err(_lib.GS355_EINVAL, bwd, *with_(grads=wrong))
+    assert "SHs or precomputed colors" in _err(_lib.GS355_EINVAL, bwd, *with_(g=_gauss(shs=True, colors=True)))
+    assert "workspace is NULL" in _err(_lib.GS355_EINVAL, bwd, *with_(ws=None))
+    assert "aligned" in _err(_lib.GS355_EINVAL, bwd, *with_(ws=0x1001))
+    assert "needed" in _err(_lib.GS355_ENOSPC, bwd, *with_(nbytes=1024))
+    assert "scratch is NULL" in _err(_lib.GS355_EINVAL, bwd, *with_(scratch=None))
+    assert "16-byte" in _err(_lib.GS355_EINVAL, bwd, *with_(scratch=0x1004))
+    assert "scratch has" in _err(_lib.GS355_ENOSPC, bwd, *with_(sbytes=16))
+    assert "32-bit" in _err(_lib.GS355_EOVERFLOW, bwd, *with_(cap=1 << 33))
 
 
 def test_visible_filter_validates():

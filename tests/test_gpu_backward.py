@@ -1,0 +1,193 @@
+"""GPU parity of the backward pass: gs355_render_backward (through the C ABI and through autograd) against the
+double-precision CPU oracle on identical seeded inputs.
+
+Bar: floating point, sums over pixels by atomics in arbitrary order.  Every gradient element must be within
+1e-4 of the tensor's largest magnitude plus 1e-3 of its own magnitude of the oracle's value (measured: a few 1e-6
+of the largest magnitude on these scenes)."""
+import numpy as np
+import pytest
+import torch
+
+from landmarksystem_amd import GaussianRasterizer, _lib, models, pipeline, scenes
+from oracle import c_oracle as co
+from tests.helpers import oracle_frame, oracle_gaussians, settings_for
+
+pytestmark = pytest.mark.gpu
+
+ABS_OF_MAX, REL = 1e-4, 1e-3
+
+
+def assert_grad_close(got, ref, name):
+    got = np.asarray(got, np.float64).reshape(ref.shape)
+    scale = np.abs(ref).max()
+    bound = ABS_OF_MAX * scale + REL * np.abs(ref)
+    err = np.abs(got - ref)
+    worst = np.unravel_index(np.argmax(err - bound), err.shape)
+    assert (err <= bound).all(), "%s: element %s differs by %g (value %g, largest magnitude %g)" % (
+        name, worst, err[worst], ref[worst], scale)
+
+
+def cotangents(scene, seed):
+    g = torch.Generator().manual_seed(seed)
+    H, W = scene.camera.height, scene.camera.width
+    return (torch.randn(3, H, W, generator=g), torch.randn(1, H, W, generator=g), torch.randn(1, H, W, generator=g))
+
+
+def oracle_backward(scene, gi, gd=None, ga=None, colors=None, cov=None, sh_degree=None):
+    cf = oracle_frame(scene, sh_degree=sh_degree)
+    cg = oracle_gaussians(scene, colors_precomp=None if colors is None else colors.numpy(),
+                          cov3D_precomp=None if cov is None else cov.numpy())
+    fwd = co.render(cf, cg)
+    return co.render_backward(cf, cg, fwd, gi.numpy(), None if gd is None else gd.numpy()[0],
+                              None if ga is None else ga.numpy()[0]), fwd
+
+
+def abi_backward(scene, device, gi, gd=None, ga=None, colors=None, cov=None, sh_degree=None, want=pipeline.GRAD_NAMES):
+    """Forward and backward through pipeline.render / pipeline.render_backward (thin ctypes calls of the C ABI)."""
+    s = settings_for(scene, device, sh_degree=sh_degree)
+    dev = lambda t: None if t is None else t.to(device)  # noqa: E731
+    inp = pipeline.FrameInputs(s, dev(scene.means3D), opacities=dev(scene.opacities),
+                               shs=None if colors is not None else dev(scene.shs), colors_precomp=dev(colors),
+                               scales=None if cov is not None else dev(scene.scales),
+                               rotations=None if cov is not None else dev(scene.rotations), cov3D_precomp=dev(cov))
+    ws = pipeline.Workspace(device)
+    out = pipeline.render(inp, ws=ws)
+    grads = pipeline.render_backward(inp, out, ws.buffer, dev(gi), dev(gd), dev(ga), want=want)
+    torch.cuda.synchronize()
+    return {k: v.cpu().numpy() for k, v in grads.items()}, out
+
+
+@pytest.mark.parametrize("deg", [0, 1, 2, 3])
+def test_backward_all_sh_degrees(gpu_device, deg):
+    scene = scenes.tiny_scene(P=400, width=100, height=70, sh_degree=deg, seed=3 + deg)
+    gi, gd, ga = cotangents(scene, deg)
+    ref, _ = oracle_backward(scene, gi, gd, ga)
+    got, _ = abi_backward(scene, gpu_device, gi, gd, ga)
+    assert set(got) == {"means3D", "means2D", "shs", "opacities", "scales", "rotations"}
+    for name, value in got.items():
+        assert_grad_close(value, ref[name], "deg %d %s" % (deg, name))
+
+
+def test_backward_with_precomputed_colours_and_covariances(gpu_device):
+    scene = scenes.tiny_scene(P=400, width=100, height=70, sh_degree=0, seed=9)
+    g = torch.Generator().manual_seed(1)
+    colors = torch.rand(scene.P, 3, generator=g)
+    cov = torch.from_numpy(np.stack([co.cov3d(scene.scales[i].numpy(), 1.0, scene.rotations[i].numpy())
+                                     for i in range(scene.P)]))
+    gi, gd, ga = cotangents(scene, 2)
+    ref, _ = oracle_backward(scene, gi, gd, ga, colors=colors, cov=cov, sh_degree=1)
+    got, _ = abi_backward(scene, gpu_device, gi, gd, ga, colors=colors, cov=cov, sh_degree=1)
+    assert set(got) == {"means3D", "means2D", "colors_precomp", "opacities", "cov3D_precomp"}
+    for name, value in got.items():
+        assert_grad_close(value, ref[name], name)
+
+
+def test_backward_image_gradient_only_and_selected_outputs(gpu_device):
+    """The training loop's case: a loss on the image alone; only some gradients requested."""
+    scene = scenes.config1()
+    gi, _, _ = cotangents(scene, 5)
+    ref, _ = oracle_backward(scene, gi)
+    got, _ = abi_backward(scene, gpu_device, gi, want=("means3D", "opacities", "means2D"))
+    assert set(got) == {"means3D", "opacities", "means2D"}
+    for name, value in got.items():
+        assert_grad_close(value, ref[name], name)
+
+
+@pytest.mark.parametrize("make,label", [
+    (lambda: scenes.config3(P=100_000, width=480, height=270), "C3/100k at 480x270"),
+    (lambda: scenes.config2(P=60_000, width=333, height=177), "C2/60k ragged image"),
+])
+def test_backward_scaled_down_configs(gpu_device, make, label):
+    scene = make()
+    gi, gd, ga = cotangents(scene, 8)
+    ref, fwd = oracle_backward(scene, gi, gd, ga)
+    got, out = abi_backward(scene, gpu_device, gi, gd, ga)
+    assert out.num_keys == fwd["num_keys"]
+    culled = fwd["radii"] == 0
+    assert culled.any()
+    for name, value in got.items():
+        assert_grad_close(value, ref[name], label + " " + name)
+        assert (value[culled] == 0).all(), name  # written, not left uninitialised
+
+
+def test_backward_of_a_crowded_tile_with_finished_pixels(gpu_device):
+    """Thousands of Gaussians over one small image: several staged batches per tile, pixels that reach the
+    1e-4 transmittance stop, and every Gaussian beyond the stop gets a zero gradient."""
+    scene = scenes.tiny_scene(P=3000, width=48, height=48, sh_degree=1, seed=31, spread=0.3, log_scale_mean=-1.2)
+    gi, gd, ga = cotangents(scene, 3)
+    ref, fwd = oracle_backward(scene, gi, gd, ga)
+    got, _ = abi_backward(scene, gpu_device, gi, gd, ga)
+    assert fwd["alpha"].max() > 0.9998
+    untouched = np.abs(ref["acc"]).sum(1) == 0
+    assert (untouched & (fwd["radii"] > 0)).sum() > 100
+    for name, value in got.items():
+        assert_grad_close(value, ref[name], name)
+    assert (got["opacities"][untouched] == 0).all()
+
+
+def test_autograd_through_the_rasterizer(gpu_device):
+    """GaussianRasterizer called as the reference's training loop calls it: gradients arrive on the leaves,
+    `means2D` carries the screen-space gradient, non-contiguous inputs get gradients of their own shape."""
+    scene = scenes.tiny_scene(P=500, width=96, height=64, sh_degree=2, seed=17)
+    gi, gd, ga = cotangents(scene, 1)
+    ref, _ = oracle_backward(scene, gi, gd, ga)
+    leaf = lambda t: t.to(gpu_device).clone().requires_grad_(True)  # noqa: E731
+    means, opac, shs, rots = leaf(scene.means3D), leaf(scene.opacities), leaf(scene.shs), leaf(scene.rotations)
+    scales6 = leaf(torch.cat([scene.scales, torch.ones(scene.P, 3)], 1))  # the models pass a strided [:, :3] slice
+    means2D = torch.zeros_like(means, requires_grad=True) + 0
+    means2D.retain_grad()
+    r = GaussianRasterizer(settings_for(scene, gpu_device))
+    image, radii, depth = r(means3D=means, means2D=means2D, shs=shs, colors_precomp=None, opacities=opac,
+                            scales=scales6[:, :3], rotations=rots, cov3D_precomp=None)
+    assert image.requires_grad and depth.requires_grad and r.last_alpha.requires_grad and not radii.requires_grad
+    loss = (image * gi.to(gpu_device)).sum() + (depth * gd.to(gpu_device)).sum() + (r.last_alpha * ga.to(gpu_device)).sum()
+    loss.backward()
+    assert opac.grad.shape == opac.shape and scales6.grad.shape == scales6.shape
+    assert (scales6.grad[:, 3:] == 0).all()
+    for name, value in (("means3D", means.grad), ("means2D", means2D.grad), ("opacities", opac.grad), ("shs", shs.grad),
+                        ("scales", scales6.grad[:, :3]), ("rotations", rots.grad)):
+        assert_grad_close(value.cpu().numpy(), ref[name], name)
+    # a second frame on the same stream before the first one's backward pass must not disturb it
+    image1, _, _ = r(means3D=means, means2D=None, shs=shs, colors_precomp=None, opacities=opac,
+                     scales=scales6[:, :3], rotations=rots, cov3D_precomp=None)
+    other = scenes.tiny_scene(P=200, width=96, height=64, sh_degree=2, seed=18)
+    with torch.no_grad():
+        r(means3D=other.means3D.to(gpu_device), shs=other.shs.to(gpu_device), opacities=other.opacities.to(gpu_device),
+          scales=other.scales.to(gpu_device), rotations=other.rotations.to(gpu_device))
+    means.grad = None
+    (image1 * gi.to(gpu_device)).sum().backward()
+    ref_image_only, _ = oracle_backward(scene, gi)
+    assert_grad_close(means.grad.cpu().numpy(), ref_image_only["means3D"], "means3D after an interleaved frame")
+
+
+def test_no_grad_call_is_the_plain_forward(gpu_device):
+    scene = scenes.tiny_scene(P=100, width=64, height=48, sh_degree=1, seed=2)
+    means = scene.means3D.to(gpu_device).requires_grad_(True)
+    r = GaussianRasterizer(settings_for(scene, gpu_device))
+    with torch.no_grad():
+        image, _, _ = r(means3D=means, shs=scene.shs.to(gpu_device), opacities=scene.opacities.to(gpu_device),
+                        scales=scene.scales.to(gpu_device), rotations=scene.rotations.to(gpu_device))
+    assert not image.requires_grad
+
+
+def test_training_step_of_the_vanilla_model(gpu_device):
+    """The reference's training forward (origin_gs/gs_model.py:112-228): all Gaussians rendered, the screen-space
+    points kept for densification; one backward pass fills the parameters' gradients."""
+    scene = scenes.tiny_scene(P=600, width=96, height=64, sh_degree=3, seed=23)
+    model = models.GaussianModel.from_activated(scene.means3D, scene.scales, scene.rotations, scene.opacities,
+                                                scene.shs).to(gpu_device)
+    for p in model.parameters():
+        p.requires_grad_(True)
+    model.train()
+    image = model(scene.camera)
+    assert image.requires_grad
+    target = torch.rand_like(image)
+    loss = (image - target).abs().mean()
+    loss.backward()
+    assert model.viewspace_points.grad is not None
+    vis = model.visibility_filter
+    assert (model.viewspace_points.grad[vis, :2].norm(dim=-1) > 0).any()
+    assert (model.viewspace_points.grad[~vis] == 0).all()
+    for name, p in model.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all(), name
+    assert model._xyz.grad.abs().max() > 0 and model._features_rest.grad.abs().max() > 0

@@ -211,7 +211,7 @@ GS355_API int gs355_anchor_filter(const gs355_frame *frame, const gs355_gaussian
  * origin_gs/gs_model.py:129-139,225-236).  It runs over the workspace the forward pass of the same frame left
  * behind (records, sorted values, ranges: nothing else may have used that workspace in between) and the
  * forward outputs. */
-#define GS355_GRAD_FLOATS 12 /* scratch floats per Gaussian */
+#define GS355_KEY_GRAD_FLOATS 16 /* scratch floats per (tile, Gaussian) key */
 
 typedef struct gs355_backward_inputs {
     const float *image;     /* [3,H,W] forward output */
@@ -239,12 +239,13 @@ typedef struct gs355_gradients {
     float *cov3D_precomp;  /* [P,6] */
 } gs355_gradients;
 
-/* Bytes of scratch gs355_render_backward needs for P Gaussians (per-Gaussian accumulators). */
-GS355_API int gs355_backward_scratch_bytes(int32_t P, size_t *bytes);
+/* Bytes of scratch gs355_render_backward needs for P Gaussians and a key capacity of n_cap: one 64-byte
+ * gradient record per key, and the index of each Gaussian's first record. */
+GS355_API int gs355_backward_scratch_bytes(int32_t P, int64_t n_cap, size_t *bytes);
 
 /* frame, g, workspace, workspace_bytes, n_cap: exactly what the forward call (gs355_render, or gs355_run through
- * the blend stage) was given.  The sums over pixels use floating-point atomics: results vary in the last bits
- * from run to run. */
+ * the blend stage) was given.  Every sum is taken in a fixed order (no floating-point atomics in global memory
+ * except within a tile's batch in LDS), so only the last bits may vary from run to run. */
 GS355_API int gs355_render_backward(const gs355_frame *frame, const gs355_gaussians *g, const void *workspace,
                                     size_t workspace_bytes, int64_t n_cap, const gs355_backward_inputs *in,
                                     void *scratch, size_t scratch_bytes, const gs355_gradients *grads, void *stream);

@@ -21,7 +21,6 @@ MAX_FAST_TILES = 36000
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
            "gs355_visible_filter", "gs355_anchor_filter", "gs355_decode_scratch_bytes", "gs355_decode_count",
            "gs355_decode_emit", "gs355_backward_scratch_bytes", "gs355_render_backward")
-GRAD_FLOATS = 12
 
 
 class Frame(C.Structure):
@@ -179,7 +178,7 @@ def load() -> C.CDLL:
     lib.gs355_decode_emit.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_int64,
                                       C.POINTER(Decoded), C.c_void_p]
     lib.gs355_decode_emit.restype = C.c_int
-    lib.gs355_backward_scratch_bytes.argtypes = [C.c_int32, C.POINTER(C.c_size_t)]
+    lib.gs355_backward_scratch_bytes.argtypes = [C.c_int32, C.c_int64, C.POINTER(C.c_size_t)]
     lib.gs355_backward_scratch_bytes.restype = C.c_int
     lib.gs355_render_backward.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_void_p, C.c_size_t, C.c_int64,
                                           C.POINTER(BackwardInputs), C.c_void_p, C.c_size_t, C.POINTER(Gradients),

@@ -279,11 +279,31 @@ int gs355_visible_filter(const gs355_frame* frame, const gs355_gaussians* g, int
     return launch_preprocess(fa, *g, true, nullptr, nullptr, nullptr, nullptr, radii, static_cast<hipStream_t>(stream));
 }
 
-int gs355_backward_scratch_bytes(int32_t P, size_t* bytes)
+namespace {
+struct BackwardScratch {
+    size_t first_key, scan_tmp, key_grads, total;
+};
+BackwardScratch backward_scratch(int32_t P, int64_t n_cap)
+{
+    BackwardScratch b;
+    size_t off = 0;
+    b.first_key = off;
+    off = align_up(off + (size_t)P * sizeof(uint32_t) + 4);
+    b.scan_tmp = off;
+    off = align_up(off + scan_tmp_words((size_t)P) * sizeof(uint32_t));
+    b.key_grads = off;
+    off = align_up(off + (size_t)n_cap * GS355_KEY_GRAD_FLOATS * sizeof(float) + 4);
+    b.total = off;
+    return b;
+}
+}  // namespace
+
+int gs355_backward_scratch_bytes(int32_t P, int64_t n_cap, size_t* bytes)
 {
     if (!bytes) return set_error(GS355_EINVAL, "bytes is NULL");
     if (P < 0) return set_error(GS355_EINVAL, "P must be >= 0 (got %d)", P);
-    *bytes = align_up((size_t)P * GS355_GRAD_FLOATS * sizeof(float));
+    if (n_cap < 0 || n_cap > kMaxKeys) return set_error(GS355_EINVAL, "n_cap out of range (got %lld)", (long long)n_cap);
+    *bytes = backward_scratch(P, n_cap).total;
     return GS355_OK;
 }
 
@@ -312,17 +332,24 @@ int gs355_render_backward(const gs355_frame* frame, const gs355_gaussians* g, co
     if (workspace_bytes < L.total_bytes)
         return set_error(GS355_ENOSPC, "workspace has %zu bytes, %zu needed (P=%d, n_cap=%lld, %dx%d)", workspace_bytes,
                          L.total_bytes, g->P, (long long)n_cap, frame->image_width, frame->image_height);
-    const size_t need = align_up((size_t)g->P * GS355_GRAD_FLOATS * sizeof(float));
+    const BackwardScratch B = backward_scratch(g->P, n_cap);
     if (g->P > 0 && !scratch) return set_error(GS355_EINVAL, "scratch is NULL");
-    if ((reinterpret_cast<uintptr_t>(scratch) & 15u) != 0) return set_error(GS355_EINVAL, "scratch must be 16-byte aligned");
-    if (scratch_bytes < need)
-        return set_error(GS355_ENOSPC, "scratch has %zu bytes, %zu needed (P=%d)", scratch_bytes, need, g->P);
+    if ((reinterpret_cast<uintptr_t>(scratch) & (kAlign - 1)) != 0)
+        return set_error(GS355_EINVAL, "scratch must be 256-byte aligned");
+    if (scratch_bytes < B.total)
+        return set_error(GS355_ENOSPC, "scratch has %zu bytes, %zu needed (P=%d, n_cap=%lld)", scratch_bytes, B.total,
+                         g->P, (long long)n_cap);
     const char* ws = static_cast<const char*>(workspace);
+    char* sc = static_cast<char*>(scratch);
     return launch_render_backward(make_args(frame), *g, reinterpret_cast<const gs355_header*>(ws + L.header),
                                   reinterpret_cast<const uint32_t*>(ws + L.ranges),
                                   reinterpret_cast<const uint32_t*>(ws + L.values[L.sorted_buffer]),
-                                  reinterpret_cast<const float*>(ws + L.records), *in, static_cast<float*>(scratch),
-                                  *grads, static_cast<hipStream_t>(stream));
+                                  reinterpret_cast<const float*>(ws + L.records),
+                                  reinterpret_cast<const uint32_t*>(ws + L.tiles_touched),
+                                  reinterpret_cast<const uint64_t*>(ws + L.rects), *in,
+                                  reinterpret_cast<uint32_t*>(sc + B.first_key),
+                                  reinterpret_cast<uint32_t*>(sc + B.scan_tmp),
+                                  reinterpret_cast<float*>(sc + B.key_grads), *grads, static_cast<hipStream_t>(stream));
 }
 
 int gs355_anchor_filter(const gs355_frame* frame, const gs355_gaussians* anchors, int32_t scale_stride,

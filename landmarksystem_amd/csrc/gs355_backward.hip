@@ -8,9 +8,13 @@
 //                    lists and the same per-pair decisions.  With f_i = colour_i . dL/dpixel, w_i = alpha_i T_i,
 //                    prefix P_i = sum_{j<=i} w_j f_j and R = out_pixel . dL/dpixel - T_final dL/dalpha_out (all
 //                    known from the forward outputs), dL/dalpha_i = T_i f_i - (R - P_i) / (1 - alpha_i): no
-//                    division by a transmittance and no second, reversed walk.  Per-pair gradients are summed
-//                    over the 16 pixels of a block with lane shuffles inside the 16-lane row, added to the staged
-//                    Gaussian's accumulators in LDS, and flushed to global memory once per batch of 256.
+//                    division by a transmittance and no second, reversed walk.  Per-pair contributions are summed
+//                    over the 16 pixels of a block by lane exchanges inside the 16-lane row, added to the staged
+//                    Gaussian's accumulators in LDS (one LDS atomic per step: LDS float atomics are slow), and
+//                    written once per batch of 256 as one 64-byte record per (tile, Gaussian) key.  No global
+//                    atomics (they cost more than the rest of the kernel): the records of a Gaussian are
+//                    consecutive, in the order its tile rectangle is walked, and the next kernel sums them in
+//                    that order, so gradients are identical from run to run.
 //   preprocess_backward  per Gaussian: conic -> 2-D covariance -> Jacobian / 3-D covariance -> scale, rotation,
 //                    mean; pixel position -> mean; colour -> SH coefficients and view direction -> mean.
 // min(0.99, opacity * G) passes the gradient unchanged, and the `means2D` gradient is in normalised device units
@@ -21,7 +25,16 @@ namespace gs355 {
 
 namespace {
 
-constexpr int kGradFloats = GS355_GRAD_FLOATS;  // dpx, dpy, dconic xyz, dopacity, drgb, ddepth, 2 unused
+constexpr int kGradFloats = 12;  // accumulators per staged Gaussian in LDS: 10 used
+constexpr int kKeyFloats = GS355_KEY_GRAD_FLOATS;  // per-key record: dpx, dpy, dconic xyz, dopacity, drgb, ddepth, 6 unused
+
+// Record slot of the key (tile, Gaussian): the Gaussian's keys in the order its tile rectangle is walked
+// (row by row), after those of all Gaussians before it.
+__device__ __forceinline__ uint32_t key_slot(uint32_t first, uint64_t rect, int tile_x, int tile_y)
+{
+    const int x0 = (int)(rect & 0xffffu), y0 = (int)((rect >> 16) & 0xffffu), x1 = (int)((rect >> 32) & 0xffffu);
+    return first + (uint32_t)((tile_y - y0) * (x1 - x0) + (tile_x - x0));
+}
 
 __device__ __forceinline__ float splat_exponent(float dx, float dy, float qx, float qy, float qz)
 {
@@ -38,14 +51,13 @@ __device__ __forceinline__ float dpp(float v)
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
 }
 
-// Sum over the 16 lanes of a row (every lane gets the total).
-__device__ __forceinline__ float row_sum(float v)
+// Two values reduced over a lane pair in one exchange: the lane with `upper` clear keeps a, the other keeps b,
+// each adds its partner's copy of the value it keeps.
+template <int kCtrl>
+__device__ __forceinline__ float keep_one_of_two(float a, float b, bool upper)
 {
-    v += dpp<0xB1>(v);   // quad_perm [1,0,3,2]
-    v += dpp<0x4E>(v);   // quad_perm [2,3,0,1]
-    v += dpp<0x141>(v);  // row_half_mirror
-    v += dpp<0x140>(v);  // row_mirror
-    return v;
+    const float send = upper ? a : b, keep = upper ? b : a;
+    return keep + dpp<kCtrl>(send);
 }
 
 struct PixelGrad {
@@ -53,11 +65,13 @@ struct PixelGrad {
     float R;               // out . g - T_final * dL/dalpha_out
 };
 
-// One 16-lane row evaluates staged Gaussian `a, b, c` on its 16 pixels and returns the row's summed gradient
-// contributions in v[0..9] (every lane holds the sums).  T carries the forward blend's state (sign = finished).
+// One 16-lane row evaluates staged Gaussian `a, b, c` on its 16 pixels.  Returns false if no lane of the wavefront
+// blended its pair; otherwise lane s < 10 of each row returns in `sum` the row's total of accumulator s:
+// the moments of dL/dpower over the pixel offsets (dpow dx, dpow dy, dpow dx^2, dpow dx dy, dpow dy^2),
+// dL/dopacity, dL/d(r, g, b, depth).  T carries the forward blend's state (sign = finished).
 __device__ __forceinline__ bool backward_one(float& T, float& prefix, const PixelGrad& pg, float pxf, float pyf,
-                                             const float4 a, const float4 b, const float4 c, bool enabled,
-                                             float v[10])
+                                             const float4 a, const float4 b, const float4 c, bool enabled, int sub,
+                                             float& sum)
 {
     const float dx = a.x - pxf, dy = a.y - pyf;
     const float power = splat_exponent(dx, dy, a.z, a.w, b.x);
@@ -73,21 +87,31 @@ __device__ __forceinline__ bool backward_one(float& T, float& prefix, const Pixe
         w = alpha * T;
         const float fg = b.z * pg.g0 + b.w * pg.g1 + c.x * pg.g2 + c.y * pg.g3;
         prefix += w * fg;
-        const float dalpha = T * fg - (pg.R - prefix) * __frcp_rn(1.0f - alpha);
+        const float dalpha = T * fg - (pg.R - prefix) * __builtin_amdgcn_rcpf(1.0f - alpha);
         dop = G * dalpha;
         dpow = b.y * dop;
         T = test_T;
     }
-    v[0] = row_sum(dpow * (-a.z * dx - a.w * dy));
-    v[1] = row_sum(dpow * (-b.x * dy - a.w * dx));
-    v[2] = row_sum(dpow * (-0.5f * dx * dx));
-    v[3] = row_sum(dpow * (-dx * dy));
-    v[4] = row_sum(dpow * (-0.5f * dy * dy));
-    v[5] = row_sum(dop);
-    v[6] = row_sum(w * pg.g0);
-    v[7] = row_sum(w * pg.g1);
-    v[8] = row_sum(w * pg.g2);
-    v[9] = row_sum(w * pg.g3);
+    const float mx = dpow * dx, my = dpow * dy;
+    // ten sums over the row's 16 lanes, transposed as they are reduced: after the exchanges inside lane pairs and
+    // quads a lane holds one of four (then two) values, the quads' partial sums are rotated together, and lane s
+    // ends with the total of value s
+    const bool b0 = (sub & 1) != 0, b1 = (sub & 2) != 0;
+    const float u0 = keep_one_of_two<0xB1>(mx, my, b0);            // quad_perm [1,0,3,2]
+    const float u1 = keep_one_of_two<0xB1>(mx * dx, mx * dy, b0);
+    const float u2 = keep_one_of_two<0xB1>(my * dy, dop, b0);
+    const float u3 = keep_one_of_two<0xB1>(w * pg.g0, w * pg.g1, b0);
+    const float u4 = keep_one_of_two<0xB1>(w * pg.g2, w * pg.g3, b0);
+    float t0 = keep_one_of_two<0x4E>(u0, u1, b1);                  // quad_perm [2,3,0,1]: value 2 b1 + b0
+    float t1 = keep_one_of_two<0x4E>(u2, u3, b1);                  // value 4 + 2 b1 + b0
+    float t2 = u4 + dpp<0x4E>(u4);                                 // value 8 + b0
+    t0 += dpp<0x124>(t0);                                          // row_ror:4
+    t1 += dpp<0x124>(t1);
+    t2 += dpp<0x124>(t2);
+    t0 += dpp<0x128>(t0);                                          // row_ror:8
+    t1 += dpp<0x128>(t1);
+    t2 += dpp<0x128>(t2);
+    sum = sub < 4 ? t0 : sub < 8 ? t1 : t2;
     return true;
 }
 
@@ -95,7 +119,8 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
     FrameArgs f, const gs355_header* __restrict__ header, const uint32_t* __restrict__ ranges,
     const uint32_t* __restrict__ values, const float* __restrict__ records, const float* __restrict__ image,
     const float* __restrict__ out_depth, const float* __restrict__ out_alpha, const float* __restrict__ g_image,
-    const float* __restrict__ g_depth, const float* __restrict__ g_alpha, float* __restrict__ grads)
+    const float* __restrict__ g_depth, const float* __restrict__ g_alpha, const uint64_t* __restrict__ rects,
+    const uint32_t* __restrict__ first_key, float* __restrict__ key_grads)
 {
     __shared__ float4 s_a[256];  // px, py, conic_x, conic_y
     __shared__ float4 s_b[256];  // conic_z, opacity, r, g
@@ -135,17 +160,19 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
     const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
     float T = inside ? 1.0f : -1.0f, prefix = 0.0f;
 
-    for (uint32_t base = lo; base < hi; base += 256) {
+    uint32_t base = lo;
+    for (; base < hi; base += 256) {
         const bool wave_done = __ballot(T > 0.0f) == 0ull;
         if (lane == 0) s_wave_done[wave] = wave_done ? 1u : 0u;
         const uint32_t j = base + tid;
-        uint32_t g = 0;
+        uint32_t slot = 0;
         if (j < hi) {
-            g = values[j];
+            const uint32_t g = values[j];
             const float4* __restrict__ rec = reinterpret_cast<const float4*>(records + (size_t)g * kRecordFloats);
             s_a[tid] = rec[0];
             s_b[tid] = rec[1];
             s_c[tid] = rec[2];
+            slot = key_slot(first_key[g], rects[g], tile_x, tile_y);
         }
         {
             float4* __restrict__ row = reinterpret_cast<float4*>(s_grad + tid * kGradFloats);
@@ -185,28 +212,33 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
             for (uint32_t i = 0; i < longest; ++i) {
                 const uint32_t kk = k_next;
                 k_next = mine[i + 1];
-                float v[10];
-                if (backward_one(T, prefix, pg, pxf, pyf, s_a[kk], s_b[kk], s_c[kk], i < my_len, v)) {
-                    // lane `sub` of each row adds slot `sub` of its Gaussian
-                    float mine_v = v[0];
-#pragma unroll
-                    for (int s = 1; s < 10; ++s) mine_v = sub == s ? v[s] : mine_v;
-                    if (sub < 10 && i < my_len && mine_v != 0.0f) atomicAdd(&s_grad[kk * kGradFloats + sub], mine_v);
+                float sum;
+                if (backward_one(T, prefix, pg, pxf, pyf, s_a[kk], s_b[kk], s_c[kk], i < my_len, sub, sum)) {
+                    // lane s of each row adds accumulator s of the row's Gaussian
+                    if (sub < 10 && i < my_len && sum != 0.0f) atomicAdd(&s_grad[kk * kGradFloats + sub], sum);
                 }
                 if (__ballot(T > 0.0f) == 0ull) break;
             }
         }
         __syncthreads();
-        // ---- flush this batch's accumulators ----
+        // ---- this batch's records: the moments turned into gradients of position and conic ----
         if (j < hi) {
-            const float* __restrict__ row = s_grad + tid * kGradFloats;
-            float* __restrict__ dst = grads + (size_t)g * kGradFloats;
-#pragma unroll
-            for (int s = 0; s < 10; ++s) {
-                const float val = row[s];
-                if (val != 0.0f) unsafeAtomicAdd(dst + s, val);
-            }
+            const float* __restrict__ m = s_grad + tid * kGradFloats;
+            const float4 a = s_a[tid];
+            const float cz = s_b[tid].x;
+            float4* __restrict__ dst = reinterpret_cast<float4*>(key_grads + (size_t)slot * kKeyFloats);
+            dst[0] = make_float4(-(a.z * m[0] + a.w * m[1]), -(cz * m[1] + a.w * m[0]), -0.5f * m[2], -m[3]);
+            dst[1] = make_float4(-0.5f * m[4], m[5], m[6], m[7]);
+            dst[2] = make_float4(m[8], m[9], 0.f, 0.f);
+            dst[3] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
+    }
+    // keys the tile never reached (every pixel finished before them) contribute nothing: every record is written
+    for (uint32_t j = base + tid; j < hi; j += 256) {
+        const uint32_t g = values[j];
+        float4* __restrict__ dst =
+            reinterpret_cast<float4*>(key_grads + (size_t)key_slot(first_key[g], rects[g], tile_x, tile_y) * kKeyFloats);
+        dst[0] = dst[1] = dst[2] = dst[3] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
 
@@ -253,7 +285,10 @@ __device__ __forceinline__ void sh_basis_grad(int deg, float x, float y, float z
 __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, gs355_gaussians g,
                                                                   const int32_t* __restrict__ radii,
                                                                   const float* __restrict__ records,
-                                                                  const float* __restrict__ grads, gs355_gradients out)
+                                                                  const uint32_t* __restrict__ tiles_touched,
+                                                                  const uint32_t* __restrict__ first_key,
+                                                                  const float* __restrict__ key_grads,
+                                                                  gs355_gradients out)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= g.P) return;
@@ -268,8 +303,18 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
     if (alive) {
         const float* __restrict__ V = f.viewmatrix;
         const float* __restrict__ Pm = f.projmatrix;
-        const float4* __restrict__ A4 = reinterpret_cast<const float4*>(grads + si * kGradFloats);
-        const float4 A0 = A4[0], A1 = A4[1], A2 = A4[2];
+        // the Gaussian's keys are consecutive records; summed in order, so the result does not vary between runs
+        float4 A0 = make_float4(0.f, 0.f, 0.f, 0.f), A1 = A0, A2 = A0;
+        {
+            const float4* __restrict__ rec = reinterpret_cast<const float4*>(key_grads + (size_t)first_key[i] * kKeyFloats);
+            const uint32_t n = tiles_touched[i];
+            for (uint32_t k = 0; k < n; ++k) {
+                const float4 r0 = rec[4 * (size_t)k], r1 = rec[4 * (size_t)k + 1], r2 = rec[4 * (size_t)k + 2];
+                A0.x += r0.x; A0.y += r0.y; A0.z += r0.z; A0.w += r0.w;
+                A1.x += r1.x; A1.y += r1.y; A1.z += r1.z; A1.w += r1.w;
+                A2.x += r2.x; A2.y += r2.y;
+            }
+        }
         const float g_px = A0.x, g_py = A0.y, gA = A0.z, gB = A0.w, gC = A1.x;
         dop = A1.y;
         dcol[0] = A1.z; dcol[1] = A1.w; dcol[2] = A2.x;
@@ -461,17 +506,20 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
 
 int launch_render_backward(const FrameArgs& f, const gs355_gaussians& g, const gs355_header* header,
                            const uint32_t* ranges, const uint32_t* values, const float* records,
-                           const gs355_backward_inputs& in, float* grads, const gs355_gradients& out, hipStream_t s)
+                           const uint32_t* tiles_touched, const uint64_t* rects, const gs355_backward_inputs& in,
+                           uint32_t* first_key, uint32_t* scan_tmp, float* key_grads, const gs355_gradients& out,
+                           hipStream_t s)
 {
     if (g.P == 0) return GS355_OK;
-    int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(grads), (size_t)g.P * kGradFloats, 0u, s);
+    int rc = launch_exclusive_scan(tiles_touched, first_key, (size_t)g.P, scan_tmp, s);
     if (rc) return rc;
     const int tiles = f.grid_x * f.grid_y;
     hipLaunchKernelGGL(blend_backward_kernel, dim3(tiles), dim3(256), 0, s, f, header, ranges, values, records,
-                       in.image, in.depth, in.alpha, in.dL_dimage, in.dL_ddepth, in.dL_dalpha, grads);
+                       in.image, in.depth, in.alpha, in.dL_dimage, in.dL_ddepth, in.dL_dalpha, rects, first_key,
+                       key_grads);
     GS355_CHECK_LAUNCH("blend backward");
     hipLaunchKernelGGL(preprocess_backward_kernel, dim3((g.P + 255) / 256), dim3(256), 0, s, f, g, in.radii, records,
-                       grads, out);
+                       tiles_touched, first_key, key_grads, out);
     GS355_CHECK_LAUNCH("preprocess backward");
     return GS355_OK;
 }

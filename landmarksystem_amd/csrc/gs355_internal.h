@@ -91,7 +91,9 @@ int launch_blend(const FrameArgs& f, const gs355_header* header, const uint32_t*
 
 int launch_render_backward(const FrameArgs& f, const gs355_gaussians& g, const gs355_header* header,
                            const uint32_t* ranges, const uint32_t* values, const float* records,
-                           const gs355_backward_inputs& in, float* grads, const gs355_gradients& out, hipStream_t s);
+                           const uint32_t* tiles_touched, const uint64_t* rects, const gs355_backward_inputs& in,
+                           uint32_t* first_key, uint32_t* scan_tmp, float* key_grads, const gs355_gradients& out,
+                           hipStream_t s);
 
 // Orders one wavefront's LDS writes before its later LDS reads (and the reverse).  The hardware executes a
 // wavefront's LDS instructions in order; the fences (wavefront scope: no instructions) and the scheduling

@@ -296,7 +296,9 @@ def render_backward(inputs: FrameInputs, out: FrameOutputs, workspace: torch.Ten
     b = _lib.BackwardInputs(_ptr(out.image), _ptr(out.depth), _ptr(out.alpha), _ptr(out.radii), _ptr(gi), _ptr(gd),
                             _ptr(ga))
     g = _lib.Gradients(*[_ptr(grads.get(n)) for n in GRAD_NAMES])
-    scratch = torch.empty(P * _lib.GRAD_FLOATS + 64, dtype=torch.float32, device=dev)
+    need = C.c_size_t(0)
+    _lib.check(_lib.load().gs355_backward_scratch_bytes(P, int(out.key_capacity), C.byref(need)))
+    scratch = torch.empty(need.value // 4, dtype=torch.float32, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
     _lib.check(_lib.load().gs355_render_backward(C.byref(inputs.frame), C.byref(inputs.gaussians), workspace.data_ptr(),
                                                  workspace.numel(), int(out.key_capacity), C.byref(b),

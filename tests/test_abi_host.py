@@ -143,10 +143,11 @@ def test_run_validates_before_any_hip_call():
 def test_render_backward_validates_before_any_hip_call():
     lib = _lib.load()
     size = C.c_size_t(0)
-    assert lib.gs355_backward_scratch_bytes(1000, C.byref(size)) == 0 and size.value >= 1000 * _lib.GRAD_FLOATS * 4
-    assert size.value % 256 == 0
-    assert "P must be" in _err(_lib.GS355_EINVAL, lib.gs355_backward_scratch_bytes, -1, C.byref(size))
-    assert _err(_lib.GS355_EINVAL, lib.gs355_backward_scratch_bytes, 10, None)
+    assert lib.gs355_backward_scratch_bytes(1000, 5000, C.byref(size)) == 0
+    assert size.value >= 5000 * 64 + 1000 * 4 and size.value % 256 == 0
+    assert "P must be" in _err(_lib.GS355_EINVAL, lib.gs355_backward_scratch_bytes, -1, 10, C.byref(size))
+    assert "n_cap" in _err(_lib.GS355_EINVAL, lib.gs355_backward_scratch_bytes, 10, -1, C.byref(size))
+    assert _err(_lib.GS355_EINVAL, lib.gs355_backward_scratch_bytes, 10, 10, None)
 
     def bwd(f, g, ws, nbytes, cap, b, scratch, sbytes, grads):
         return lib.gs355_render_backward(C.byref(f) if f else None, C.byref(g) if g else None, ws, nbytes, cap,
@@ -181,7 +182,7 @@ def test_render_backward_validates_before_any_hip_call():
     assert "aligned" in _err(_lib.GS355_EINVAL, bwd, *with_(ws=0x1001))
     assert "needed" in _err(_lib.GS355_ENOSPC, bwd, *with_(nbytes=1024))
     assert "scratch is NULL" in _err(_lib.GS355_EINVAL, bwd, *with_(scratch=None))
-    assert "16-byte" in _err(_lib.GS355_EINVAL, bwd, *with_(scratch=0x1004))
+    assert "256-byte" in _err(_lib.GS355_EINVAL, bwd, *with_(scratch=0x1004))
     assert "scratch has" in _err(_lib.GS355_ENOSPC, bwd, *with_(sbytes=16))
     assert "32-bit" in _err(_lib.GS355_EOVERFLOW, bwd, *with_(cap=1 << 33))
 

@@ -282,6 +282,11 @@ __device__ __forceinline__ void sh_basis_grad(int deg, float x, float y, float z
     b[15] = kShC3[6] * x * (xx - 3.0f * yy); bx[15] = kShC3[6] * (3.0f * xx - 3.0f * yy); by[15] = kShC3[6] * -6.0f * xy;
 }
 
+constexpr int kShStride = 52;  // floats per Gaussian in the SH staging area (16-B reads of 64 lanes on distinct banks)
+
+// kMode 0: SH blocks (if any) are read and written by their own lanes.  1 and 2: 16-coefficient blocks, 16-byte
+// aligned, staged through LDS; 2 also fetches the coefficients (needed for degree > 0 only).
+template <int kMode>
 __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, gs355_gaussians g,
                                                                   const int32_t* __restrict__ radii,
                                                                   const float* __restrict__ records,
@@ -290,29 +295,54 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
                                                                   const float* __restrict__ key_grads,
                                                                   gs355_gradients out)
 {
+    // Full 16-coefficient SH blocks travel through LDS: each wavefront moves the 12 KB of its 64 Gaussians'
+    // coefficients (in) and coefficient gradients (out) with coalesced 16-B accesses; a lane works on its own row.
+    __shared__ float4 s_sh[kMode == 0 ? 1 : 4 * 64 * kShStride / 4];
+
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= g.P) return;
-    const size_t si = (size_t)i;
+    const bool valid = i < g.P;
+    const size_t si = (size_t)(valid ? i : g.P - 1);
     const int M = f.sh_coeffs;
-    const bool alive = radii[i] > 0;
+    const bool alive = valid && radii[si] > 0;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const size_t wave_first = (size_t)blockIdx.x * blockDim.x + (size_t)wave * 64;
+    const int count = (int)min((size_t)64, (size_t)g.P > wave_first ? (size_t)g.P - wave_first : (size_t)0);
+    constexpr bool staged = kMode != 0, fetch_sh = kMode == 2;
+    float4* __restrict__ mine = s_sh + (staged ? wave * 64 * (kShStride / 4) : 0);
+    float* __restrict__ my_row = reinterpret_cast<float*>(mine) + (staged ? lane * kShStride : 0);
+
     float dmean[3] = {0.f, 0.f, 0.f}, d2[3] = {0.f, 0.f, 0.f}, dscale[3] = {0.f, 0.f, 0.f};
     float drot[4] = {0.f, 0.f, 0.f, 0.f}, dcov[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, dcol[3] = {0.f, 0.f, 0.f};
     float dop = 0.f;
     float b[16], gcol[3] = {0.f, 0.f, 0.f};
+    float nx = 0.f, ny = 0.f, nz = 0.f, inv_len = 0.f;
+    float bx[16], by[16], bz[16];
     int K = 0;
     if (alive) {
         const float* __restrict__ V = f.viewmatrix;
         const float* __restrict__ Pm = f.projmatrix;
-        // the Gaussian's keys are consecutive records; summed in order, so the result does not vary between runs
+        // the Gaussian's keys are consecutive records; summed in order, so the result does not vary between runs.
+        // Four records are requested at a time (indices past the last one re-read it and are not added).
         float4 A0 = make_float4(0.f, 0.f, 0.f, 0.f), A1 = A0, A2 = A0;
         {
-            const float4* __restrict__ rec = reinterpret_cast<const float4*>(key_grads + (size_t)first_key[i] * kKeyFloats);
-            const uint32_t n = tiles_touched[i];
-            for (uint32_t k = 0; k < n; ++k) {
-                const float4 r0 = rec[4 * (size_t)k], r1 = rec[4 * (size_t)k + 1], r2 = rec[4 * (size_t)k + 2];
-                A0.x += r0.x; A0.y += r0.y; A0.z += r0.z; A0.w += r0.w;
-                A1.x += r1.x; A1.y += r1.y; A1.z += r1.z; A1.w += r1.w;
-                A2.x += r2.x; A2.y += r2.y;
+            const float4* __restrict__ rec = reinterpret_cast<const float4*>(key_grads + (size_t)first_key[si] * kKeyFloats);
+            const uint32_t n = tiles_touched[si];
+            for (uint32_t k0 = 0; k0 < n; k0 += 4) {
+                float4 r[4][3];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const size_t k = min(k0 + (uint32_t)u, n - 1);
+#pragma unroll
+                    for (int q = 0; q < 3; ++q) r[u][q] = rec[4 * k + q];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (k0 + (uint32_t)u < n) {
+                        A0.x += r[u][0].x; A0.y += r[u][0].y; A0.z += r[u][0].z; A0.w += r[u][0].w;
+                        A1.x += r[u][1].x; A1.y += r[u][1].y; A1.z += r[u][1].z; A1.w += r[u][1].w;
+                        A2.x += r[u][2].x; A2.y += r[u][2].y;
+                    }
+                }
             }
         }
         const float g_px = A0.x, g_py = A0.y, gA = A0.z, gB = A0.w, gC = A1.x;
@@ -439,12 +469,13 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
                              qy * dR[1][2] + qx * dR[2][0] + qy * dR[2][1]);
         }
 
-        // ---- colour: SH coefficients and view direction ----
+        // ---- colour: view direction, SH basis and its gradient ----
         if (g.shs) {
             const float dirx = x - f.campos[0], diry = y - f.campos[1], dirz = z - f.campos[2];
-            const float inv_len = 1.0f / sqrtf(dirx * dirx + diry * diry + dirz * dirz);
-            const float nx = dirx * inv_len, ny = diry * inv_len, nz = dirz * inv_len;
-            float bx[16], by[16], bz[16];
+            inv_len = 1.0f / sqrtf(dirx * dirx + diry * diry + dirz * dirz);
+            nx = dirx * inv_len;
+            ny = diry * inv_len;
+            nz = dirz * inv_len;
             sh_basis_grad(f.sh_degree, nx, ny, nz, b, bx, by, bz);
             K = (f.sh_degree + 1) * (f.sh_degree + 1);
             // the forward pass clamped the colour at zero: a zero in the record means no gradient
@@ -452,25 +483,78 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
             gcol[0] = rec[6] > 0.0f ? dcol[0] : 0.0f;
             gcol[1] = rec[7] > 0.0f ? dcol[1] : 0.0f;
             gcol[2] = rec[8] > 0.0f ? dcol[2] : 0.0f;
-            if (f.sh_degree > 0) {
-                const float* __restrict__ sh = g.shs + si * M * 3;
-                float dn[3] = {0.f, 0.f, 0.f};
+        }
+    }
+
+    // ---- SH coefficients: their part of the mean's gradient (through the view direction), and their own ----
+    if (g.shs) {
+        if (fetch_sh) {
+            // coefficients of the wavefront's Gaussians: all loads in flight together, then into the rows (slots
+            // past the last Gaussian re-read it)
+            float4 sh_in[12];
 #pragma unroll
-                for (int k = 1; k < 16; ++k) {
-                    if (k < K) {
-                        const float t = gcol[0] * sh[3 * k] + gcol[1] * sh[3 * k + 1] + gcol[2] * sh[3 * k + 2];
-                        dn[0] += t * bx[k];
-                        dn[1] += t * by[k];
-                        dn[2] += t * bz[k];
+            for (int it = 0; it < 12; ++it) {
+                const int q4 = it * 64 + lane;
+                const size_t e = min(wave_first + (size_t)(q4 / 12), (size_t)g.P - 1);
+                sh_in[it] = reinterpret_cast<const float4*>(g.shs + e * 48)[q4 % 12];
+            }
+#pragma unroll
+            for (int it = 0; it < 12; ++it) {
+                const int q4 = it * 64 + lane;
+                mine[(q4 / 12) * (kShStride / 4) + q4 % 12] = sh_in[it];
+            }
+            wave_lds_sync();
+        }
+        if (alive && f.sh_degree > 0) {
+            const float* __restrict__ sh = staged ? my_row : g.shs + si * M * 3;
+            float dn[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+            for (int k = 1; k < 16; ++k) {
+                if (k < K) {
+                    const float t = gcol[0] * sh[3 * k] + gcol[1] * sh[3 * k + 1] + gcol[2] * sh[3 * k + 2];
+                    dn[0] += t * bx[k];
+                    dn[1] += t * by[k];
+                    dn[2] += t * bz[k];
+                }
+            }
+            const float dot = nx * dn[0] + ny * dn[1] + nz * dn[2];
+            dmean[0] += (dn[0] - nx * dot) * inv_len;
+            dmean[1] += (dn[1] - ny * dot) * inv_len;
+            dmean[2] += (dn[2] - nz * dot) * inv_len;
+        }
+        if (out.shs) {
+            if (staged) {
+                wave_lds_sync();  // rows were read above
+#pragma unroll
+                for (int k = 0; k < 16; ++k) {
+                    const float bk = (alive && k < K) ? b[k] : 0.0f;
+                    my_row[3 * k] = bk * gcol[0];
+                    my_row[3 * k + 1] = bk * gcol[1];
+                    my_row[3 * k + 2] = bk * gcol[2];
+                }
+                wave_lds_sync();
+#pragma unroll
+                for (int it = 0; it < 12; ++it) {
+                    const int q4 = it * 64 + lane;
+                    const int e = q4 / 12, m = q4 % 12;
+                    if (e < count) reinterpret_cast<float4*>(out.shs + (wave_first + e) * 48)[m] = mine[e * (kShStride / 4) + m];
+                }
+            } else if (valid) {
+                float* __restrict__ o = out.shs + si * M * 3;
+#pragma unroll
+                for (int k = 0; k < 16; ++k) {
+                    if (k < M) {
+                        const float bk = (alive && k < K) ? b[k] : 0.0f;
+                        o[3 * k] = bk * gcol[0];
+                        o[3 * k + 1] = bk * gcol[1];
+                        o[3 * k + 2] = bk * gcol[2];
                     }
                 }
-                const float dot = nx * dn[0] + ny * dn[1] + nz * dn[2];
-                dmean[0] += (dn[0] - nx * dot) * inv_len;
-                dmean[1] += (dn[1] - ny * dot) * inv_len;
-                dmean[2] += (dn[2] - nz * dot) * inv_len;
+                for (int k = 48; k < 3 * M; ++k) o[k] = 0.0f;  // coefficient rows beyond degree 3
             }
         }
     }
+    if (!valid) return;
 
     if (out.means3D)
 #pragma unroll
@@ -491,15 +575,6 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
     if (out.cov3D_precomp)
 #pragma unroll
         for (int k = 0; k < 6; ++k) out.cov3D_precomp[6 * si + k] = dcov[k];
-    if (out.shs) {
-        float* __restrict__ o = out.shs + si * M * 3;
-        for (int k = 0; k < M; ++k) {
-            const float bk = (alive && k < K) ? b[k < 16 ? k : 0] : 0.0f;
-            o[3 * k] = bk * gcol[0];
-            o[3 * k + 1] = bk * gcol[1];
-            o[3 * k + 2] = bk * gcol[2];
-        }
-    }
 }
 
 }  // namespace
@@ -518,8 +593,18 @@ int launch_render_backward(const FrameArgs& f, const gs355_gaussians& g, const g
                        in.image, in.depth, in.alpha, in.dL_dimage, in.dL_ddepth, in.dL_dalpha, rects, first_key,
                        key_grads);
     GS355_CHECK_LAUNCH("blend backward");
-    hipLaunchKernelGGL(preprocess_backward_kernel, dim3((g.P + 255) / 256), dim3(256), 0, s, f, g, in.radii, records,
-                       tiles_touched, first_key, key_grads, out);
+    const bool staged = g.shs != nullptr && f.sh_coeffs == 16 && (reinterpret_cast<uintptr_t>(g.shs) & 15u) == 0 &&
+                        (out.shs == nullptr || (reinterpret_cast<uintptr_t>(out.shs) & 15u) == 0);
+    const dim3 grid((g.P + 255) / 256), block(256);
+    if (!staged)
+        hipLaunchKernelGGL(preprocess_backward_kernel<0>, grid, block, 0, s, f, g, in.radii, records, tiles_touched,
+                           first_key, key_grads, out);
+    else if (f.sh_degree == 0)
+        hipLaunchKernelGGL(preprocess_backward_kernel<1>, grid, block, 0, s, f, g, in.radii, records, tiles_touched,
+                           first_key, key_grads, out);
+    else
+        hipLaunchKernelGGL(preprocess_backward_kernel<2>, grid, block, 0, s, f, g, in.radii, records, tiles_touched,
+                           first_key, key_grads, out);
     GS355_CHECK_LAUNCH("preprocess backward");
     return GS355_OK;
 }

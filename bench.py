@@ -55,6 +55,7 @@ def parse_args():
     ap.add_argument("--no-model-level", action="store_true",
                     help="skip the model-level variants (their launches of the same kernels on other inputs would "
                          "mix into the per-kernel averages of a profiler run)")
+    ap.add_argument("--no-backward", action="store_true", help="skip the backward-pass timing")
     ap.add_argument("--two-in-flight", action="store_true",
                     help="also time the frames with two in flight on alternating streams (reported beside `value`)")
     return ap.parse_args()
@@ -370,6 +371,37 @@ def main():
     stages["rates"] = {"gaussians_per_s_preprocess": round(P / stage_ms["preprocess"] * 1e3),
                        "sorted_keys_per_s": round(N / sort_ms * 1e3) if N else 0,
                        "blend_frames_per_s": round(1e3 / stage_ms["blend"], 1)}
+
+    # backward pass of the same frame (the training loop's loss.backward() on an image loss): all gradients of a
+    # forward render, reported beside the forward stages, never part of `value`
+    if not args.no_backward:
+        ws_b = pipeline.Workspace(dev)
+        ws_b.key_capacity = n_cap
+        out_b = pipeline.render(inp, ws=ws_b)
+        g_image = torch.randn(3, inp.height, inp.width, device=dev)
+        t_bwd = {}
+        for label, want in (("all_gradients", pipeline.GRAD_NAMES),
+                            ("without_sh_gradient", tuple(n for n in pipeline.GRAD_NAMES if n != "shs"))):
+            for _ in range(3):
+                pipeline.render_backward(inp, out_b, ws_b.buffer, g_image, want=want)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(args.stage_steps):
+                pipeline.render_backward(inp, out_b, ws_b.buffer, g_image, want=want)
+            e1.record()
+            torch.cuda.synchronize()
+            t_bwd[label] = e0.elapsed_time(e1) / args.stage_steps
+        # algorithmic bytes: a 64-B gradient record per key written and 48 B of it read back; per key the sorted
+        # value, the 48-B record of its Gaussian, rectangle and first-record index; per visible Gaussian its inputs
+        # and record; per Gaussian radius, key count, first-record index and every gradient written
+        bwd_bytes = N * (64 + 48 + 4 + 48 + 12) + V * (12 + 12 + 16 + 4 * 3 * scene.shs.shape[1] + 48) + \
+            P * (12 + 12 + 12 + 4 + 12 + 16 + 4 * 3 * scene.shs.shape[1])
+        stages["backward"] = {"ms": round(t_bwd["all_gradients"], 4),
+                              "ms_without_sh_gradient": round(t_bwd["without_sh_gradient"], 4),
+                              "bytes": bwd_bytes, "GBps": round(bwd_bytes / t_bwd["all_gradients"] / 1e6, 1),
+                              "forward_plus_backward_frames_per_s":
+                                  round(1e3 / (ms_per_step + t_bwd["all_gradients"]), 1)}
+        del ws_b, out_b
 
     # counter-measured traffic only applies to the workload it was measured on
     traffic = MEASURED_TRAFFIC_BYTES if default_workload else {}

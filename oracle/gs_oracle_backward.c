@@ -71,6 +71,12 @@ typedef struct {
     float dx, dy, G, alpha, T;
 } orc_hit;
 
+#define ORC_ADD(target, value)                 \
+    do {                                       \
+        double v__ = (value);                  \
+        _Pragma("omp atomic") (target) += v__; \
+    } while (0)
+
 /* Backward of orc_blend.  g_rgb [3,H,W]; g_depth, g_alpha [H,W] or NULL.
  * acc: double[P][ORC_GRAD], zero-filled by the caller; pixel-space gradients
  * of (px, py), of the conic as it enters the exponent
@@ -81,8 +87,13 @@ void orc_blend_backward(const orc_frame *f, const uint32_t *ranges, const uint32
 {
     int W = f->image_width, H = f->image_height;
     int grid_x = (W + ORC_TILE - 1) / ORC_TILE, grid_y = (H + ORC_TILE - 1) / ORC_TILE;
+    /* tiles in parallel; a Gaussian's accumulators are shared between the tiles it touches, hence the atomic adds
+     * (doubles: the order of the additions changes the sums by ~1e-16 relative, far below any comparison) */
+#pragma omp parallel
+    {
     size_t cap = 1024;
     orc_hit *hits = (orc_hit *)malloc(cap * sizeof *hits);
+#pragma omp for schedule(dynamic, 4)
     for (int t = 0; t < grid_x * grid_y; ++t) {
         int tx0 = (t % grid_x) * ORC_TILE, ty0 = (t / grid_x) * ORC_TILE;
         uint32_t lo = ranges[2 * t], hi = ranges[2 * t + 1];
@@ -132,7 +143,7 @@ void orc_blend_backward(const orc_frame *f, const uint32_t *ranges, const uint32
                         behind[c] = last_alpha * last_col[c] + (1.0 - last_alpha) * behind[c];
                         last_col[c] = col[c];
                         dL_dalpha += (col[c] - behind[c]) * gc[c];
-                        A[6 + c] += a * Tk * gc[c];
+                        ORC_ADD(A[6 + c], a * Tk * gc[c]);
                     }
                     dL_dalpha *= Tk;
                     last_alpha = a;
@@ -140,16 +151,17 @@ void orc_blend_backward(const orc_frame *f, const uint32_t *ranges, const uint32
                     double G = h->G, dx = h->dx, dy = h->dy;
                     double dL_dG = co[3] * dL_dalpha; /* through the min(0.99, .) unchanged */
                     double dL_dpower = G * dL_dG;
-                    A[0] += dL_dpower * (-(double)co[0] * dx - (double)co[1] * dy);
-                    A[1] += dL_dpower * (-(double)co[2] * dy - (double)co[1] * dx);
-                    A[2] += dL_dpower * (-0.5 * dx * dx);
-                    A[3] += dL_dpower * (-dx * dy);
-                    A[4] += dL_dpower * (-0.5 * dy * dy);
-                    A[5] += G * dL_dalpha;
+                    ORC_ADD(A[0], dL_dpower * (-(double)co[0] * dx - (double)co[1] * dy));
+                    ORC_ADD(A[1], dL_dpower * (-(double)co[2] * dy - (double)co[1] * dx));
+                    ORC_ADD(A[2], dL_dpower * (-0.5 * dx * dx));
+                    ORC_ADD(A[3], dL_dpower * (-dx * dy));
+                    ORC_ADD(A[4], dL_dpower * (-0.5 * dy * dy));
+                    ORC_ADD(A[5], G * dL_dalpha);
                 }
             }
     }
     free(hits);
+    }
 }
 
 static const double SH_C0 = 0.28209479177387814;
@@ -206,6 +218,7 @@ void orc_preprocess_backward(const orc_frame *f, const orc_gaussians *g, const i
     double W_img = f->image_width, H_img = f->image_height;
     double fx = W_img / (2.0 * (double)f->tanfovx), fy = H_img / (2.0 * (double)f->tanfovy);
     double limx = 1.3 * (double)f->tanfovx, limy = 1.3 * (double)f->tanfovy;
+#pragma omp parallel for schedule(static)
     for (int i = 0; i < g->P; ++i) {
         if (radii[i] <= 0) continue;
         const double *A = acc + (size_t)i * ORC_GRAD;

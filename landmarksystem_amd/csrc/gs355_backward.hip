@@ -413,9 +413,10 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
         const float cb = a0[0] * Sa1[0] + a0[1] * Sa1[1] + a0[2] * Sa1[2];
         const float cc = a1[0] * Sa1[0] + a1[1] * Sa1[1] + a1[2] * Sa1[2] + 0.3f;
         const float D = 1.0f / (ca * cc - cb * cb), D2 = D * D;
-        const float d_ca = gA * (-cc * cc * D2) + gB * (cb * cc * D2) + gC * (D - ca * cc * D2);
-        const float d_cb = gA * (2.f * cb * cc * D2) + gB * (-D - 2.f * cb * cb * D2) + gC * (2.f * ca * cb * D2);
-        const float d_cc = gA * (D - ca * cc * D2) + gB * (ca * cb * D2) + gC * (-ca * ca * D2);
+        // conic = (cc, -cb, ca) / det; with det - ca cc = -cb^2 the derivatives need no difference of near-equal terms
+        const float d_ca = D2 * (-cc * cc * gA + cb * cc * gB - cb * cb * gC);
+        const float d_cb = D2 * (2.f * cb * cc * gA - (ca * cc + cb * cb) * gB + 2.f * ca * cb * gC);
+        const float d_cc = D2 * (-cb * cb * gA + ca * cb * gB - ca * ca * gC);
         // symmetric gradient of the 3-D covariance, packed with the off-diagonal entries counted once each
         float dS[3][3];
 #pragma unroll

@@ -1,6 +1,6 @@
 /*
- * gs355 -- C ABI of the MI355X (gfx950) forward rasterizer for 3D Gaussian
- * splatting.
+ * gs355 -- C ABI of the MI355X (gfx950) rasterizer for 3D Gaussian splatting:
+ * the forward pass, its backward pass, and the anchor decode in front of it.
  *
  * This library replaces the native extension behind the reference's Python
  * package `opt_gaussian_rasterization` (third-party CUDA submodule, empty in

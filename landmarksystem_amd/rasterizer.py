@@ -28,6 +28,7 @@ plain forward pass.  When gradients are enabled and an input requires them
 library's backward pass; `means2D` then receives the screen-space gradient
 the reference's densification reads (gaussian_encoding.py:729-743).
 """
+from types import SimpleNamespace
 from typing import NamedTuple, Optional
 
 import torch
@@ -65,16 +66,20 @@ class _RasterizeGaussians(torch.autograd.Function):
         out = pipeline.render(inputs, ws=ws)
         # the next frame on this stream gets a fresh buffer; this one lives until the backward pass is done
         ctx.workspace, ws.buffer = ws.buffer, None
-        ctx.settings, ctx.out = settings, out
+        ctx.settings, ctx.key_capacity = settings, out.key_capacity
         ctx.set_materialize_grads(False)
-        ctx.save_for_backward(means3D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp)
+        # outputs go through save_for_backward too: kept on ctx directly they would tie it into a reference cycle
+        ctx.save_for_backward(means3D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp,
+                              out.image, out.depth, out.alpha, out.radii)
         ctx.means2D_like = None if means2D is None else (means2D.shape, means2D.dtype)
         ctx.mark_non_differentiable(out.radii)
         return out.image, out.radii, out.depth, out.alpha
 
     @staticmethod
     def backward(ctx, g_image, _g_radii, g_depth, g_alpha):
-        means3D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp = ctx.saved_tensors
+        (means3D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp,
+         image, depth, alpha, radii) = ctx.saved_tensors
+        out = SimpleNamespace(image=image, depth=depth, alpha=alpha, radii=radii, key_capacity=ctx.key_capacity)
         originals = dict(means3D=means3D, opacities=opacities, shs=shs, colors_precomp=colors_precomp, scales=scales,
                          rotations=rotations, cov3D_precomp=cov3D_precomp)
         needs = dict(zip(_INPUT_NAMES, ctx.needs_input_grad[1:]))
@@ -84,9 +89,9 @@ class _RasterizeGaussians(torch.autograd.Function):
                                       colors_precomp=colors_precomp, scales=scales, rotations=rotations,
                                       cov3D_precomp=cov3D_precomp)
         if g_image is None:
-            g_image = torch.zeros_like(ctx.out.image)
+            g_image = torch.zeros_like(image)
         want = [n for n in _INPUT_NAMES if needs[n]]
-        grads = pipeline.render_backward(inputs, ctx.out, ctx.workspace, g_image, g_depth, g_alpha, want=want)
+        grads = pipeline.render_backward(inputs, out, ctx.workspace, g_image, g_depth, g_alpha, want=want)
         ctx.workspace = None
         result = [None]
         for n in _INPUT_NAMES:

@@ -363,20 +363,25 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
 #pragma unroll
         for (int k = 0; k < 3; ++k) dmean[k] = Pm[4 * k] * d_phx + Pm[4 * k + 1] * d_phy + Pm[4 * k + 3] * d_phw;
 
-        // ---- 3-D covariance ----
-        float S[6], s[3] = {0.f, 0.f, 0.f}, q[4] = {0.f, 0.f, 0.f, 0.f}, R[3][3] = {};
+        // ---- 3-D covariance, Jacobian of the projection, 2-D covariance, conic: in double precision ----
+        // An elongated splat (axes 50:1) hides its thin axes in the low bits of the fp32 covariance, and its 2-D
+        // determinant is a difference of nearly equal products; the gradients of scale and rotation are small
+        // differences of terms built from them.  fp64 vector arithmetic runs at the fp32 rate on this chip and
+        // the kernel waits for memory, so the chain costs nothing in double and loses nothing.
+        typedef double real;
+        real S[6], s[3] = {0., 0., 0.}, q[4] = {0., 0., 0., 0.}, R[3][3] = {};
         if (g.cov3D_precomp) {
 #pragma unroll
             for (int k = 0; k < 6; ++k) S[k] = g.cov3D_precomp[6 * si + k];
         } else {
 #pragma unroll
-            for (int k = 0; k < 3; ++k) s[k] = f.scale_modifier * g.scales[3 * si + k];
+            for (int k = 0; k < 3; ++k) s[k] = (real)f.scale_modifier * (real)g.scales[3 * si + k];
 #pragma unroll
             for (int k = 0; k < 4; ++k) q[k] = g.rotations[4 * si + k];
-            const float r = q[0], qx = q[1], qy = q[2], qz = q[3];
-            R[0][0] = 1.f - 2.f * (qy * qy + qz * qz); R[0][1] = 2.f * (qx * qy - r * qz); R[0][2] = 2.f * (qx * qz + r * qy);
-            R[1][0] = 2.f * (qx * qy + r * qz); R[1][1] = 1.f - 2.f * (qx * qx + qz * qz); R[1][2] = 2.f * (qy * qz - r * qx);
-            R[2][0] = 2.f * (qx * qz - r * qy); R[2][1] = 2.f * (qy * qz + r * qx); R[2][2] = 1.f - 2.f * (qx * qx + qy * qy);
+            const real r = q[0], qx = q[1], qy = q[2], qz = q[3];
+            R[0][0] = 1. - 2. * (qy * qy + qz * qz); R[0][1] = 2. * (qx * qy - r * qz); R[0][2] = 2. * (qx * qz + r * qy);
+            R[1][0] = 2. * (qx * qy + r * qz); R[1][1] = 1. - 2. * (qx * qx + qz * qz); R[1][2] = 2. * (qy * qz - r * qx);
+            R[2][0] = 2. * (qx * qz - r * qy); R[2][1] = 2. * (qy * qz + r * qx); R[2][2] = 1. - 2. * (qx * qx + qy * qy);
             int n = 0;
 #pragma unroll
             for (int a = 0; a < 3; ++a)
@@ -384,90 +389,100 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
                 for (int c = a; c < 3; ++c)
                     S[n++] = R[a][0] * s[0] * R[c][0] * s[0] + R[a][1] * s[1] * R[c][1] * s[1] + R[a][2] * s[2] * R[c][2] * s[2];
         }
-        const float Sm[3][3] = {{S[0], S[1], S[2]}, {S[1], S[3], S[4]}, {S[2], S[4], S[5]}};
+        const real Sm[3][3] = {{S[0], S[1], S[2]}, {S[1], S[3], S[4]}, {S[2], S[4], S[5]}};
 
-        // ---- Jacobian of the projection, 2-D covariance, conic ----
-        const float pvx = V[0] * x + V[4] * y + V[8] * z + V[12];
-        const float pvy = V[1] * x + V[5] * y + V[9] * z + V[13];
-        const float tz = V[2] * x + V[6] * y + V[10] * z + V[14];
-        const float limx = 1.3f * f.tanfovx, limy = 1.3f * f.tanfovy;
-        const float rx = pvx / tz, ry = pvy / tz;
-        const float cx = rx > limx ? limx : rx < -limx ? -limx : 0.0f;  // non-zero: clamped to +-lim
-        const float cy = ry > limy ? limy : ry < -limy ? -limy : 0.0f;
-        const float tx = cx != 0.0f ? cx * tz : pvx, ty = cy != 0.0f ? cy * tz : pvy;
-        const float itz = 1.0f / tz, itz2 = itz * itz;
-        const float J00 = f.focal_x * itz, J02 = -(f.focal_x * tx) * itz2;
-        const float J11 = f.focal_y * itz, J12 = -(f.focal_y * ty) * itz2;
-        float a0[3], a1[3], Sa0[3], Sa1[3];
+        real Vd[12];  // the three columns of the view matrix the chain uses, rows 0..2
 #pragma unroll
         for (int k = 0; k < 3; ++k) {
-            a0[k] = J00 * V[4 * k] + J02 * V[4 * k + 2];
-            a1[k] = J11 * V[4 * k + 1] + J12 * V[4 * k + 2];
+            Vd[3 * k] = V[4 * k];
+            Vd[3 * k + 1] = V[4 * k + 1];
+            Vd[3 * k + 2] = V[4 * k + 2];
+        }
+        const real xd = x, yd = y, zd = z;
+        const real pvx = Vd[0] * xd + Vd[3] * yd + Vd[6] * zd + (real)V[12];
+        const real pvy = Vd[1] * xd + Vd[4] * yd + Vd[7] * zd + (real)V[13];
+        const real tz = Vd[2] * xd + Vd[5] * yd + Vd[8] * zd + (real)V[14];
+        const real fx = (real)f.W / (2. * (real)f.tanfovx), fy = (real)f.H / (2. * (real)f.tanfovy);
+        const real limx = 1.3 * (real)f.tanfovx, limy = 1.3 * (real)f.tanfovy;
+        const real itz = 1. / tz, itz2 = itz * itz;
+        const real rx = pvx * itz, ry = pvy * itz;
+        const real cx = rx > limx ? limx : rx < -limx ? -limx : 0.;  // non-zero: clamped to +-lim
+        const real cy = ry > limy ? limy : ry < -limy ? -limy : 0.;
+        const real tx = cx != 0. ? cx * tz : pvx, ty = cy != 0. ? cy * tz : pvy;
+        const real J00 = fx * itz, J02 = -(fx * tx) * itz2;
+        const real J11 = fy * itz, J12 = -(fy * ty) * itz2;
+        real a0[3], a1[3], Sa0[3], Sa1[3];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            a0[k] = J00 * Vd[3 * k] + J02 * Vd[3 * k + 2];
+            a1[k] = J11 * Vd[3 * k + 1] + J12 * Vd[3 * k + 2];
         }
 #pragma unroll
         for (int k = 0; k < 3; ++k) {
             Sa0[k] = Sm[k][0] * a0[0] + Sm[k][1] * a0[1] + Sm[k][2] * a0[2];
             Sa1[k] = Sm[k][0] * a1[0] + Sm[k][1] * a1[1] + Sm[k][2] * a1[2];
         }
-        const float ca = a0[0] * Sa0[0] + a0[1] * Sa0[1] + a0[2] * Sa0[2] + 0.3f;
-        const float cb = a0[0] * Sa1[0] + a0[1] * Sa1[1] + a0[2] * Sa1[2];
-        const float cc = a1[0] * Sa1[0] + a1[1] * Sa1[1] + a1[2] * Sa1[2] + 0.3f;
-        const float D = 1.0f / (ca * cc - cb * cb), D2 = D * D;
+        const real ca = a0[0] * Sa0[0] + a0[1] * Sa0[1] + a0[2] * Sa0[2] + 0.3;
+        const real cb = a0[0] * Sa1[0] + a0[1] * Sa1[1] + a0[2] * Sa1[2];
+        const real cc = a1[0] * Sa1[0] + a1[1] * Sa1[1] + a1[2] * Sa1[2] + 0.3;
+        const real D = 1. / (ca * cc - cb * cb), D2 = D * D;
         // conic = (cc, -cb, ca) / det; with det - ca cc = -cb^2 the derivatives need no difference of near-equal terms
-        const float d_ca = D2 * (-cc * cc * gA + cb * cc * gB - cb * cb * gC);
-        const float d_cb = D2 * (2.f * cb * cc * gA - (ca * cc + cb * cb) * gB + 2.f * ca * cb * gC);
-        const float d_cc = D2 * (-cb * cb * gA + ca * cb * gB - ca * ca * gC);
+        const real gAd = gA, gBd = gB, gCd = gC;
+        const real d_ca = D2 * (-cc * cc * gAd + cb * cc * gBd - cb * cb * gCd);
+        const real d_cb = D2 * (2. * cb * cc * gAd - (ca * cc + cb * cb) * gBd + 2. * ca * cb * gCd);
+        const real d_cc = D2 * (-cb * cb * gAd + ca * cb * gBd - ca * ca * gCd);
         // symmetric gradient of the 3-D covariance, packed with the off-diagonal entries counted once each
-        float dS[3][3];
+        real dS[3][3];
 #pragma unroll
         for (int k = 0; k < 3; ++k)
 #pragma unroll
             for (int l = 0; l < 3; ++l)
-                dS[k][l] = d_ca * a0[k] * a0[l] + d_cb * 0.5f * (a0[k] * a1[l] + a1[k] * a0[l]) + d_cc * a1[k] * a1[l];
-        float d_J00 = 0.f, d_J02 = 0.f, d_J11 = 0.f, d_J12 = 0.f;
+                dS[k][l] = d_ca * a0[k] * a0[l] + d_cb * 0.5 * (a0[k] * a1[l] + a1[k] * a0[l]) + d_cc * a1[k] * a1[l];
+        real d_J00 = 0., d_J02 = 0., d_J11 = 0., d_J12 = 0.;
 #pragma unroll
         for (int k = 0; k < 3; ++k) {
-            const float d_a0 = 2.f * d_ca * Sa0[k] + d_cb * Sa1[k];
-            const float d_a1 = 2.f * d_cc * Sa1[k] + d_cb * Sa0[k];
-            d_J00 += d_a0 * V[4 * k];
-            d_J02 += d_a0 * V[4 * k + 2];
-            d_J11 += d_a1 * V[4 * k + 1];
-            d_J12 += d_a1 * V[4 * k + 2];
+            const real d_a0 = 2. * d_ca * Sa0[k] + d_cb * Sa1[k];
+            const real d_a1 = 2. * d_cc * Sa1[k] + d_cb * Sa0[k];
+            d_J00 += d_a0 * Vd[3 * k];
+            d_J02 += d_a0 * Vd[3 * k + 2];
+            d_J11 += d_a1 * Vd[3 * k + 1];
+            d_J12 += d_a1 * Vd[3 * k + 2];
         }
-        const float itz3 = itz2 * itz;
-        const float d_tx = d_J02 * (-f.focal_x * itz2), d_ty = d_J12 * (-f.focal_y * itz2);
-        const float d_tz = d_J00 * (-f.focal_x * itz2) + d_J11 * (-f.focal_y * itz2) +
-                           d_J02 * (2.f * f.focal_x * tx * itz3) + d_J12 * (2.f * f.focal_y * ty * itz3);
-        const float d_pvx = cx != 0.0f ? 0.0f : d_tx, d_pvy = cy != 0.0f ? 0.0f : d_ty;
-        const float d_pvz = d_tz + cx * d_tx + cy * d_ty + g_depth;
+        const real itz3 = itz2 * itz;
+        const real d_tx = d_J02 * (-fx * itz2), d_ty = d_J12 * (-fy * itz2);
+        const real d_tz = d_J00 * (-fx * itz2) + d_J11 * (-fy * itz2) + d_J02 * (2. * fx * tx * itz3) +
+                          d_J12 * (2. * fy * ty * itz3);
+        const real d_pvx = cx != 0. ? 0. : d_tx, d_pvy = cy != 0. ? 0. : d_ty;
+        const real d_pvz = d_tz + cx * d_tx + cy * d_ty + (real)g_depth;
 #pragma unroll
-        for (int k = 0; k < 3; ++k) dmean[k] += V[4 * k] * d_pvx + V[4 * k + 1] * d_pvy + V[4 * k + 2] * d_pvz;
+        for (int k = 0; k < 3; ++k)
+            dmean[k] += (float)(Vd[3 * k] * d_pvx + Vd[3 * k + 1] * d_pvy + Vd[3 * k + 2] * d_pvz);
 
         if (g.cov3D_precomp) {
-            dcov[0] = dS[0][0]; dcov[1] = 2.f * dS[0][1]; dcov[2] = 2.f * dS[0][2];
-            dcov[3] = dS[1][1]; dcov[4] = 2.f * dS[1][2]; dcov[5] = dS[2][2];
+            dcov[0] = (float)dS[0][0]; dcov[1] = (float)(2. * dS[0][1]); dcov[2] = (float)(2. * dS[0][2]);
+            dcov[3] = (float)dS[1][1]; dcov[4] = (float)(2. * dS[1][2]); dcov[5] = (float)dS[2][2];
         } else {
             // Sigma = L L^T with L = R diag(s): dL = 2 dS L
-            float dR[3][3];
+            real dR[3][3];
 #pragma unroll
             for (int k = 0; k < 3; ++k) {
-                float ds = 0.f;
+                real ds = 0.;
 #pragma unroll
                 for (int a = 0; a < 3; ++a) {
-                    const float dL = 2.f * (dS[a][0] * R[0][k] + dS[a][1] * R[1][k] + dS[a][2] * R[2][k]) * s[k];
+                    const real dL = 2. * (dS[a][0] * R[0][k] + dS[a][1] * R[1][k] + dS[a][2] * R[2][k]) * s[k];
                     ds += dL * R[a][k];
                     dR[a][k] = dL * s[k];
                 }
-                dscale[k] = ds * f.scale_modifier;
+                dscale[k] = (float)(ds * (real)f.scale_modifier);
             }
-            const float r = q[0], qx = q[1], qy = q[2], qz = q[3];
-            drot[0] = 2.f * (-qz * dR[0][1] + qy * dR[0][2] + qz * dR[1][0] - qx * dR[1][2] - qy * dR[2][0] + qx * dR[2][1]);
-            drot[1] = 2.f * (qy * dR[0][1] + qz * dR[0][2] + qy * dR[1][0] - 2.f * qx * dR[1][1] - r * dR[1][2] +
-                             qz * dR[2][0] + r * dR[2][1] - 2.f * qx * dR[2][2]);
-            drot[2] = 2.f * (-2.f * qy * dR[0][0] + qx * dR[0][1] + r * dR[0][2] + qx * dR[1][0] + qz * dR[1][2] -
-                             r * dR[2][0] + qz * dR[2][1] - 2.f * qy * dR[2][2]);
-            drot[3] = 2.f * (-2.f * qz * dR[0][0] - r * dR[0][1] + qx * dR[0][2] + r * dR[1][0] - 2.f * qz * dR[1][1] +
-                             qy * dR[1][2] + qx * dR[2][0] + qy * dR[2][1]);
+            const real r = q[0], qx = q[1], qy = q[2], qz = q[3];
+            drot[0] = (float)(2. * (-qz * dR[0][1] + qy * dR[0][2] + qz * dR[1][0] - qx * dR[1][2] - qy * dR[2][0] + qx * dR[2][1]));
+            drot[1] = (float)(2. * (qy * dR[0][1] + qz * dR[0][2] + qy * dR[1][0] - 2. * qx * dR[1][1] - r * dR[1][2] +
+                                    qz * dR[2][0] + r * dR[2][1] - 2. * qx * dR[2][2]));
+            drot[2] = (float)(2. * (-2. * qy * dR[0][0] + qx * dR[0][1] + r * dR[0][2] + qx * dR[1][0] + qz * dR[1][2] -
+                                    r * dR[2][0] + qz * dR[2][1] - 2. * qy * dR[2][2]));
+            drot[3] = (float)(2. * (-2. * qz * dR[0][0] - r * dR[0][1] + qx * dR[0][2] + r * dR[1][0] - 2. * qz * dR[1][1] +
+                                    qy * dR[1][2] + qx * dR[2][0] + qy * dR[2][1]));
         }
 
         // ---- colour: view direction, SH basis and its gradient ----

@@ -42,6 +42,13 @@ def oracle_backward(scene, gi, gd=None, ga=None, colors=None, cov=None, sh_degre
     cg = oracle_gaussians(scene, colors_precomp=None if colors is None else colors.numpy(),
                           cov3D_precomp=None if cov is None else cov.numpy())
     fwd = co.render(cf, cg)
+    # Pixels where the forward pass took a discrete decision (alpha < 1/255, T (1 - alpha) < 1e-4) within rounding
+    # of its threshold may legitimately decide otherwise on the GPU (the forward parity tests exclude them too):
+    # their cotangents are zeroed, IN PLACE, so that the GPU run that follows sees the same loss.
+    keep = torch.from_numpy(fwd["fragile"] == 0)
+    for t in (gi, gd, ga):
+        if t is not None:
+            t.mul_(keep)
     return co.render_backward(cf, cg, fwd, gi.numpy(), None if gd is None else gd.numpy()[0],
                               None if ga is None else ga.numpy()[0]), fwd
 
@@ -206,21 +213,12 @@ def test_full_size_headline_frame_backward_equals_the_oracle(gpu_device):
     ref, fwd = oracle_backward(scene, gi)
     got, out = abi_backward(scene, gpu_device, gi)
     assert out.num_keys == fwd["num_keys"] > 10_000_000
-    # 6M ill-conditioned Gaussians (anisotropy up to 1:50) through an fp32 chain of 1/det^2 terms: a handful of the
-    # 10^8 gradient elements lose more digits than the bar of the smaller scenes allows.  Every element within 1e-3
-    # of the tensor's largest magnitude, and all but one in 10^5 within the usual bar.
     for name, value in got.items():
-        r = ref[name]
-        err = np.abs(np.asarray(value, np.float64).reshape(r.shape) - r)
-        scale = np.abs(r).max()
-        assert err.max() <= 1e-3 * scale, "6M %s: %g of %g" % (name, err.max(), scale)
-        row = np.abs(r).reshape(r.shape[0], -1).max(axis=1).reshape((-1,) + (1,) * (r.ndim - 1))
-        outside = (err > ABS_OF_MAX * scale + REL * row).mean()
-        assert outside <= 1e-5, "6M %s: fraction %g outside the bar" % (name, outside)
+        assert_grad_close(value, ref[name], "6M " + name)
     again, _ = abi_backward(scene, gpu_device, gi)
     for name, value in got.items():
         scale = np.abs(value).max()
-        assert np.abs(value - again[name]).max() <= 1e-3 * scale, name  # the same ill-conditioned few amplify last bits
+        assert np.abs(value - again[name]).max() <= 1e-5 * scale, name
 
 
 def test_backward_after_the_classic_pipeline(gpu_device):

@@ -260,3 +260,30 @@ def test_backward_edge_cases(gpu_device):
     grads = pipeline.render_backward(inp, out, ws.buffer, gi.to(gpu_device))
     torch.cuda.synchronize()
     assert all(v.numel() == 0 for v in grads.values())
+
+
+def test_gradient_descent_through_the_model_fits_a_target(gpu_device):
+    """End to end, as the reference's trainer uses the rasterizer (origin_gs/gs_trainer.py:117-137): a perturbed copy
+    of a scene is optimised with Adam against the original's rendering; the L1 loss must fall by more than half."""
+    scene = scenes.tiny_scene(P=400, width=96, height=64, sh_degree=1, seed=41, log_scale_mean=-1.8)
+    make = lambda s: models.GaussianModel.from_activated(s.means3D, s.scales, s.rotations, s.opacities, s.shs,  # noqa: E731
+                                                         sh_degree=1).to(gpu_device)
+    with torch.no_grad():
+        target = make(scene).eval()(scene.camera)
+    g = torch.Generator().manual_seed(0)
+    scene.means3D += 0.03 * torch.randn(scene.P, 3, generator=g)
+    scene.shs += 0.1 * torch.randn(scene.shs.shape, generator=g)
+    scene.scales *= torch.exp(0.2 * torch.randn(scene.P, 3, generator=g))
+    model = make(scene).train()
+    for p in model.parameters():
+        p.requires_grad_(True)
+    opt = torch.optim.Adam(model.parameters(), lr=5e-3)
+    losses = []
+    for _ in range(60):
+        loss = (model(scene.camera) - target).abs().mean()
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert losses[-1] < 0.5 * losses[0], (losses[0], losses[-1])
+    assert all(np.isfinite(losses))

@@ -276,6 +276,22 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     fps = args.steps / elapsed
 
+    # per-frame latency: the reference's own protocol (synchronise, forward, synchronise around every frame, the
+    # first five frames dropped: benchmarks/nerf/origin_gs/gs_evaluator.py:104-114,136), and its spread
+    per_frame = []
+    with torch.no_grad():
+        for _ in range(min(args.steps, 60) + 5):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            rast(**kwargs)
+            torch.cuda.synchronize()
+            per_frame.append((time.perf_counter() - t0) * 1e3)
+    per_frame = sorted(per_frame[5:])
+    pick = lambda q: round(per_frame[min(len(per_frame) - 1, int(q * len(per_frame)))], 4)  # noqa: E731
+    latency = {"mean_ms": round(sum(per_frame) / len(per_frame), 4), "median_ms": pick(0.5), "p10_ms": pick(0.1),
+               "p90_ms": pick(0.9), "frames": len(per_frame),
+               "frames_per_s": round(1e3 * len(per_frame) / sum(per_frame), 2)}
+
     # the same frames with two in flight (alternating HIP streams, one workspace each): the next frame's
     # HBM-bound preprocess overlaps the current frame's VALU-bound blend.  Reported beside `value`, never as it.
     # Opt-in (--two-in-flight): overlapping kernels would distort the per-kernel durations of a profiler trace.
@@ -443,6 +459,7 @@ def main():
         "stages": stages,
         "model_forward_frames_per_s": model_fps,
         "two_frames_in_flight_frames_per_s": fps_two_in_flight,
+        "synchronised_per_frame": latency,
     }
     if not args.no_cpu_baseline:
         try:

@@ -281,9 +281,10 @@ class GaussianModel(nn.Module):
             scales, rotations = self.get_scaling, self.get_rotation
         if override_color is not None:
             colors_precomp = override_color
-        elif self.convert_SHs_python:
-            raise NotImplementedError("convert_SHs_python: SH -> RGB runs inside the preprocess kernel")
         else:
+            # convert_SHs_python only chooses where SH -> RGB is evaluated in the reference (torch statements,
+            # origin_gs/gs_model.py:184-193, or its rasterizer); here the preprocess kernel evaluates the same
+            # expression, clamp_min(eval_sh + 0.5, 0), for either setting
             shs = self.get_features
         if fused:
             rendered_image, radii, _ = self.renderer(

@@ -392,6 +392,39 @@ def test_tile_sort_fallback_on_massive_depth_ties(gpu_device, same, spread, labe
     assert run_lengths.max() >= same, label
 
 
+def test_splats_whose_extent_lands_on_a_tile_edge(gpu_device):
+    """Adversarial for the integer pipeline: Gaussians picked because an edge of their extent (centre -/+ radius)
+    falls closest to a multiple of 16 pixels, each repeated with its mean moved by up to 64 units in the last place
+    along every axis, so that many of them sit within rounding of a tile boundary or of a radius step.  Radii,
+    tile counts, keys, sorted order and ranges must still match the oracle bit for bit."""
+    pool = scenes.config1(P=200_000, width=320, height=208)
+    pre = co.preprocess(oracle_frame(pool), oracle_gaussians(pool))
+    vis = pre["radii"] > 0
+    r = pre["radii"].astype(np.float32)
+    edges = np.stack([pre["xy"][:, 0] - r, pre["xy"][:, 0] + r + 15.0, pre["xy"][:, 1] - r, pre["xy"][:, 1] + r + 15.0], 1) / 16.0
+    dist = np.abs(edges - np.round(edges)).min(axis=1)
+    dist[~vis] = np.inf
+    pick = np.argsort(dist)[:400]
+    assert dist[pick].max() < 2e-3
+    means, idx = [], []
+    base = pool.means3D.numpy()[pick]
+    for axis in range(3):
+        for steps in (-64, -8, -1, 0, 1, 8, 64):  # units in the last place, through the bit pattern
+            m = base.copy()
+            m[:, axis] = (m[:, axis].view(np.int32) + np.int32(steps)).view(np.float32)
+            means.append(m)
+            idx.append(pick)
+    idx = np.concatenate(idx)
+    scene = scenes.GaussianScene("edges", torch.from_numpy(np.concatenate(means)), pool.scales[idx], pool.rotations[idx],
+                                 pool.opacities[idx], pool.shs[idx], pool.sh_degree, pool.cameras, pool.bg)
+    ref = oracle_render(scene)
+    assert len(np.unique(ref["pre"]["tiles_touched"][:len(pick) * 7].reshape(7, -1), axis=0)) > 1  # the nudges do flip decisions
+    check_against_oracle(run_all_stages(scene, gpu_device), ref, "tile edges")
+    fast = run_fast_path(scene, gpu_device)
+    for name in ("ranges", "sorted_keys", "sorted_values"):
+        np.testing.assert_array_equal(fast[name], ref[name], err_msg=name)
+
+
 def test_images_beyond_the_tile_bucket_limit(gpu_device):
     """More than 36000 tiles: the per-tile counters of the bucketed stages no longer fit in LDS.  The C entry point
     says so; the Python driver renders such frames through the classic stages, with the same result contract."""

@@ -265,7 +265,7 @@ class GaussianModel(nn.Module):
         differentiable with respect to the parameters, and `viewspace_points` receives the screen-space gradient
         that the reference's densification reads (:129-139, :225-236)."""
         viewpoint_camera = viewpoint_camera.to(self._xyz.device)
-        fused = (self.fuse_prefilter and not self.training and render_exclude_filter is None
+        fused = (self.fuse_prefilter and render_exclude_filter is None
                  and scaling_modifier == 1.0)  # the reference's prefilter always uses scale modifier 1
         if not fused:
             voxel_visible_mask = self.prefilter_voxel(viewpoint_camera)
@@ -286,25 +286,27 @@ class GaussianModel(nn.Module):
             # origin_gs/gs_model.py:184-193, or its rasterizer); here the preprocess kernel evaluates the same
             # expression, clamp_min(eval_sh + 0.5, 0), for either setting
             shs = self.get_features
+        screenspace_points = None
+        if self.training and torch.is_grad_enabled():
+            screenspace_points = torch.zeros_like(means3D, requires_grad=True) + 0
+            screenspace_points.retain_grad()
+        self.viewspace_points = screenspace_points
         if fused:
             rendered_image, radii, _ = self.renderer(
-                means3D=means3D, means2D=None, shs=shs, colors_precomp=colors_precomp, opacities=opacity,
+                means3D=means3D, means2D=screenspace_points, shs=shs, colors_precomp=colors_precomp, opacities=opacity,
                 scales=scales, rotations=rotations, cov3D_precomp=cov3D_precomp)
-            self._radii_all, self._radii, self._visibility_filter = radii, None, None
+            # eval: radii of the visible subset, as after the reference's gather; training: of all Gaussians
+            self._radii_all, self._visibility_filter = radii, None
+            self._radii = radii if self.training else None
             return rendered_image
         if not self.training:  # the reference renders only what its prefilter kept (origin_gs/gs_model.py:199-208)
             mask = voxel_visible_mask.nonzero().squeeze(-1)
             pick = lambda t: None if t is None else t[mask]  # noqa: E731
             means3D, shs, colors_precomp, opacity = pick(means3D), pick(shs), pick(colors_precomp), pick(opacity)
             scales, rotations, cov3D_precomp = pick(scales), pick(rotations), pick(cov3D_precomp)
-        screenspace_points = None
-        if self.training and torch.is_grad_enabled():
-            screenspace_points = torch.zeros_like(means3D, requires_grad=True) + 0
-            screenspace_points.retain_grad()
         rendered_image, radii, _ = self.renderer(
             means3D=means3D, means2D=screenspace_points, shs=shs, colors_precomp=colors_precomp, opacities=opacity,
             scales=scales, rotations=rotations, cov3D_precomp=cov3D_precomp)
-        self.viewspace_points = screenspace_points
         self._radii_all, self.visibility_filter, self.radii = None, voxel_visible_mask, radii
         return rendered_image
 

@@ -202,6 +202,19 @@ def test_training_step_of_the_vanilla_model(gpu_device):
     for name, p in model.named_parameters():
         assert p.grad is not None and torch.isfinite(p.grad).all(), name
     assert model._xyz.grad.abs().max() > 0 and model._features_rest.grad.abs().max() > 0
+    assert model.radii.shape[0] == scene.P  # training: no gather, radii of every Gaussian (what densification indexes)
+    # the single-pass variant (no separate visibility prefilter) leaves the same by-products and gradients
+    fused = models.GaussianModel.from_activated(scene.means3D, scene.scales, scene.rotations, scene.opacities,
+                                                scene.shs, fuse_prefilter=True).to(gpu_device).train()
+    for p in fused.parameters():
+        p.requires_grad_(True)
+    image2 = fused(scene.camera)
+    (image2 - target).abs().mean().backward()
+    assert torch.equal(image2, image) and torch.equal(fused.visibility_filter, vis)
+    assert torch.equal(fused.radii, model.radii)
+    torch.testing.assert_close(fused._xyz.grad, model._xyz.grad, rtol=1e-4, atol=1e-6 * float(model._xyz.grad.abs().max()))
+    torch.testing.assert_close(fused.viewspace_points.grad, model.viewspace_points.grad, rtol=1e-4,
+                               atol=1e-6 * float(model.viewspace_points.grad.abs().max()))
 
 
 def test_full_size_headline_frame_backward_equals_the_oracle(gpu_device):

@@ -21,6 +21,10 @@ namespace gs355 {
 namespace {
 
 constexpr int kInlineTiles = 32;  // splats touching more tiles than this are expanded by the whole workgroup
+#ifndef GS355_BIN_ITEMS
+#define GS355_BIN_ITEMS 4
+#endif
+constexpr int kBinItems = GS355_BIN_ITEMS;  // Gaussians per thread and round of the binning walk
 
 // ---------------------------------------------------------------------------
 // Binning.  Workgroup c owns Gaussians [c * per_group, (c+1) * per_group) and a
@@ -41,7 +45,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P
                                                           uint64_t* __restrict__ buckets)
 {
     extern __shared__ uint32_t s_tile[];  // [tiles]
-    __shared__ uint32_t s_queue[kBinThreads];
+    __shared__ uint32_t s_queue[kBinItems * kBinThreads];
     __shared__ uint32_t s_nqueue, s_visible;
 
     if (kScatter && header->overflow) return;
@@ -54,26 +58,38 @@ __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P
     const int g_end = min(P, g_begin + per_group);
     uint32_t visible = 0;
 
-    for (int base = g_begin; base < g_end; base += kBinThreads) {
+    for (int base = g_begin; base < g_end; base += kBinItems * kBinThreads) {
         if (tid == 0) s_nqueue = 0;
         __syncthreads();
-        const int i = base + tid;
-        if (i < g_end) {
-            const uint64_t r = rects[i];
-            const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
-                      y1 = (int)(r >> 48);
-            const int w = x1 - x0, area = w * (y1 - y0);
-            if (area > 0) {
-                ++visible;
-                if (area > kInlineTiles) {
-                    s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
-                } else {
-                    const uint64_t payload = kScatter ? ((uint64_t)depth_bits[i] << 32) | (uint64_t)(uint32_t)i : 0ull;
-                    for (int ty = y0; ty < y1; ++ty)
-                        for (int tx = x0; tx < x1; ++tx) {
-                            const uint32_t slot = atomicAdd(&s_tile[ty * f.grid_x + tx], 1u);
-                            if (kScatter) buckets[slot] = payload;
-                        }
+        // a thread's Gaussians of this round: their rectangles (and depths) are requested together
+        uint64_t rr[kBinItems];
+        uint32_t dd[kBinItems];
+#pragma unroll
+        for (int u = 0; u < kBinItems; ++u) {
+            const int i = min(base + u * kBinThreads + tid, g_end - 1);
+            rr[u] = rects[i];
+            dd[u] = kScatter ? depth_bits[i] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < kBinItems; ++u) {
+            const int i = base + u * kBinThreads + tid;
+            if (i < g_end) {
+                const uint64_t r = rr[u];
+                const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
+                          y1 = (int)(r >> 48);
+                const int w = x1 - x0, area = w * (y1 - y0);
+                if (area > 0) {
+                    ++visible;
+                    if (area > kInlineTiles) {
+                        s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
+                    } else {
+                        const uint64_t payload = kScatter ? ((uint64_t)dd[u] << 32) | (uint64_t)(uint32_t)i : 0ull;
+                        for (int ty = y0; ty < y1; ++ty)
+                            for (int tx = x0; tx < x1; ++tx) {
+                                const uint32_t slot = atomicAdd(&s_tile[ty * f.grid_x + tx], 1u);
+                                if (kScatter) buckets[slot] = payload;
+                            }
+                    }
                 }
             }
         }

@@ -445,3 +445,42 @@ def test_images_beyond_the_tile_bucket_limit(gpu_device):
     solid = ref["fragile"] == 0
     image = got.image.cpu().numpy()
     assert np.abs(image - ref["image"])[:, solid].max() <= 1e-4 and psnr(image, ref["image"]) >= 60.0
+
+
+def test_non_finite_and_degenerate_inputs(gpu_device):
+    """Gaussians with NaN / infinite positions, NaN, zero or enormous scales, zero quaternions and NaN opacity among
+    ordinary ones: nothing hangs, the poisoned ones are culled or rendered exactly as the oracle does, the rest of
+    the frame is untouched."""
+    scene = scenes.tiny_scene(P=400, width=96, height=64, sh_degree=1, seed=77)
+    nan, inf = float("nan"), float("inf")
+    scene.means3D[0] = torch.tensor([nan, 0.0, 0.0])
+    scene.means3D[1] = torch.tensor([0.0, inf, 0.0])
+    scene.means3D[2] = torch.tensor([0.0, 0.0, -inf])
+    scene.means3D[3] = torch.tensor([1e30, -1e30, 1e30])
+    scene.scales[4] = torch.tensor([nan, 0.1, 0.1])
+    scene.scales[5] = torch.tensor([0.0, 0.0, 0.0])
+    scene.scales[6] = torch.tensor([1e18, 1e18, 1e18])
+    scene.scales[7] = torch.tensor([inf, 0.1, 0.1])
+    scene.rotations[8] = torch.zeros(4)
+    scene.rotations[9] = torch.tensor([nan, 0.0, 0.0, 1.0])
+    scene.scales[10] = torch.tensor([30.0, 1e-6, 1e-6])  # a needle across the whole image
+    scene.opacities[11] = 0.0
+    scene.opacities[12] = 1.0
+    scene.shs[13] = 1e30
+    ref = oracle_render(scene)
+    got = run_all_stages(scene, gpu_device)
+    np.testing.assert_array_equal(got["radii"], ref["radii"])
+    np.testing.assert_array_equal(got["tiles_touched"], ref["pre"]["tiles_touched"])
+    np.testing.assert_array_equal(got["sorted_keys"], ref["sorted_keys"])
+    np.testing.assert_array_equal(got["sorted_values"], ref["sorted_values"])
+    np.testing.assert_array_equal(got["ranges"], ref["ranges"])
+    assert (ref["radii"][[0, 1, 2, 3, 4, 6, 7, 9]] == 0).all()  # not representable on screen: culled
+    assert ref["radii"][5] > 0 and ref["radii"][8] > 0 and ref["radii"][10] > 2000  # low-pass floor; identity; needle
+    fast = run_fast_path(scene, gpu_device)
+    np.testing.assert_array_equal(fast["sorted_keys"], ref["sorted_keys"])
+    for name in ("image", "alpha"):
+        g, r = got[name], ref[name]
+        np.testing.assert_array_equal(np.isfinite(g), np.isfinite(r), err_msg=name)
+        ok = np.isfinite(r) & (ref["fragile"] == 0)
+        assert (np.abs(g - r)[ok] <= 1e-4 * np.maximum(1.0, np.abs(r[ok]))).all(), name  # one colour is 1e29
+        np.testing.assert_array_equal(fast[name], g)

@@ -315,6 +315,7 @@ class ScaffoldGS(nn.Module):
     """Scaffold-GS: anchors decoded into neural Gaussians per frame."""
 
     _ckpt_kind = "scaffold"
+    _decoder_options = (("use_feat_bank", False), ("view_dim", 3))
 
     def __init__(self, anchor=None, anchor_feat=None, offset=None, scaling=None, rotation=None, n_offsets: int = 10,
                  feat_dim: int = 32, add_opacity_dist: bool = True, add_cov_dist: bool = True,
@@ -335,8 +336,10 @@ class ScaffoldGS(nn.Module):
             add_color_dist = _cfg(config, "add_color_dist", add_color_dist)
             white_bkgd, act_cache = _cfg(config, "white_bkgd", white_bkgd), _cfg(config, "act_cache", act_cache)
             self.fuse_prefilter = _cfg(config, "fuse_prefilter", fuse_prefilter)
-            for name, allowed in (("use_feat_bank", False), ("appearance_dim", 0), ("add_level", False),
-                                  ("view_dim", 3)):
+            # the options the reference's model hands to its AnchorDecoder: scaffold_gs/gs_model.py:126-134 passes
+            # neither add_level nor appearance_dim (its config's add_level=True default never reaches the decoder);
+            # octree_gs/gs_model.py:165-176 passes both
+            for name, allowed in self._decoder_options:
                 if _cfg(config, name, allowed) != allowed:
                     raise NotImplementedError("%s=%r: the fused anchor decode supports %s=%r only"
                                               % (name, _cfg(config, name, allowed), name, allowed))
@@ -487,6 +490,7 @@ class OctreeGS(ScaffoldGS):
     """Octree-GS: Scaffold-GS plus a per-frame level-of-detail mask over the anchors."""
 
     _ckpt_kind = "octree"
+    _decoder_options = ScaffoldGS._decoder_options + (("appearance_dim", 0), ("add_level", False))
     _encoding_keys = ScaffoldGS._encoding_keys + ("_level", "_extra_level")
 
     def __init__(self, anchor=None, anchor_feat=None, offset=None, scaling=None, rotation=None, level=None,

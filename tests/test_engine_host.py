@@ -107,6 +107,11 @@ def test_config_built_models_load_their_checkpoints(tmp_path):
     assert all(torch.equal(a, b) for a, b in zip(o.parameters(), empty.parameters()))
     with pytest.raises(NotImplementedError, match="appearance_dim"):
         OctreeGS(dict(appearance_dim=32))
+    # the Scaffold-GS model never hands add_level / appearance_dim to its decoder (scaffold_gs/gs_model.py:126-134),
+    # so its config's add_level=True default (:33) must be accepted
+    ScaffoldGS(dict(n_offsets=10, feat_dim=32, add_level=True, appearance_dim=32))
+    with pytest.raises(NotImplementedError, match="use_feat_bank"):
+        ScaffoldGS(dict(use_feat_bank=True))
 
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU error")

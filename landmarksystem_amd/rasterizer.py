@@ -33,6 +33,7 @@ from typing import NamedTuple, Optional
 
 import torch
 from torch import nn
+from torch.autograd.function import once_differentiable
 
 from . import pipeline
 
@@ -76,6 +77,7 @@ class _RasterizeGaussians(torch.autograd.Function):
         return out.image, out.radii, out.depth, out.alpha
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, g_image, _g_radii, g_depth, g_alpha):
         (means3D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp,
          image, depth, alpha, radii) = ctx.saved_tensors

@@ -292,6 +292,17 @@ GS355_API int gs355_decode_scratch_bytes(int32_t A, size_t *bytes);
 GS355_API int gs355_decode_count(const gs355_decoder *dec, const gs355_anchors *an, uint32_t *counts, uint32_t *offsets,
                        void *scratch, size_t scratch_bytes, void *stream);
 
+/* gs355_decode_count for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same inputs, outputs and
+ * results as gs355_decode_count; the scan's scratch is a fixed array inside the library (one copy per GPU,
+ * 49 440 bytes, held until the process ends) instead of a caller buffer, and no allocating routine is called.
+ * At most 2^24 anchors: more returns GS355_ENOSPC.  The device that owns `stream` and the buffers must be the
+ * current device.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams
+ * or threads) race; calls on one stream are ordered.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress), so make that call outside any graph capture. */
+GS355_API int gs355_decode_count_static(const gs355_decoder *dec, const gs355_anchors *an, uint32_t *counts,
+                                        uint32_t *offsets, void *stream);
+
 /* Pass 2: decode all heads and write the kept Gaussians in boolean-mask order (row-major over visible anchor,
  * offset) into outputs with room for `capacity` Gaussians. */
 GS355_API int gs355_decode_emit(const gs355_decoder *dec, const gs355_anchors *an, const uint32_t *offsets, int64_t capacity,

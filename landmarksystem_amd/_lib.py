@@ -20,7 +20,7 @@ MAX_FAST_TILES = 36000
 
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
            "gs355_visible_filter", "gs355_anchor_filter", "gs355_decode_scratch_bytes", "gs355_decode_count",
-           "gs355_decode_emit", "gs355_backward_scratch_bytes", "gs355_render_backward")
+           "gs355_decode_count_static", "gs355_decode_emit", "gs355_backward_scratch_bytes", "gs355_render_backward")
 
 
 class Frame(C.Structure):
@@ -175,6 +175,8 @@ def load() -> C.CDLL:
     lib.gs355_decode_count.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_void_p, C.c_void_p,
                                        C.c_size_t, C.c_void_p]
     lib.gs355_decode_count.restype = C.c_int
+    lib.gs355_decode_count_static.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.gs355_decode_count_static.restype = C.c_int
     lib.gs355_decode_emit.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_int64,
                                       C.POINTER(Decoded), C.c_void_p]
     lib.gs355_decode_emit.restype = C.c_int

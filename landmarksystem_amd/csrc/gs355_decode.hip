@@ -32,6 +32,8 @@
 // anchor, offset).  Two launches: count kept offsets per anchor (opacity head
 // only) -> exclusive scan -> emit (all heads; the opacity head is recomputed
 // with the identical instruction sequence, so counts and emission agree).
+#include <atomic>
+
 #include "gs355_internal.h"
 
 namespace gs355 {
@@ -468,6 +470,37 @@ static dim3 decode_grid(int A, int cap)
 
 using namespace gs355;
 
+// ---- gs355_decode_count for callers that cannot allocate -----------------------------------------------------
+// The scan's block sums live in a file-scope device array instead of a caller-provided scratch buffer.  Every
+// GPU holds its own copy of the array at its own address; host code never uses the array's name as an address
+// (it is a host-side stand-in) but the pointer hipGetSymbolAddress returns for the current device, resolved
+// once per device and kept.
+constexpr int32_t kStaticCountMaxAnchors = 1 << 24;
+constexpr size_t kStaticScratchWords = ((size_t)kStaticCountMaxAnchors / kScanTile) * 3 + 8 + 64;
+static __device__ __align__(256) uint32_t scratch[kStaticScratchWords];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<uint32_t*> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(uint32_t** out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_error(GS355_EHIP, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return set_error(GS355_EINVAL, "device index %d is outside [0, %d)", dev, kMaxDevices);
+    uint32_t* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* q = nullptr;
+        e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !q)
+            return set_error(GS355_EHIP, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        p = static_cast<uint32_t*>(q);
+        g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing threads resolve the same address
+    }
+    *out = p;
+    return GS355_OK;
+}
+
 extern "C" {
 
 int gs355_decode_scratch_bytes(int32_t A, size_t* bytes)
@@ -479,13 +512,13 @@ int gs355_decode_scratch_bytes(int32_t A, size_t* bytes)
 }
 
 int gs355_decode_count(const gs355_decoder* dec, const gs355_anchors* an, uint32_t* counts, uint32_t* offsets,
-                       void* scratch, size_t scratch_bytes, void* stream)
+                       void* scratch_buf, size_t scratch_bytes, void* stream)
 {
     DecodeArgs a;
     int rc = fill_args(dec, an, &a);
     if (rc) return rc;
     if (a.A == 0) return GS355_OK;
-    if (!counts || !offsets || !scratch) return set_error(GS355_EINVAL, "counts / offsets / scratch is NULL");
+    if (!counts || !offsets || !scratch_buf) return set_error(GS355_EINVAL, "counts / offsets / scratch is NULL");
     size_t need = 0;
     gs355_decode_scratch_bytes(a.A, &need);
     if (scratch_bytes < need)
@@ -494,7 +527,31 @@ int gs355_decode_count(const gs355_decoder* dec, const gs355_anchors* an, uint32
     hipLaunchKernelGGL(decode_kernel<true>, decode_grid(a.A, 1024), dim3(256), 0, s, a, counts, (const uint32_t*)nullptr, 0u,
                        (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr);
     GS355_CHECK_LAUNCH("decode: count");
-    return launch_exclusive_scan(counts, offsets, (size_t)a.A, static_cast<uint32_t*>(scratch), s);
+    return launch_exclusive_scan(counts, offsets, (size_t)a.A, static_cast<uint32_t*>(scratch_buf), s);
+}
+
+int gs355_decode_count_static(const gs355_decoder* dec, const gs355_anchors* an, uint32_t* counts, uint32_t* offsets,
+                              void* stream)
+{
+    DecodeArgs a;
+    int rc = fill_args(dec, an, &a);
+    if (rc) return rc;
+    if (a.A > kStaticCountMaxAnchors)
+        return set_error(GS355_ENOSPC, "gs355_decode_count_static handles at most %d anchors (got %d); use gs355_decode_count",
+                         kStaticCountMaxAnchors, a.A);
+    if (a.A == 0) return GS355_OK;
+    if (!counts || !offsets) return set_error(GS355_EINVAL, "counts / offsets is NULL");
+    static_assert(kStaticScratchWords * sizeof(uint32_t) >=
+                      (((size_t)kStaticCountMaxAnchors + kScanTile - 1) / kScanTile * 3 + 8) * sizeof(uint32_t) + 256,
+                  "static scratch covers the scan of the largest accepted anchor count");
+    uint32_t* tmp = nullptr;
+    if ((rc = static_scratch(&tmp))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(decode_kernel<true>, decode_grid(a.A, 1024), dim3(256), 0, s, a, counts, (const uint32_t*)nullptr, 0u,
+                       (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr);
+    GS355_CHECK_LAUNCH("decode: count");
+    // the scan writes every block sum before it reads it: nothing in the array has to start at zero
+    return launch_exclusive_scan(counts, offsets, (size_t)a.A, tmp, s);
 }
 
 int gs355_decode_emit(const gs355_decoder* dec, const gs355_anchors* an, const uint32_t* offsets, int64_t capacity,

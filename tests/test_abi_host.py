@@ -291,3 +291,17 @@ def test_header_is_plain_c(tmp_path):
     want = [C.sizeof(t) for t in (_lib.Header, _lib.Frame, _lib.Gaussians, _lib.Outputs, _lib.Layout, _lib.AnchorLod,
                                   _lib.Decoder, _lib.Anchors, _lib.Decoded)]
     assert [int(v) for v in out] == want
+
+
+def test_static_count_rejects_more_anchors_than_its_array_covers():
+    lib = _lib.load()
+    d = _lib.Decoder()
+    d.feat_dim, d.n_offsets = 32, 10
+    for j in range(3):
+        d.in_dim[j] = 36
+        d.w0[j] = d.b0[j] = d.w1[j] = d.b1[j] = 0x1000
+    an = _lib.Anchors()
+    an.A = (1 << 24) + 1
+    an.anchor = an.feat = an.offset = an.scaling = an.visible_mask = an.campos = 0x1000
+    rc = lib.gs355_decode_count_static(C.byref(d), C.byref(an), 0x1000, 0x1000, None)  # rejected before any HIP call
+    assert rc == _lib.GS355_ENOSPC and b"at most" in lib.gs355_last_error()

@@ -33,10 +33,12 @@ def mlp(h, params):
 
 
 def decode(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, mlps, n_offsets=10,
-           add_dist=(True, True, True)):
+           add_dist=(True, True, True), keep_override=None):
     """mlps: {"opacity"|"cov"|"color": (W0[32,in], b0[32], W1[k,32], b1[k])}.
     Returns xyz[G,3], color[G,3], opacity[G,1], scaling[G,3], rot[G,4] and the
-    flat keep mask over (visible anchor, offset)."""
+    flat keep mask over (visible anchor, offset).  `keep_override` (flat bool
+    over (visible anchor, offset)) replaces the mask opacity > 0: tests use it
+    to obtain the values of offsets whose opacity is within rounding of zero."""
     if visible_mask is None:
         visible_mask = torch.ones(anchor.shape[0], dtype=torch.bool)
     a = anchor[visible_mask].float()
@@ -52,7 +54,7 @@ def decode(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, ml
     for head, use_dist in zip(HEADS, add_dist):
         outs[head] = mlp(with_dist if use_dist else without, mlps[head])
     neural_opacity = torch.tanh(outs["opacity"]).reshape(-1, 1)
-    keep = (neural_opacity > 0.0).view(-1)
+    keep = (neural_opacity > 0.0).view(-1) if keep_override is None else keep_override.view(-1).bool()
     color = torch.sigmoid(outs["color"]).reshape(-1, 3)[keep]
     cov = outs["cov"].reshape(-1, 7)[keep]
     rep = torch.arange(a.shape[0]).repeat_interleave(n_offsets)[keep]

@@ -372,10 +372,13 @@ void orc_tile_ranges(uint64_t n, const uint64_t *keys, int tiles, uint32_t *rang
 }
 
 /* Front-to-back alpha blending.  out_rgb [3,H,W], out_depth [H,W], out_alpha
- * [H,W].  `fragile` (optional, [H,W]) is set to 1 for pixels where some
- * discrete decision (power>0, alpha<1/255, T(1-alpha)<1e-4) was taken within
- * rounding distance of its threshold, so that a second implementation with a
- * different exp() or multiply-add fusion may legitimately decide otherwise.
+ * [H,W].  `fragile` (optional, [H,W]) counts, per pixel (saturating at 255), the
+ * discrete decisions (power>0, alpha<1/255, T(1-alpha)<1e-4) that were taken
+ * within rounding distance of their threshold, so that a second implementation
+ * with a different exp() or multiply-add fusion may legitimately decide
+ * otherwise.  0 = every decision of the pixel is safe; each counted decision can
+ * move the pixel by at most one contribution of weight 1/255 (or the 1e-4
+ * remainder of a finished pixel).
  * stats (optional): [0]=evaluated (pixel,Gaussian) pairs, [1]=accepted pairs,
  * [2]=sum over tiles of 256 * (range entries consumed before every pixel of
  * the tile was finished). */
@@ -407,13 +410,13 @@ void orc_blend(const orc_frame *f, const uint32_t *ranges, const uint32_t *value
                         float t1 = co[0] * dx * dx, t2 = co[2] * dy * dy, t3 = co[1] * dx * dy;
                         float power = -0.5f * (t1 + t2) - t3;
                         ++evaluated;
-                        if (fabsf(power) <= 1e-5f * (fabsf(t1) + fabsf(t2) + fabsf(t3))) frag = 1;
+                        if (fabsf(power) <= 1e-5f * (fabsf(t1) + fabsf(t2) + fabsf(t3))) ++frag;
                         if (power > 0.f) continue;
                         float alpha = fminf(0.99f, co[3] * expf(power));
-                        if (fabsf(alpha - 1.0f / 255.0f) < 1e-4f * (1.0f / 255.0f)) frag = 1;
+                        if (fabsf(alpha - 1.0f / 255.0f) < 1e-4f * (1.0f / 255.0f)) ++frag;
                         if (alpha < 1.0f / 255.0f) continue;
                         float test_T = T * (1.f - alpha);
-                        if (fabsf(test_T - 0.0001f) < 1e-4f * 0.0001f) frag = 1;
+                        if (fabsf(test_T - 0.0001f) < 1e-4f * 0.0001f) ++frag;
                         if (test_T < 0.0001f) break;
                         ++accepted;
                         C0 += rgb[3 * (size_t)gi] * alpha * T;
@@ -428,7 +431,7 @@ void orc_blend(const orc_frame *f, const uint32_t *ranges, const uint32_t *value
                     out_rgb[2 * (size_t)H * W + o] = C2 + T * f->bg[2];
                     if (out_depth) out_depth[o] = D;
                     if (out_alpha) out_alpha[o] = 1.f - T;
-                    if (fragile) fragile[o] = (uint8_t)frag;
+                    if (fragile) fragile[o] = (uint8_t)(frag > 255 ? 255 : frag);
                     uint32_t used = (j < hi ? j + 1 : hi) - lo;
                     if (used > deepest) deepest = used;
                 }

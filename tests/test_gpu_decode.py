@@ -24,16 +24,38 @@ def build_decoder(sc, device, add_dist=(True, True, True)):
     return dec.to(device).eval()
 
 
-def compare(got, ref, A_vis):
+UNSURE = 1e-5  # |opacity| below this: the matrix cores and the CPU GEMM may put the offset on either side of the mask
+
+
+def compare(got, ref, redo):
+    """GPU outputs against the oracle's.  Offsets whose decoded opacity is within UNSURE of zero may legitimately fall
+    on either side of the mask `opacity > 0`; every other offset must be present, in order, within TOL.  `redo(keep)`
+    re-runs the oracle with a given keep mask (to obtain its values for the doubtful offsets the GPU kept)."""
     xyz, color, opacity, scaling, rot, x5, x6 = got
     assert x5 is None and x6 is None
-    # opacities within rounding of zero may legitimately fall on either side of the mask
     raw = ref["raw_opacity"].numpy()
-    unsure = int((np.abs(raw) < 1e-5).sum())
-    G = ref["xyz"].shape[0]
-    assert abs(xyz.shape[0] - G) <= unsure
-    if xyz.shape[0] != G:
-        pytest.skip("mask differs on an opacity within 1e-5 of zero")
+    sure, unsure = raw > UNSURE, np.abs(raw) <= UNSURE
+    G = int(xyz.shape[0])
+    assert int(sure.sum()) <= G <= int(sure.sum() + unsure.sum())
+    if unsure.any():
+        # decide, doubtful offset by doubtful offset, whether the GPU kept it: at the slot it would occupy the GPU's
+        # position must be the oracle's position of that offset and its opacity must be tiny
+        wide = redo(torch.from_numpy(sure | unsure))
+        wide_index = np.flatnonzero(sure | unsure)
+        slot_in_wide = {int(i): k for k, i in enumerate(wide_index)}
+        gx, go = xyz.cpu().numpy(), opacity.cpu().numpy().reshape(-1)
+        keep = sure.copy()
+        kept_before = np.cumsum(sure) - sure  # sure offsets before each flat index
+        extra = 0
+        for i in np.flatnonzero(unsure):
+            slot = int(kept_before[i]) + extra
+            w = wide["xyz"][slot_in_wide[int(i)]].numpy()
+            if slot < G and abs(go[slot]) <= 4 * UNSURE and np.abs(gx[slot] - w).max() <= TOL * max(1.0, np.abs(w).max()):
+                keep[i] = True
+                extra += 1
+        ref = redo(torch.from_numpy(keep))
+        print("decode: %d offsets within %g of the mask threshold, %d kept by the GPU" % (int(unsure.sum()), UNSURE, extra))
+    assert G == ref["xyz"].shape[0]
     for name, t in (("xyz", xyz), ("color", color), ("opacity", opacity), ("scaling", scaling), ("rot", rot)):
         want = ref[name].numpy()
         assert t.shape == want.shape, name
@@ -42,7 +64,8 @@ def compare(got, ref, A_vis):
         assert err / scale <= TOL, "%s: max-abs %g (scale %g)" % (name, err, scale)
 
 
-@pytest.mark.parametrize("A,frac", [(5000, 0.5), (33, 1.0), (1, 1.0), (4097, 0.1), (100_000, 0.35)])
+@pytest.mark.parametrize("A,frac", [(5000, 0.5), (33, 1.0), (1, 1.0), (4097, 0.1), (100_000, 0.35), (500_000, 0.45),
+                                    (500_000, 1.0)])
 def test_decode_matches_oracle(gpu_device, A, frac):
     sc = scenes.config5(A=A)
     g = torch.Generator().manual_seed(A)
@@ -54,8 +77,9 @@ def test_decode_matches_oracle(gpu_device, A, frac):
     got = dec(camera_center=cam.to(gpu_device), anchor=sc.anchor.to(gpu_device),
               anchor_feat=sc.anchor_feat.to(gpu_device), offset=sc.offset.to(gpu_device),
               scaling=sc.scaling.to(gpu_device), visible_mask=vis.to(gpu_device))
-    ref = ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp, sc.n_offsets)
-    compare(got, ref, int(vis.sum()))
+    redo = lambda keep=None: ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp,  # noqa: E731
+                                       sc.n_offsets, keep_override=keep)
+    compare(got, redo(), redo)
 
 
 def test_decode_heads_without_distance_and_fewer_offsets(gpu_device):
@@ -70,9 +94,9 @@ def test_decode_heads_without_distance_and_fewer_offsets(gpu_device):
     cam = sc.camera.camera_center
     got = dec(cam.to(gpu_device), sc.anchor.to(gpu_device), sc.anchor_feat.to(gpu_device), sc.offset.to(gpu_device),
               sc.scaling.to(gpu_device), vis.to(gpu_device))
-    ref = ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp, 6,
-                    add_dist=(True, True, False))
-    compare(got, ref, int(vis.sum()))
+    redo = lambda keep=None: ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp, 6,  # noqa: E731
+                                       add_dist=(True, True, False), keep_override=keep)
+    compare(got, redo(), redo)
 
 
 def test_decode_nothing_visible_and_default_mask(gpu_device):
@@ -84,8 +108,9 @@ def test_decode_nothing_visible_and_default_mask(gpu_device):
     out = dec(cam, *args, torch.zeros(700, dtype=torch.bool, device=gpu_device))
     assert out[0].shape == (0, 3) and out[4].shape == (0, 4)
     out = dec(cam, *args, None)  # visible_mask=None means every anchor
-    ref = ao.decode(sc.camera.camera_center, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, None, sc.mlp, 10)
-    compare(out, ref, 700)
+    redo = lambda keep=None: ao.decode(sc.camera.camera_center, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling,  # noqa: E731
+                                       None, sc.mlp, 10, keep_override=keep)
+    compare(out, redo(), redo)
 
 
 def test_unsupported_configurations_are_refused():

@@ -2,6 +2,7 @@
 (tests/test_inference_framework/test_inference.py:255-285, tests/utils.py:172-201) —
 `engine = init_inference(ModelClass, InferModuleOrNone, model_config, inference_config)` then
 `engine(viewpoint_cam, 1.0, None, None)` — against the same model built directly from tensors."""
+import numpy as np
 import pytest
 import torch
 
@@ -9,6 +10,8 @@ from landmarksystem_amd import checkpoints as ck
 from landmarksystem_amd import scenes
 from landmarksystem_amd.engine import InferenceModule, init_inference
 from landmarksystem_amd.models import GaussianModel, OctreeGS, ScaffoldGS
+
+from tests.helpers import check_anchor_model_frame, check_images, vanilla_model_reference
 
 pytestmark = pytest.mark.gpu
 
@@ -40,6 +43,9 @@ def test_engine_renders_checkpoints_like_the_direct_models(gpu_device, tmp_path)
     assert out.shape == (3, 270, 480) and not out.requires_grad
     assert torch.equal(out, vanilla(scene.camera))
     assert "scaling" in engine.base_model._cache  # act_cache from the model config
+    ref = vanilla_model_reference(engine.base_model, scene.camera)  # the engine's tensors through the oracle
+    check_images(dict(image=out.cpu().numpy()), ref, "engine, vanilla checkpoint")
+    np.testing.assert_array_equal(engine.base_model.visibility_filter.cpu().numpy(), ref["radii"] > 0)
 
     anchors = scenes.config5(A=20_000, width=480, height=270)
     scaffold = ScaffoldGS.from_scene(anchors).to(gpu_device).eval()
@@ -47,7 +53,9 @@ def test_engine_renders_checkpoints_like_the_direct_models(gpu_device, tmp_path)
     engine = init_inference(ScaffoldGS, None, dict(ckpt=str(tmp_path / "s" / "point_cloud.ply"), n_offsets=10,
                                                    feat_dim=32, add_opacity_dist=True, add_cov_dist=True,
                                                    add_color_dist=True), dict(runtime="Torch"))
-    assert torch.equal(engine(anchors.camera, 1.0, None, None), scaffold(anchors.camera))
+    out = engine(anchors.camera, 1.0, None, None)
+    assert torch.equal(out, scaffold(anchors.camera))
+    check_anchor_model_frame(engine.base_model, anchors.camera, out, "engine, Scaffold-GS checkpoint")
 
     level = torch.randint(0, 5, (20_000,), generator=torch.Generator().manual_seed(5))
     octree = OctreeGS(anchors.anchor, anchors.anchor_feat, anchors.offset, torch.log(anchors.scaling),
@@ -59,7 +67,9 @@ def test_engine_renders_checkpoints_like_the_direct_models(gpu_device, tmp_path)
                   appearance_dim=0, add_opacity_dist=True, add_cov_dist=True, add_color_dist=True, enable_lod=True)
     engine = init_inference(OctreeGS, InferenceOctreeGSModule, config, dict(runtime="Kernel"))
     assert engine.base_model.voxel_size == 0.5 and engine.base_model.standard_dist == 250.0
-    assert torch.equal(engine(anchors.camera, 1.0, None, None), octree(anchors.camera))
+    out = engine(anchors.camera, 1.0, None, None)
+    assert torch.equal(out, octree(anchors.camera))
+    check_anchor_model_frame(engine.base_model, anchors.camera, out, "engine, Octree-GS checkpoint")
 
 
 def test_render_trajectory_equals_frame_by_frame(gpu_device):

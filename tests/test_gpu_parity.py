@@ -12,12 +12,9 @@ import torch
 
 from landmarksystem_amd import _lib, pipeline, scenes
 from oracle import c_oracle as co
-from tests.helpers import oracle_frame, oracle_gaussians, psnr, settings_for, u32, u64
+from tests.helpers import IMG_TOL, check_images, oracle_frame, oracle_gaussians, settings_for, u32, u64
 
 pytestmark = pytest.mark.gpu
-
-IMG_TOL = 1e-4
-PSNR_MIN = 60.0
 
 
 def run_all_stages(scene, device, colors_precomp=None, cov3D_precomp=None, cam=None, n_cap=None, sh_degree=None):
@@ -100,20 +97,8 @@ def check_against_oracle(got, ref, label=""):
     np.testing.assert_array_equal(got["sorted_keys"], ref["sorted_keys"], err_msg=label + " sorted keys")
     np.testing.assert_array_equal(got["sorted_values"], ref["sorted_values"], err_msg=label + " sorted values")
     np.testing.assert_array_equal(got["ranges"], ref["ranges"], err_msg=label + " ranges")
-    # --- images: tolerance ----------------------------------------------------
-    solid = ref["fragile"] == 0
-    frac_fragile = 1.0 - solid.mean()
-    assert frac_fragile < 0.02, "too many threshold-adjacent pixels: %g" % frac_fragile
-    for name, g, r in (("image", got["image"], ref["image"]), ("depth", got["depth"], ref["depth"]),
-                       ("alpha", got["alpha"], ref["alpha"])):
-        diff = np.abs(g - r)
-        scale = 1.0
-        if name == "depth":  # depth accumulates z * w: tolerance relative to the scene's depth scale
-            scale = max(1.0, float(np.abs(r).max()))
-        err = float((diff[..., solid]).max()) / scale if solid.any() else 0.0
-        assert err <= IMG_TOL, "%s %s max-abs %g (scale %g)" % (label, name, err, scale)
-        p = psnr(g / scale, r / scale)
-        assert p >= PSNR_MIN, "%s %s PSNR %g" % (label, name, p)
+    # --- images: tolerance (safe pixels 1e-4, every pixel bounded by its near-threshold decisions, PSNR) ------
+    check_images(got, ref, label)
 
 
 def oracle_render(scene, **kw):
@@ -203,8 +188,8 @@ def test_key_capacity_overflow_is_reported_and_recovered(gpu_device):
     ref = oracle_render(scene)
     assert ws.overflows == 1 and out.num_keys == ref["num_keys"]
     assert ws.key_capacity >= ref["num_keys"]
-    solid = ref["fragile"] == 0
-    assert np.abs(out.image.cpu().numpy() - ref["image"])[:, solid].max() <= IMG_TOL
+    check_images(dict(image=out.image.cpu().numpy(), depth=out.depth.cpu().numpy(), alpha=out.alpha.cpu().numpy()),
+                 ref, "overflow redo")
 
 
 def test_rerun_is_bit_identical(gpu_device):
@@ -290,10 +275,8 @@ def test_tile_bucketed_path_equals_oracle(gpu_device, make, label):
     np.testing.assert_array_equal(got["ranges"], ref["ranges"], err_msg=label + " ranges")
     np.testing.assert_array_equal(got["sorted_keys"], ref["sorted_keys"], err_msg=label + " sorted keys")
     np.testing.assert_array_equal(got["sorted_values"], ref["sorted_values"], err_msg=label + " sorted values")
-    solid = ref["fragile"] == 0
-    assert np.abs(got["image"] - ref["image"])[:, solid].max() <= IMG_TOL
-    assert np.abs(got["alpha"] - ref["alpha"])[solid].max() <= IMG_TOL
-    assert psnr(got["image"], ref["image"]) >= PSNR_MIN
+    # the crowded scenes are made of faint Gaussians (opacity 0.004 .. 0.024 around the 1/255 threshold)
+    check_images(got, ref, label, max_fragile_frac=0.5 if "ties" in label else 0.02)
     if "ties" in label:
         k = got["sorted_keys"]
         assert (k[1:] == k[:-1]).any()
@@ -325,9 +308,7 @@ def test_config4_scaled_down_4k_trajectory(gpu_device):
         np.testing.assert_array_equal(got["ranges"], ref["ranges"])
         np.testing.assert_array_equal(got["sorted_keys"], ref["sorted_keys"])
         np.testing.assert_array_equal(got["sorted_values"], ref["sorted_values"])
-        solid = ref["fragile"] == 0
-        assert np.abs(got["image"] - ref["image"])[:, solid].max() <= IMG_TOL
-        assert psnr(got["image"], ref["image"]) >= PSNR_MIN
+        check_images(got, ref, "C4/1.5M pose %d" % k)
 
 
 def test_full_size_headline_frame_properties(gpu_device):
@@ -363,11 +344,50 @@ def test_full_size_headline_frame_equals_the_oracle(gpu_device):
     assert got["num_keys"] == ref["num_keys"] > 10_000_000
     for name in ("radii", "ranges", "sorted_keys", "sorted_values"):
         np.testing.assert_array_equal(got[name], ref[name], err_msg=name)
-    solid = ref["fragile"] == 0
-    assert solid.mean() > 0.98
-    assert np.abs(got["image"] - ref["image"])[:, solid].max() <= IMG_TOL
-    assert psnr(got["image"], ref["image"]) >= PSNR_MIN
-    assert np.abs(got["alpha"] - ref["alpha"])[solid].max() <= IMG_TOL
+    check_images(got, ref, "C3 full size")
+
+
+def check_fast_path_against_oracle(scene, device, label):
+    """One frame through the shipped stage sequence against the oracle: radii, every sorted key and value and the
+    ranges bit for bit, image / depth / alpha to the frame bars."""
+    got = run_fast_path(scene, device)
+    ref = oracle_render(scene)
+    assert got["num_keys"] == ref["num_keys"] > 0
+    for name in ("radii", "ranges", "sorted_keys", "sorted_values"):
+        np.testing.assert_array_equal(got[name], ref[name], err_msg=label + " " + name)
+    check_images(got, ref, label)
+    return got, ref
+
+
+def test_full_size_config2_equals_the_oracle(gpu_device):
+    """1M Gaussians around the origin at 1080p (dense centre: the largest tile buckets of the five workloads)."""
+    scene = scenes.config2()
+    got, ref = check_fast_path_against_oracle(scene, gpu_device, "C2 full size")
+    assert scene.P == 1_000_000 and got["num_keys"] > 1_000_000
+    classic = run_all_stages(scene, gpu_device)
+    check_against_oracle(classic, ref, "C2 full size, classic stages")
+    for name in ("sorted_keys", "sorted_values", "ranges", "image", "depth", "alpha"):
+        np.testing.assert_array_equal(classic[name], got[name], err_msg=name)
+
+
+@pytest.fixture(scope="module")
+def config4_scene():
+    print("generating the 20M-Gaussian scene ...", flush=True)
+    return scenes.config4()
+
+
+@pytest.mark.parametrize("pose", [0, 17])
+def test_full_size_config4_4k_frame_equals_the_oracle(gpu_device, config4_scene, pose):
+    """20M Gaussians at 3840x2160 (32,400 tiles; a workspace of about 2 GB) for poses of the trajectory."""
+    scene = config4_scene
+    assert scene.P == 20_000_000 and len(scene.cameras) == 30
+    one = scenes.GaussianScene(scene.name, scene.means3D, scene.scales, scene.rotations, scene.opacities,
+                               scene.shs, scene.sh_degree, [scene.cameras[pose]], scene.bg)
+    print("C4 pose %d" % pose, flush=True)
+    got, ref = check_fast_path_against_oracle(one, gpu_device, "C4 full size pose %d" % pose)
+    frac = (ref["radii"] > 0).mean()
+    assert 0.15 < frac < 0.7, frac
+    assert got["num_keys"] > 10_000_000
 
 
 @pytest.mark.parametrize("same,spread,label", [(1800, 0, "one depth only"), (1500, 2500, "one heavy depth among many"),
@@ -442,9 +462,8 @@ def test_images_beyond_the_tile_bucket_limit(gpu_device):
     ref = co.render(oracle_frame(scene), oracle_gaussians(scene))
     assert got.num_keys == ref["num_keys"]
     np.testing.assert_array_equal(got.radii.cpu().numpy(), ref["radii"])
-    solid = ref["fragile"] == 0
-    image = got.image.cpu().numpy()
-    assert np.abs(image - ref["image"])[:, solid].max() <= 1e-4 and psnr(image, ref["image"]) >= 60.0
+    check_images(dict(image=got.image.cpu().numpy(), depth=got.depth.cpu().numpy(), alpha=got.alpha.cpu().numpy()),
+                 ref, "beyond the bucket limit")
 
 
 def test_non_finite_and_degenerate_inputs(gpu_device):

@@ -5,11 +5,17 @@ on one MI355X (synthetic city-block scene, SH degree 3, RGB + depth + alpha).
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--gaussians P]
 
 A step is one full frame through GaussianRasterizer.forward (the product path:
-preprocess -> scan -> duplicate -> sort -> ranges -> blend) with every input
-already resident in HBM.  Prints ONE JSON line with the frame rate, a
+preprocess -> tile count -> tile scatter -> per-tile sort -> blend) with every
+input already resident in HBM.  Prints ONE JSON line with the frame rate, a
 per-stage breakdown timed with HIP events on the launch stream, the roofline
-figure of the dominant stage and a CPU baseline (the PyTorch-CPU rasterizer of
-the same semantics on the host cores, on a bounded sample of the workload).
+figure of the dominant stage and a CPU baseline measured in the same run on
+the host cores: the PyTorch-CPU rasterizer of the same semantics on a bounded
+sample of the workload, and the C checker over the whole frame, which also
+counts the (pixel, Gaussian) pairs the blend's algorithmic flops are defined by.
+
+--config 4 (20M Gaussians, 3840x2160, 30 poses) and --config 5 (Scaffold-GS,
+500k anchors decoded on the matrix cores, then rasterized) print lines of the
+same structure for those workloads.
 """
 import argparse
 import json
@@ -22,20 +28,24 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
-
-# HBM bytes per launch of the heaviest kernels on the default workload (6M Gaussians, 1080p), from two
-# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what
-# the same counter reads for the 1 GiB copy of --calibration-copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
-# "keys_sort_ranges" is the sum over the kernels of the tile count, scatter and tile sort stages.
-MEASURED_TRAFFIC_BYTES = {"blend": 1849.2e6, "preprocess": 1701.9e6, "keys_sort_ranges": 838.8e6}
-# (pixel, Gaussian) pairs of the default workload's blend, counted by the CPU checker (`python -m oracle.workload_stats 3`):
-# every list entry a pixel visits before it terminates / the pairs applied to a pixel (alpha >= 1/255).  Properties
-# of the seeded scene, not of a kernel; 25 flop per evaluated pair is the blend's algorithmic work.
-BLEND_PAIRS = {"evaluated": 1.612e9, "accepted": 1.001e8}
-# fp32 flops the blend kernel issues per launch on that workload (64 x (2 FMA + MUL + ADD) from a `rocprofv3 --pmc` run)
-BLEND_ISSUED_FLOPS = 11.12e9
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3  # MI355X fp32 vector peak (packed FMA); this build issues unpacked FP32 only
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+# HBM bytes per launch of the stages of the default workload (6M Gaussians, 1080p), read from hardware counters in
+# separate profiler runs of this script, NOT measured by the run that prints them: two `rocprofv3 --pmc` runs
+# (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads for the 1 GiB copy of
+# --calibration-copy.  The bench line names the file they were read from; tests/test_bench_constants.py holds these
+# numbers to that file.  "keys_sort_ranges" is the sum over the kernels of the tile count, scatter and sort stages.
+COUNTER_TRAFFIC = {
+    "source": "profiles/bench_c3_6M_1080p_hbm_traffic.txt",
+    "workload": "configs[2]",
+    "bytes": {"blend": 1849.4e6, "preprocess": 1701.8e6, "keys_sort_ranges": 844.7e6},
+    # fp32 flops the blend kernel issues per launch (64 lanes x (2 FMA + MUL + ADD) wavefront instructions), from
+    # profiles/bench_c3_6M_1080p_valu_counters.txt
+    "blend_issued_flops": 11.12e9,
+    "blend_issued_flops_source": "profiles/bench_c3_6M_1080p_valu_counters.txt",
+}
 
 
 def parse_args():
@@ -44,9 +54,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=3, choices=[1, 2, 3, 4, 5],
-                    help="3 = the headline workload; 4 (20M Gaussians, 4K, 30 poses) and 5 (Scaffold-GS, 500k anchors) "
-                         "print a reduced line")
-    ap.add_argument("--gaussians", type=int, default=None, help="override the Gaussian count (not the headline workload)")
+                    help="3 = the headline workload; 4 = 20M Gaussians, 4K, 30 poses; 5 = Scaffold-GS, 500k anchors")
+    ap.add_argument("--gaussians", type=int, default=None, help="override the Gaussian / anchor count (not the named workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--stage-steps", type=int, default=20)
     ap.add_argument("--calibration-copy", action="store_true",
@@ -61,17 +70,21 @@ def parse_args():
     return ap.parse_args()
 
 
-def settings_for(scene, device):
+def settings_for(scene, device, cam=None, sh_degree=None):
     from landmarksystem_amd import GaussianRasterizationSettings
 
-    cam = scene.camera.to(device)
+    cam = (cam or scene.camera).to(device)
     return GaussianRasterizationSettings(
         image_height=cam.height, image_width=cam.width, tanfovx=math.tan(cam.FovX * 0.5),
         tanfovy=math.tan(cam.FovY * 0.5), bg=scene.bg.to(device), scale_modifier=1.0,
-        viewmatrix=cam.world_view_transform, projmatrix=cam.full_proj_transform, sh_degree=scene.sh_degree,
+        viewmatrix=cam.world_view_transform, projmatrix=cam.full_proj_transform,
+        sh_degree=scene.sh_degree if sh_degree is None else sh_degree,
         campos=cam.camera_center, prefiltered=False, debug=False,
     )
 
+
+# ----------------------------------------------------------------------------------------------------------------
+# GPU side: stage timings and algorithmic work of one rasterizer frame
 
 def time_stages(torch, pipeline, inp, out, ws, n_cap, stages, steps):
     for _, m in stages:  # warm
@@ -91,8 +104,8 @@ def time_stages(torch, pipeline, inp, out, ws, n_cap, stages, steps):
 
 
 def stage_breakdown(torch, pipeline, _lib, inp, n_cap, steps):
-    """Average milliseconds per stage, HIP events on the launch stream: the
-    shipped pipeline (tile-bucketed sort) and, beside it, the classic
+    """Average milliseconds per stage, HIP events on the launch stream (torch's current stream, the one every
+    kernel of the library is enqueued on): the shipped pipeline (tile-bucketed sort) and, beside it, the classic
     duplicate / LSD radix sort / ranges stages it replaces."""
     ws = pipeline.Workspace(inp.device)
     out = pipeline.FrameOutputs(inp)
@@ -110,9 +123,10 @@ def stage_breakdown(torch, pipeline, _lib, inp, n_cap, steps):
     return ms, stats
 
 
-def algorithmic_work(P, V, N, tiles, npix, sh_coeffs, passes, blend_pairs):
-    """Algorithmic bytes / flops per frame and stage."""
-    b_in = 12 + 12 + 16 + 4 + 12 * sh_coeffs  # mean, scale, quat, opacity, SH
+def algorithmic_work(P, V, N, tiles, npix, colour_bytes, passes):
+    """Algorithmic bytes per frame and stage.  `colour_bytes`: bytes of colour input per Gaussian (12 x SH
+    coefficients, or 12 for precomputed colours)."""
+    b_in = 12 + 12 + 16 + 4 + colour_bytes  # mean, scale, quat, opacity, colour input
     return {
         "preprocess": 12 * P + 8 * P + V * (b_in - 12) + V * 40,
         "scan": 8 * P,
@@ -120,140 +134,216 @@ def algorithmic_work(P, V, N, tiles, npix, sh_coeffs, passes, blend_pairs):
         "sort": N * (8 + passes * 24),
         "ranges": 8 * N + 8 * tiles,
         "blend_bytes": 40 * N + 20 * npix,
-        "blend_flops": 25 * blend_pairs,
     }
 
 
-def bench_trajectory(args, torch, dev):
-    """configs[3]: large slab at 4K over a trajectory of aerial poses."""
-    from landmarksystem_amd import GaussianRasterizer, scenes
+def raster_report(stage_ms, stats, P, tiles, npix, colour_bytes, pairs, counters):
+    """The `stages` object and the roofline of the dominant stage for one rasterizer frame.
 
-    scene = scenes.config4(args.gaussians) if args.gaussians else scenes.config4()
-    d = scene.to(dev)
-    rast = GaussianRasterizer(settings_for(scene, dev))
-    base = rast.raster_settings
-    poses = [base._replace(viewmatrix=c.world_view_transform, projmatrix=c.full_proj_transform,
-                           campos=c.camera_center) for c in d.cameras]
-    kwargs = dict(means3D=d.means3D, means2D=None, shs=d.shs, colors_precomp=None, opacities=d.opacities,
-                  scales=d.scales, rotations=d.rotations, cov3D_precomp=None)
-    keys, visible = [], []
+    pairs:    {"evaluated", "accepted", "tile_work"} counted by the C checker in this run, or None (then the blend
+              is priced with the kernel-independent upper bound 256 x sum of tile range lengths, labelled as such).
+    counters: COUNTER_TRAFFIC when it applies to this workload, else None."""
+    V, N = stats["num_visible"], stats["num_keys"]
+    work = algorithmic_work(P, V, N, tiles, npix, colour_bytes, stats["sort_passes"])
+    cbytes = counters["bytes"] if counters else {}
+
+    def hbm(ms, nbytes, counter_bytes=None):
+        d = {"ms": round(ms, 4), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
+             "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        if counter_bytes:
+            d.update({"counter_bytes": counter_bytes, "counter_GBps": round(counter_bytes / ms / 1e6, 1),
+                      "frac_hbm_counter": round(counter_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)})
+        return d
+
+    stages = {"preprocess": hbm(stage_ms["preprocess"], work["preprocess"], cbytes.get("preprocess"))}
+    # key generation + sort + ranges.  "bytes" is the algorithmic figure of the stages this path replaces (scan,
+    # duplicate, 8-bit LSD radix sort, ranges): an equivalent-work number, not traffic of the shipped kernels, which
+    # never run those passes.  counter_bytes / frac_hbm_counter (where present) are what the kernels really moved.
+    sort_bytes = work["scan"] + work["duplicate"] + work["sort"] + work["ranges"]
+    sort_ms = stage_ms["tile_count"] + stage_ms["tile_scatter"] + stage_ms["tile_sort"]
+    for name in ("tile_count", "tile_scatter", "tile_sort"):
+        stages[name] = {"ms": round(stage_ms[name], 4)}
+    stages["keys_sort_ranges"] = hbm(sort_ms, sort_bytes, cbytes.get("keys_sort_ranges"))
+    stages["keys_sort_ranges"]["accounting"] = ("bytes = scan + duplicate + LSD radix sort (%d passes of 24 B/key) + ranges"
+                                                " that the tile-bucketed stages replace; floor_bytes = 24 B/key"
+                                                % stats["sort_passes"])
+    stages["keys_sort_ranges"]["floor_bytes"] = 24 * N
+    stages["keys_sort_ranges"]["frac_hbm_floor"] = round(24 * N / sort_ms / 1e6 / HBM_PEAK_GBS, 4) if N else 0.0
+    stages["classic_lsd_path"] = {"scan_ms": round(stage_ms["scan"], 4), "duplicate_ms": round(stage_ms["duplicate"], 4),
+                                  "sort_ms": round(stage_ms["sort"], 4), "ranges_ms": round(stage_ms["ranges"], 4),
+                                  "sort_GBps": round(work["sort"] / stage_ms["sort"] / 1e6, 1),
+                                  "sort_frac_hbm": round(work["sort"] / stage_ms["sort"] / 1e6 / HBM_PEAK_GBS, 4)}
+    ms = stage_ms["blend"]
+    upper = 25 * 256 * stats["range_sum"]
+    blend = {"ms": round(ms, 4), "flops_upper": upper, "TFLOPs_upper": round(upper / ms / 1e9, 2),
+             "frac_fp32_upper": round(upper / ms / 1e9 / FP32_PEAK_TFLOPS, 4)}
+    if pairs:
+        flops = 25 * pairs["evaluated"]
+        blend.update({
+            "pairs_evaluated": pairs["evaluated"], "pairs_accepted": pairs["accepted"], "tile_work": pairs["tile_work"],
+            "pairs_source": "C checker (oracle/gs_oracle.c) over the whole frame, in this run",
+            "flops_algorithmic": flops, "TFLOPs_algorithmic": round(flops / ms / 1e9, 2),
+            "frac_fp32_algorithmic": round(flops / ms / 1e9 / FP32_PEAK_TFLOPS, 4),
+            "TFLOPs_tile_work": round(25 * pairs["tile_work"] / ms / 1e9, 2),
+            "accepted_pairs_per_s": round(pairs["accepted"] / ms * 1e3)})
+    if counters:
+        blend.update({"TFLOPs_issued": round(counters["blend_issued_flops"] / ms / 1e9, 2),
+                      "frac_fp32_issued": round(counters["blend_issued_flops"] / ms / 1e9 / FP32_PEAK_TFLOPS, 4),
+                      "issued_flops_source": counters["blend_issued_flops_source"]})
+    stages["blend"] = blend
+    pre_sort_ms = stage_ms["preprocess"] + sort_ms
+    counter_sum = cbytes.get("preprocess", 0) + cbytes.get("keys_sort_ranges", 0) if counters else None
+    stages["preprocess_plus_sort"] = hbm(pre_sort_ms, work["preprocess"] + sort_bytes, counter_sum)
+    stages["rates"] = {"gaussians_per_s_preprocess": round(P / stage_ms["preprocess"] * 1e3),
+                       "sorted_keys_per_s": round(N / sort_ms * 1e3) if N else 0,
+                       "blend_frames_per_s": round(1e3 / stage_ms["blend"], 1)}
+
+    shipped = {"preprocess": stage_ms["preprocess"], "keys_sort_ranges": sort_ms, "blend": stage_ms["blend"]}
+    dominant = max(shipped, key=lambda n: shipped[n])
+    traffic = {"bytes": cbytes[dominant], "source": counters["source"],
+               "note": "from earlier profiler runs of this workload, not measured by this run"} \
+        if counters and dominant in cbytes else None
+    if dominant == "blend":
+        kind = "algorithmic" if pairs else "upper"
+        roofline = {"bound": "valu", "kernel": "blend_kernel", "achieved": blend["TFLOPs_" + kind],
+                    "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": blend["frac_fp32_" + kind], "traffic": traffic,
+                    "note": "FP32 vector-ALU kernel (no matrix cores); peak is the MI355X fp32 vector figure (packed FMA; "
+                            "this build issues unpacked fp32, half of it).  flops = 25 x the (pixel, Gaussian) pairs the "
+                            "per-pixel loop evaluates" + (
+                                ", counted by the C checker in this run; the kernel skips pairs whose alpha is provably "
+                                "< 1/255, so it issues fewer flops than that" if pairs else
+                                ", bounded above by 256 x the sum of the tile range lengths")}
+    else:
+        roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": traffic}
+    return stages, roofline
+
+
+def backward_report(torch, pipeline, inp, n_cap, N, V, P, sh_coeffs, ms_per_step, stage_steps):
+    """Backward pass of the same frame (the training loop's loss.backward() on an image loss): all gradients of a
+    forward render, reported beside the forward stages, never part of `value`."""
+    dev = inp.device
+    ws_b = pipeline.Workspace(dev)
+    ws_b.key_capacity = n_cap
+    out_b = pipeline.render(inp, ws=ws_b)
+    g_image = torch.randn(3, inp.height, inp.width, device=dev)
+    t_bwd = {}
+    for label, want in (("all_gradients", pipeline.GRAD_NAMES),
+                        ("without_sh_gradient", tuple(n for n in pipeline.GRAD_NAMES if n != "shs"))):
+        for _ in range(3):
+            pipeline.render_backward(inp, out_b, ws_b.buffer, g_image, want=want)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(stage_steps):
+            pipeline.render_backward(inp, out_b, ws_b.buffer, g_image, want=want)
+        e1.record()
+        torch.cuda.synchronize()
+        t_bwd[label] = e0.elapsed_time(e1) / stage_steps
+    # algorithmic bytes: a 64-B gradient record per key written and 48 B of it read back; per key the sorted
+    # value, the 48-B record of its Gaussian, rectangle and first-record index; per visible Gaussian its inputs
+    # and record; per Gaussian radius, key count, first-record index and every gradient written
+    bwd_bytes = N * (64 + 48 + 4 + 48 + 12) + V * (12 + 12 + 16 + 4 * 3 * sh_coeffs + 48) + \
+        P * (12 + 12 + 12 + 4 + 12 + 16 + 4 * 3 * sh_coeffs)
+    return {"ms": round(t_bwd["all_gradients"], 4), "ms_without_sh_gradient": round(t_bwd["without_sh_gradient"], 4),
+            "bytes": bwd_bytes, "GBps": round(bwd_bytes / t_bwd["all_gradients"] / 1e6, 1),
+            "forward_plus_backward_frames_per_s": round(1e3 / (ms_per_step + t_bwd["all_gradients"]), 1)}
+
+
+# ----------------------------------------------------------------------------------------------------------------
+# CPU side (rank 0, N = 1): the checkers timed on the host cores.  Only this leg touches oracle/.
+
+def cpu_pair_stats(scene, cam=None, colors_precomp=None, sh_degree=None):
+    """The C checker over the whole frame: the (pixel, Gaussian) pair counts that define the blend's algorithmic
+    flops, and the checker's own frame time on the host cores."""
+    import numpy as np
+
+    from oracle import c_oracle as co
+    cam = cam or scene.camera
+    fr = co.Frame(cam.width, cam.height, math.tan(cam.FovX * 0.5), math.tan(cam.FovY * 0.5),
+                  cam.world_view_transform.cpu().numpy(), cam.full_proj_transform.cpu().numpy(),
+                  cam.camera_center.cpu().numpy(), scene.bg.cpu().numpy(), 1.0,
+                  scene.sh_degree if sh_degree is None else sh_degree)
+    kw = dict(scales=scene.scales.numpy(), rotations=scene.rotations.numpy())
+    if colors_precomp is not None:
+        kw["colors_precomp"] = np.ascontiguousarray(colors_precomp)
+    else:
+        kw["shs"] = scene.shs.numpy()
+    g = co.Gaussians(scene.means3D.numpy(), scene.opacities.numpy(), **kw)
+    threads = co.set_threads(min(os.cpu_count() or 1, 16))
+    t0 = time.perf_counter()
+    out = co.render(fr, g, keep_intermediates=False)
+    seconds = time.perf_counter() - t0
+    return {"evaluated": out["pairs_evaluated"], "accepted": out["pairs_accepted"], "tile_work": out["tile_work"],
+            "num_keys": out["num_keys"], "seconds": seconds, "threads": threads}
+
+
+def cpu_baseline(scene, pairs, colors_precomp=None, extra_seconds=0.0, extra_note=""):
+    """cpu_baseline object: the PyTorch-CPU rasterizer (bounded sample) with the C checker's whole-frame time beside it."""
+    from oracle import torch_oracle
+
+    base = torch_oracle.timed_baseline(scene, colors_precomp=colors_precomp, extra_seconds=extra_seconds,
+                                       extra_note=extra_note)
+    if pairs:
+        base["c_checker"] = {"frames_per_s": round(1.0 / (pairs["seconds"] + extra_seconds), 4), "threads": pairs["threads"],
+                             "sample": "oracle/gs_oracle.c, the whole frame (%d keys) in %.2f s" % (pairs["num_keys"],
+                                                                                                 pairs["seconds"])}
+    return base
+
+
+def guarded(fn, *a, **kw):
+    """The CPU leg is a reported figure, never a reason to lose the GPU numbers."""
+    try:
+        return fn(*a, **kw), None
+    except Exception as exc:  # noqa: BLE001
+        return None, repr(exc)
+
+
+# ----------------------------------------------------------------------------------------------------------------
+
+def frame_loop(torch, rast, kwargs, warmup, steps, settings_list=None):
+    """W untimed frames, then exactly K frames bracketed by synchronisation; frames/s and ms per frame."""
     with torch.no_grad():
-        for k in range(len(poses)):  # warm-up pass over the trajectory, also collects the per-pose statistics
-            rast.raster_settings = poses[k]
-            _, radii, _ = rast(**kwargs)
-            keys.append(rast.last_num_keys)
-            visible.append(int((radii > 0).sum()))
+        for k in range(warmup):
+            if settings_list:
+                rast.raster_settings = settings_list[k % len(settings_list)]
+            rast(**kwargs)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for k in range(args.steps):
-            rast.raster_settings = poses[k % len(poses)]
+        for k in range(steps):
+            if settings_list:
+                rast.raster_settings = settings_list[k % len(settings_list)]
             rast(**kwargs)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
-    cam = scene.camera
-    print(json.dumps({
-        "metric": "4K frames/sec at 20M Gaussians over 30 aerial poses (1 GPU)", "value": round(args.steps / elapsed, 2),
-        "unit": "frames/s", "n_gpus": 1, "steps": args.steps, "warmup": len(poses),
-        "ms_per_step": round(elapsed * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "configs[3]: %s, %d Gaussians, SH degree 3, %dx%d, %d poses" %
-                               (scene.name, scene.P, cam.width, cam.height, len(poses)),
-                   "keys_min_mean_max": [min(keys), int(sum(keys) / len(keys)), max(keys)],
-                   "visible_fraction_min_max": [round(min(visible) / scene.P, 3), round(max(visible) / scene.P, 3)]},
-    }))
+    return steps / elapsed, elapsed * 1e3 / steps
 
 
-def bench_scaffold(args, torch, dev):
-    """configs[4]: Scaffold-GS, anchors decoded on the matrix cores, then rasterized."""
-    from landmarksystem_amd import scenes
-    from landmarksystem_amd.models import ScaffoldGS
-
-    scene = scenes.config5(args.gaussians) if args.gaussians else scenes.config5()
-    model = ScaffoldGS.from_scene(scene, act_cache=True).to(dev).eval()
-    cam = scene.camera.to(dev)
-    for _ in range(args.warmup):
-        model(cam)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        model(cam)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    # the same frames with the one-kernel anchor prefilter, and an Octree-GS model over the same anchors (random
-    # levels 0..4) with the reference's level-of-detail sequence and with the fused prefilter
-    from landmarksystem_amd.models import OctreeGS
-    variants = {}
-    level = torch.randint(0, 5, (scene.anchor.shape[0],), generator=torch.Generator().manual_seed(5))
-    for name, make in () if args.no_model_level else (
-        ("scaffold_fused_prefilter", lambda: ScaffoldGS.from_scene(scene, act_cache=True, fuse_prefilter=True)),
-        ("octree_reference_sequence", lambda: OctreeGS(
-            scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
-            voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True)),
-        ("octree_fused_prefilter", lambda: OctreeGS(
-            scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
-            voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True, fuse_prefilter=True)),
-    ):
-        other = make()
-        other.anchor_decoder.load_state_dict(model.anchor_decoder.state_dict())
-        other = other.to(dev).eval()
-        for _ in range(5):
-            other(cam)
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        for _ in range(args.steps):
-            other(cam)
-        torch.cuda.synchronize()
-        variants[name] = round(args.steps / (time.perf_counter() - t1), 2)
-        del other
-    # decode alone, HIP events on the launch stream
-    vis = model.voxel_visible_mask
-    dec_args = dict(camera_center=cam.camera_center, anchor=model.get_anchor, anchor_feat=model.get_anchor_feat,
-                    offset=model.get_offset, scaling=model.get_scaling, visible_mask=vis)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(args.stage_steps):
-        out = model.anchor_decoder(**dec_args)
-    e1.record()
-    torch.cuda.synchronize()
-    dec_ms = e0.elapsed_time(e1) / args.stage_steps
-    a_vis, G = int(vis.sum()), out[0].shape[0]
-    flops = 13952 * a_vis
-    nbytes = a_vis * (128 + 120 + 24 + 12) * 2 + scene.anchor.shape[0] * (1 + 8) + G * 56  # inputs read by both passes
-    print(json.dumps({
-        "metric": "1080p frames/sec, Scaffold-GS with 500k anchors (1 GPU)", "value": round(args.steps / elapsed, 2),
-        "unit": "frames/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(elapsed * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 matrix inputs (hi+lo pairs), f32 accumulate", "data": "synthetic",
-        "config": {"workload": "configs[4]: %d anchors x %d offsets, 1920x1080" % (scene.anchor.shape[0], scene.n_offsets),
-                   "visible_anchors": a_vis, "decoded_gaussians": G},
-        "model_variants_frames_per_s": variants,
-        "decode": {"ms": round(dec_ms, 4), "anchors_per_s": round(a_vis / dec_ms * 1e3), "flops": flops,
-                   "TFLOPs": round(flops / dec_ms / 1e9, 3), "frac_mfma_f16": round(flops / dec_ms / 1e9 / 2500.0, 6),
-                   "bytes": nbytes, "GBps": round(nbytes / dec_ms / 1e6, 1),
-                   "frac_hbm": round(nbytes / dec_ms / 1e6 / HBM_PEAK_GBS, 4),
-                   "note": "two launches (count, emit) plus a scan and one host read-back of the output size; the "
-                           "stage is bound by HBM and launch latency, not by the matrix cores (17 flop/B)"},
-    }))
+def synchronised_latency(torch, call, frames):
+    """The reference's own protocol: synchronise, forward, synchronise around every frame, the first five frames
+    dropped (benchmarks/nerf/origin_gs/gs_evaluator.py:104-114,136), and its spread."""
+    per_frame = []
+    with torch.no_grad():
+        for _ in range(frames + 5):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            call()
+            torch.cuda.synchronize()
+            per_frame.append((time.perf_counter() - t0) * 1e3)
+    per_frame = sorted(per_frame[5:])
+    pick = lambda q: round(per_frame[min(len(per_frame) - 1, int(q * len(per_frame)))], 4)  # noqa: E731
+    return {"mean_ms": round(sum(per_frame) / len(per_frame), 4), "median_ms": pick(0.5), "p10_ms": pick(0.1),
+            "p90_ms": pick(0.9), "frames": len(per_frame), "frames_per_s": round(1e3 * len(per_frame) / sum(per_frame), 2)}
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build renders on one GPU; --gpus %d is not supported (run with --gpus 1)" % args.gpus,
-              file=sys.stderr)
-        sys.exit(2)
-    import torch
+def base_line(metric, fps, ms_per_step, args, warmup, dtype, config):
+    return {"metric": metric, "value": round(fps, 2), "unit": "frames/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": config}
 
+
+def bench_vanilla(args, torch, dev):
+    """configs[0..2]: one camera, the vanilla rasterizer call of the reference's model."""
     from landmarksystem_amd import GaussianRasterizer, _lib, pipeline, scenes
-
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    _lib.load()
-    dev = torch.device("cuda", 0)
-    torch.cuda.set_device(dev)
-    if args.config == 4:
-        return bench_trajectory(args, torch, dev)
-    if args.config == 5:
-        return bench_scaffold(args, torch, dev)
 
     t0 = time.time()
     make = scenes.BY_INDEX[args.config]
@@ -263,34 +353,8 @@ def main():
     rast = GaussianRasterizer(settings_for(scene, dev))
     kwargs = dict(means3D=d.means3D, means2D=None, shs=d.shs, colors_precomp=None, opacities=d.opacities,
                   scales=d.scales, rotations=d.rotations, cov3D_precomp=None)
-
-    with torch.no_grad():
-        for _ in range(args.warmup):
-            rast(**kwargs)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            image, radii, depth = rast(**kwargs)
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    fps = args.steps / elapsed
-
-    # per-frame latency: the reference's own protocol (synchronise, forward, synchronise around every frame, the
-    # first five frames dropped: benchmarks/nerf/origin_gs/gs_evaluator.py:104-114,136), and its spread
-    per_frame = []
-    with torch.no_grad():
-        for _ in range(min(args.steps, 60) + 5):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            rast(**kwargs)
-            torch.cuda.synchronize()
-            per_frame.append((time.perf_counter() - t0) * 1e3)
-    per_frame = sorted(per_frame[5:])
-    pick = lambda q: round(per_frame[min(len(per_frame) - 1, int(q * len(per_frame)))], 4)  # noqa: E731
-    latency = {"mean_ms": round(sum(per_frame) / len(per_frame), 4), "median_ms": pick(0.5), "p10_ms": pick(0.1),
-               "p90_ms": pick(0.9), "frames": len(per_frame),
-               "frames_per_s": round(1e3 * len(per_frame) / sum(per_frame), 2)}
+    fps, ms_per_step = frame_loop(torch, rast, kwargs, args.warmup, args.steps)
+    latency = synchronised_latency(torch, lambda: rast(**kwargs), min(args.steps, 60))
 
     # the same frames with two in flight (alternating HIP streams, one workspace each): the next frame's
     # HBM-bound preprocess overlaps the current frame's VALU-bound blend.  Reported beside `value`, never as it.
@@ -298,20 +362,21 @@ def main():
     fps_two_in_flight = None
     if args.two_in_flight:
         streams = [torch.cuda.Stream(device=dev) for _ in range(2)]
-        for k in range(4):
-            with torch.cuda.stream(streams[k % 2]):
-                rast(**kwargs)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for k in range(args.steps):
-            with torch.cuda.stream(streams[k % 2]):
-                rast(**kwargs)
-        torch.cuda.synchronize()
+        with torch.no_grad():
+            for k in range(4):
+                with torch.cuda.stream(streams[k % 2]):
+                    rast(**kwargs)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for k in range(args.steps):
+                with torch.cuda.stream(streams[k % 2]):
+                    rast(**kwargs)
+            torch.cuda.synchronize()
         fps_two_in_flight = round(args.steps / (time.perf_counter() - t0), 2)
 
     # model-level frame rate: the reference's forward sequence (visibility prefilter, gather of the survivors,
-    # rasterize) and the fused single-pass variant that produces the same frame
-    # (third variant: the same scene stored along a Morton curve, a load-time option of the checkpoint loaders)
+    # rasterize), the fused single-pass variant that produces the same frame, and that variant with the scene
+    # stored along a Morton curve (a load-time option of the checkpoint loaders)
     from landmarksystem_amd.models import GaussianModel, morton_order
     model_fps = {}
     for name, fuse, ordered in (() if args.no_model_level else (
@@ -340,135 +405,220 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # per-stage breakdown on the same inputs
     inp = pipeline.FrameInputs(rast.raster_settings, d.means3D, opacities=d.opacities, shs=d.shs, scales=d.scales,
                                rotations=d.rotations)
     n_cap = pipeline.default_workspace(dev).key_capacity
     stage_ms, stats = stage_breakdown(torch, pipeline, _lib, inp, n_cap, args.stage_steps)
     P, V, N = scene.P, stats["num_visible"], stats["num_keys"]
-    tiles, npix = inp.tiles, inp.width * inp.height
-
-    # blend work: exact pair count from the CPU oracle would need minutes at this size; use the
-    # kernel-independent upper bound 256 * (sum of tile range lengths), as defined for the blend stage
-    blend_pairs_upper = 256 * stats["range_sum"]
-    work = algorithmic_work(P, V, N, tiles, npix, scene.shs.shape[1], stats["sort_passes"], blend_pairs_upper)
-    def hbm(name, ms, nbytes):
-        return {"ms": round(ms, 4), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
-                "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
-
-    stages = {"preprocess": hbm("preprocess", stage_ms["preprocess"], work["preprocess"])}
-    # key generation + sort + ranges: the shipped tile-bucketed stages (bin, tile_sort) produce the same sorted
-    # pairs and ranges as duplicate + LSD radix sort + ranges, so they are charged the same algorithmic bytes
-    sort_bytes = work["scan"] + work["duplicate"] + work["sort"] + work["ranges"]
-    sort_ms = stage_ms["tile_count"] + stage_ms["tile_scatter"] + stage_ms["tile_sort"]
-    for name in ("tile_count", "tile_scatter", "tile_sort"):
-        stages[name] = {"ms": round(stage_ms[name], 4)}
-    stages["keys_sort_ranges"] = hbm("keys_sort_ranges", sort_ms, sort_bytes)
-    stages["keys_sort_ranges"]["floor_bytes"] = 24 * N
-    stages["classic_lsd_path"] = {"scan_ms": round(stage_ms["scan"], 4), "duplicate_ms": round(stage_ms["duplicate"], 4), "sort_ms": round(stage_ms["sort"], 4),
-                                  "ranges_ms": round(stage_ms["ranges"], 4),
-                                  "sort_GBps": round(work["sort"] / stage_ms["sort"] / 1e6, 1)}
-    ms = stage_ms["blend"]
-    default_workload = args.config == 3 and not args.gaussians
-    stages["blend"] = {"ms": round(ms, 4), "flops_upper": work["blend_flops"],
-                       "TFLOPs_upper": round(work["blend_flops"] / ms / 1e9, 2),
-                       "frac_fp32_upper": round(work["blend_flops"] / ms / 1e9 / FP32_PEAK_TFLOPS, 4)}
-    if default_workload:
-        flops = 25 * BLEND_PAIRS["evaluated"]
-        stages["blend"].update({
-            "pairs_evaluated": BLEND_PAIRS["evaluated"], "pairs_accepted": BLEND_PAIRS["accepted"],
-            "flops_algorithmic": flops, "TFLOPs_algorithmic": round(flops / ms / 1e9, 2),
-            "frac_fp32_algorithmic": round(flops / ms / 1e9 / FP32_PEAK_TFLOPS, 4),
-            "TFLOPs_issued": round(BLEND_ISSUED_FLOPS / ms / 1e9, 2),
-            "frac_fp32_issued": round(BLEND_ISSUED_FLOPS / ms / 1e9 / FP32_PEAK_TFLOPS, 4)})
-    pre_sort_bytes = work["preprocess"] + sort_bytes
-    pre_sort_ms = stage_ms["preprocess"] + sort_ms
-    stages["preprocess_plus_sort"] = hbm("preprocess_plus_sort", pre_sort_ms, pre_sort_bytes)
-    stages["rates"] = {"gaussians_per_s_preprocess": round(P / stage_ms["preprocess"] * 1e3),
-                       "sorted_keys_per_s": round(N / sort_ms * 1e3) if N else 0,
-                       "blend_frames_per_s": round(1e3 / stage_ms["blend"], 1)}
-
-    # backward pass of the same frame (the training loop's loss.backward() on an image loss): all gradients of a
-    # forward render, reported beside the forward stages, never part of `value`
+    pairs, pairs_error = (None, None) if args.no_cpu_baseline else guarded(cpu_pair_stats, scene)
+    counters = COUNTER_TRAFFIC if (args.config == 3 and not args.gaussians) else None
+    stages, roofline = raster_report(stage_ms, stats, P, inp.tiles, inp.width * inp.height, 12 * scene.shs.shape[1],
+                                     pairs, counters)
+    if pairs and pairs["num_keys"] != N:
+        stages["blend"]["pairs_note"] = "the checker counted %d keys, the GPU %d" % (pairs["num_keys"], N)
     if not args.no_backward:
-        ws_b = pipeline.Workspace(dev)
-        ws_b.key_capacity = n_cap
-        out_b = pipeline.render(inp, ws=ws_b)
-        g_image = torch.randn(3, inp.height, inp.width, device=dev)
-        t_bwd = {}
-        for label, want in (("all_gradients", pipeline.GRAD_NAMES),
-                            ("without_sh_gradient", tuple(n for n in pipeline.GRAD_NAMES if n != "shs"))):
-            for _ in range(3):
-                pipeline.render_backward(inp, out_b, ws_b.buffer, g_image, want=want)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(args.stage_steps):
-                pipeline.render_backward(inp, out_b, ws_b.buffer, g_image, want=want)
-            e1.record()
-            torch.cuda.synchronize()
-            t_bwd[label] = e0.elapsed_time(e1) / args.stage_steps
-        # algorithmic bytes: a 64-B gradient record per key written and 48 B of it read back; per key the sorted
-        # value, the 48-B record of its Gaussian, rectangle and first-record index; per visible Gaussian its inputs
-        # and record; per Gaussian radius, key count, first-record index and every gradient written
-        bwd_bytes = N * (64 + 48 + 4 + 48 + 12) + V * (12 + 12 + 16 + 4 * 3 * scene.shs.shape[1] + 48) + \
-            P * (12 + 12 + 12 + 4 + 12 + 16 + 4 * 3 * scene.shs.shape[1])
-        stages["backward"] = {"ms": round(t_bwd["all_gradients"], 4),
-                              "ms_without_sh_gradient": round(t_bwd["without_sh_gradient"], 4),
-                              "bytes": bwd_bytes, "GBps": round(bwd_bytes / t_bwd["all_gradients"] / 1e6, 1),
-                              "forward_plus_backward_frames_per_s":
-                                  round(1e3 / (ms_per_step + t_bwd["all_gradients"]), 1)}
-        del ws_b, out_b
-
-    # counter-measured traffic only applies to the workload it was measured on
-    traffic = MEASURED_TRAFFIC_BYTES if default_workload else {}
-    shipped = {"preprocess": stage_ms["preprocess"], "keys_sort_ranges": sort_ms,
-               "blend": stage_ms["blend"]}
-    dominant = max(shipped, key=lambda n: shipped[n])
-    if dominant == "blend":
-        kind = "algorithmic" if default_workload else "upper"
-        roofline = {"bound": "mfma", "kernel": "blend_kernel", "achieved": stages["blend"]["TFLOPs_" + kind],
-                    "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": stages["blend"]["frac_fp32_" + kind],
-                    "traffic": traffic.get("blend"),
-                    "note": "FP32 VALU kernel (no MFMA); peak is the MI355X fp32 vector figure (packed FMA; this build "
-                            "issues unpacked fp32, half of it).  flops = 25 x the (pixel, Gaussian) pairs the per-pixel "
-                            "loop evaluates" + (" (counted by the CPU checker for this seeded scene); the kernel skips "
-                            "pairs whose alpha is provably < 1/255, so it issues fewer flops than that: see "
-                            "stages.blend.TFLOPs_issued" if default_workload else
-                            ", bounded above by 256 x sum of tile range lengths")}
-    else:
-        roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": traffic.get(dominant)}
-
-    result = {
-        "metric": "1080p frames/sec at 6M Gaussians (1 GPU)",
-        "value": round(fps, 2),
-        "unit": "frames/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": "configs[%d]: %s, %d Gaussians, SH degree %d, %dx%d, RGB+depth+alpha" %
-                               (args.config - 1, scene.name, P, scene.sh_degree, inp.width, inp.height),
-                   "visible": V, "keys": N, "tiles": tiles, "scene_gen_s": round(gen_s, 1)},
-        "roofline": roofline,
-        "stages": stages,
-        "model_forward_frames_per_s": model_fps,
-        "two_frames_in_flight_frames_per_s": fps_two_in_flight,
-        "synchronised_per_frame": latency,
-    }
+        stages["backward"] = backward_report(torch, pipeline, inp, n_cap, N, V, P, scene.shs.shape[1], ms_per_step,
+                                             args.stage_steps)
+    metric = "1080p frames/sec at 6M Gaussians (1 GPU)" if args.config == 3 and not args.gaussians else \
+        "%dx%d frames/sec at %d Gaussians (1 GPU)" % (inp.width, inp.height, P)
+    result = base_line(metric, fps, ms_per_step, args, args.warmup, "f32", {
+        "workload": "configs[%d]: %s, %d Gaussians, SH degree %d, %dx%d, RGB+depth+alpha" %
+                    (args.config - 1, scene.name, P, scene.sh_degree, inp.width, inp.height),
+        "visible": V, "keys": N, "tiles": inp.tiles, "scene_gen_s": round(gen_s, 1)})
+    result.update({"roofline": roofline, "stages": stages, "model_forward_frames_per_s": model_fps,
+                   "two_frames_in_flight_frames_per_s": fps_two_in_flight, "synchronised_per_frame": latency})
     if not args.no_cpu_baseline:
-        try:
-            from oracle import torch_oracle
-
-            result["cpu_baseline"] = torch_oracle.timed_baseline(scene)
-        except Exception as exc:  # the baseline is a reported figure, never a reason to lose the GPU numbers
-            result["cpu_baseline"] = {"error": repr(exc)}
+        base, err = guarded(cpu_baseline, scene, pairs)
+        result["cpu_baseline"] = base if base else {"error": err}
+        if pairs_error:
+            result["cpu_baseline"]["c_checker_error"] = pairs_error
     print(json.dumps(result))
+
+
+def bench_trajectory(args, torch, dev):
+    """configs[3]: large slab at 4K over a trajectory of aerial poses.  `value` is the frame rate over the
+    trajectory; the stage breakdown, roofline and CPU baseline are those of its first pose."""
+    from landmarksystem_amd import GaussianRasterizer, _lib, pipeline, scenes
+
+    t0 = time.time()
+    scene = scenes.config4(args.gaussians) if args.gaussians else scenes.config4()
+    gen_s = time.time() - t0
+    d = scene.to(dev)
+    rast = GaussianRasterizer(settings_for(scene, dev))
+    base = rast.raster_settings
+    poses = [base._replace(viewmatrix=c.world_view_transform, projmatrix=c.full_proj_transform,
+                           campos=c.camera_center) for c in d.cameras]
+    kwargs = dict(means3D=d.means3D, means2D=None, shs=d.shs, colors_precomp=None, opacities=d.opacities,
+                  scales=d.scales, rotations=d.rotations, cov3D_precomp=None)
+    keys, visible = [], []
+    with torch.no_grad():
+        for k in range(len(poses)):  # warm-up pass over the trajectory, also collects the per-pose statistics
+            rast.raster_settings = poses[k]
+            _, radii, _ = rast(**kwargs)
+            keys.append(rast.last_num_keys)
+            visible.append(int((radii > 0).sum()))
+    fps, ms_per_step = frame_loop(torch, rast, kwargs, 0, args.steps, settings_list=poses)
+
+    rast.raster_settings = poses[0]
+    inp = pipeline.FrameInputs(poses[0], d.means3D, opacities=d.opacities, shs=d.shs, scales=d.scales,
+                               rotations=d.rotations)
+    n_cap = pipeline.default_workspace(dev).key_capacity
+    stage_ms, stats = stage_breakdown(torch, pipeline, _lib, inp, n_cap, max(3, args.stage_steps // 2))
+    pairs, pairs_error = (None, None) if args.no_cpu_baseline else guarded(cpu_pair_stats, scene)
+    stages, roofline = raster_report(stage_ms, stats, scene.P, inp.tiles, inp.width * inp.height,
+                                     12 * scene.shs.shape[1], pairs, None)
+    cam = scene.camera
+    result = base_line("4K frames/sec at 20M Gaussians over 30 aerial poses (1 GPU)", fps, ms_per_step, args,
+                       len(poses), "f32", {
+        "workload": "configs[3]: %s, %d Gaussians, SH degree 3, %dx%d, %d poses" %
+                    (scene.name, scene.P, cam.width, cam.height, len(poses)),
+        "keys_min_mean_max": [min(keys), int(sum(keys) / len(keys)), max(keys)],
+        "visible_fraction_min_max": [round(min(visible) / scene.P, 3), round(max(visible) / scene.P, 3)],
+        "stages_of": "pose 0 (%d keys, %d visible)" % (stats["num_keys"], stats["num_visible"]),
+        "tiles": inp.tiles, "scene_gen_s": round(gen_s, 1)})
+    result.update({"roofline": roofline, "stages": stages})
+    if not args.no_cpu_baseline:
+        base, err = guarded(cpu_baseline, scene, pairs)
+        result["cpu_baseline"] = base if base else {"error": err}
+        if pairs_error:
+            result["cpu_baseline"]["c_checker_error"] = pairs_error
+    print(json.dumps(result))
+
+
+def bench_scaffold(args, torch, dev):
+    """configs[4]: Scaffold-GS, anchors decoded on the matrix cores, then rasterized."""
+    from landmarksystem_amd import _lib, pipeline, scenes
+    from landmarksystem_amd.models import OctreeGS, ScaffoldGS
+
+    scene = scenes.config5(args.gaussians) if args.gaussians else scenes.config5()
+    A = scene.anchor.shape[0]
+    model = ScaffoldGS.from_scene(scene, act_cache=True).to(dev).eval()  # the reference's own forward sequence
+    cam = scene.camera.to(dev)
+    for _ in range(args.warmup):
+        model(cam)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model(cam)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    fps, ms_per_step = args.steps / elapsed, elapsed * 1e3 / args.steps
+    latency = synchronised_latency(torch, lambda: model(cam), min(args.steps, 60))
+
+    # the same frames with the one-kernel anchor prefilter, and an Octree-GS model over the same anchors (random
+    # levels 0..4) with the reference's level-of-detail sequence and with the fused prefilter
+    variants = {}
+    level = torch.randint(0, 5, (A,), generator=torch.Generator().manual_seed(5))
+    for name, make in () if args.no_model_level else (
+        ("scaffold_fused_prefilter", lambda: ScaffoldGS.from_scene(scene, act_cache=True, fuse_prefilter=True)),
+        ("octree_reference_sequence", lambda: OctreeGS(
+            scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
+            voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True)),
+        ("octree_fused_prefilter", lambda: OctreeGS(
+            scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
+            voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True, fuse_prefilter=True)),
+    ):
+        other = make()
+        other.anchor_decoder.load_state_dict(model.anchor_decoder.state_dict())
+        other = other.to(dev).eval()
+        for _ in range(5):
+            other(cam)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            other(cam)
+        torch.cuda.synchronize()
+        variants[name] = round(args.steps / (time.perf_counter() - t1), 2)
+        del other
+
+    # stages: anchor prefilter and decode alone (HIP events on the launch stream), then the rasterizer stages on the
+    # decoded Gaussians
+    def timed(call):
+        for _ in range(3):
+            call()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.stage_steps):
+            res = call()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.stage_steps, res
+
+    with torch.no_grad():
+        prefilter_ms, vis = timed(lambda: model.prefilter_voxel(cam))
+        dec_args = dict(camera_center=cam.camera_center, anchor=model.get_anchor, anchor_feat=model.get_anchor_feat,
+                        offset=model.get_offset, scaling=model.get_scaling, visible_mask=vis)
+        dec_ms, dec = timed(lambda: model.anchor_decoder(**dec_args))
+    xyz, color, opacity, scaling, rot = dec[:5]
+    a_vis, G = int(vis.sum()), int(xyz.shape[0])
+    flops = 13952 * a_vis
+    dec_bytes = a_vis * (128 + 120 + 24 + 12) + A * 1 + G * 56
+    settings = settings_for(scene, dev, sh_degree=1)
+    inp = pipeline.FrameInputs(settings, xyz, opacities=opacity, colors_precomp=color, scales=scaling, rotations=rot)
+    n_cap = max(pipeline.default_workspace(dev).key_capacity, 1 << 20)
+    stage_ms, stats = stage_breakdown(torch, pipeline, _lib, inp, n_cap, args.stage_steps)
+
+    decoded = scenes.GaussianScene("decoded", xyz.cpu(), scaling.cpu(), rot.cpu(), opacity.cpu(),
+                                   torch.zeros(G, 1, 3), 1, [scene.camera], scene.bg)
+    pairs, pairs_error = (None, None) if args.no_cpu_baseline else guarded(
+        cpu_pair_stats, decoded, colors_precomp=color.cpu().numpy(), sh_degree=1)
+    stages, roofline = raster_report(stage_ms, stats, G, inp.tiles, inp.width * inp.height, 12, pairs, None)
+    stages["anchor_prefilter"] = {"ms": round(prefilter_ms, 4), "bytes": 36 * A,
+                                  "GBps": round(36 * A / prefilter_ms / 1e6, 1),
+                                  "frac_hbm": round(36 * A / prefilter_ms / 1e6 / HBM_PEAK_GBS, 4)}
+    stages["decode"] = {"ms": round(dec_ms, 4), "anchors_per_s": round(a_vis / dec_ms * 1e3), "flops": flops,
+                        "TFLOPs": round(flops / dec_ms / 1e9, 3),
+                        "frac_mfma_f16": round(flops / dec_ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 6),
+                        "bytes": dec_bytes, "GBps": round(dec_bytes / dec_ms / 1e6, 1),
+                        "frac_hbm": round(dec_bytes / dec_ms / 1e6 / HBM_PEAK_GBS, 4),
+                        "note": "bound by HBM and instruction issue, not by the matrix cores (17 flop/B); bytes = inputs "
+                                "of the visible anchors once + the visibility mask + 56 B per emitted Gaussian"}
+    if dec_ms > max(stage_ms["preprocess"], stage_ms["blend"],
+                    stage_ms["tile_count"] + stage_ms["tile_scatter"] + stage_ms["tile_sort"]):
+        roofline = {"bound": "hbm", "kernel": "decode_kernel", "achieved": stages["decode"]["GBps"], "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": stages["decode"]["frac_hbm"], "traffic": None,
+                    "mfma_frac": stages["decode"]["frac_mfma_f16"]}
+    result = base_line("1080p frames/sec, Scaffold-GS with 500k anchors (1 GPU)", fps, ms_per_step, args, args.warmup,
+                       "f32 (decode: f16 matrix inputs as hi+lo pairs, f32 accumulate)", {
+        "workload": "configs[4]: %d anchors x %d offsets, 1920x1080" % (A, scene.n_offsets),
+        "visible_anchors": a_vis, "decoded_gaussians": G, "keys": stats["num_keys"], "tiles": inp.tiles})
+    result.update({"roofline": roofline, "stages": stages, "model_variants_frames_per_s": variants,
+                   "synchronised_per_frame": latency})
+    if not args.no_cpu_baseline:
+        def whole():
+            from oracle import anchor_oracle
+            t1 = time.perf_counter()
+            anchor_oracle.decode(scene.camera.camera_center, scene.anchor, scene.anchor_feat, scene.offset,
+                                 scene.scaling, vis.cpu(), scene.mlp, scene.n_offsets)
+            dec_s = time.perf_counter() - t1
+            return cpu_baseline(decoded, pairs, colors_precomp=color.cpu(), extra_seconds=dec_s,
+                                extra_note="anchor decode (oracle/anchor_oracle.py, %d visible anchors) %.2fs + " % (a_vis, dec_s))
+        base, err = guarded(whole)
+        result["cpu_baseline"] = base if base else {"error": err}
+        if pairs_error:
+            result["cpu_baseline"]["c_checker_error"] = pairs_error
+    print(json.dumps(result))
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build renders on one GPU; --gpus %d is not supported (run with --gpus 1)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from landmarksystem_amd import _lib
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    _lib.load()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    if args.config == 4:
+        return bench_trajectory(args, torch, dev)
+    if args.config == 5:
+        return bench_scaffold(args, torch, dev)
+    return bench_vanilla(args, torch, dev)
 
 
 if __name__ == "__main__":

@@ -14,6 +14,8 @@
 // order a stable sort of the emission-ordered keys produces.
 //
 // No workgroup waits on another; persistent loops run over fixed lists.
+#include <atomic>
+
 #include "gs355_internal.h"
 
 namespace gs355 {
@@ -21,10 +23,7 @@ namespace gs355 {
 namespace {
 
 constexpr int kInlineTiles = 32;  // splats touching more tiles than this are expanded by the whole workgroup
-#ifndef GS355_BIN_ITEMS
-#define GS355_BIN_ITEMS 4
-#endif
-constexpr int kBinItems = GS355_BIN_ITEMS;  // Gaussians per thread and round of the binning walk
+constexpr int kBinItems = 4;      // Gaussians per thread and round of the binning walk
 
 // ---------------------------------------------------------------------------
 // Binning.  Workgroup c owns Gaussians [c * per_group, (c+1) * per_group) and a
@@ -861,10 +860,32 @@ int bin_groups(int32_t P, int* per_group)
     return groups < 1 ? 1 : groups;
 }
 
-static int set_bin_lds(const void* fn, size_t bytes)
+// Dynamic LDS beyond 64 KB has to be allowed per kernel.  The limits are raised once per process and device to
+// the largest size any launch can ask for, so that concurrent frames of different image sizes (other streams,
+// other threads) never lower the limit under each other.
+template <typename K>
+static hipError_t raise_lds_limit(K kernel, size_t bytes)
 {
-    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return set_error(GS355_EHIP, "bin: LDS attribute: %s", hipGetErrorString(e));
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)bytes);
+}
+
+static int allow_large_lds()
+{
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> done[kMaxDevices];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_error(GS355_EHIP, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return set_error(GS355_EINVAL, "device index %d is outside [0, %d)", dev, kMaxDevices);
+    if (done[dev].load(std::memory_order_acquire)) return GS355_OK;
+    const size_t bin_bytes = (size_t)kBinMaxTiles * sizeof(uint32_t);
+    if ((e = raise_lds_limit(bin_kernel<false>, bin_bytes)) != hipSuccess ||
+        (e = raise_lds_limit(bin_kernel<true>, bin_bytes)) != hipSuccess ||
+        (e = raise_lds_limit(tile_sort_list_1024x5_kernel, LdsSorter<1024, 5>::kBytes)) != hipSuccess ||
+        (e = raise_lds_limit(tile_sort_list_kernel<1024, 10>, LdsSorter<1024, 10>::kBytes)) != hipSuccess)
+        return set_error(GS355_EHIP, "LDS limit of the binning / tile sort kernels: %s", hipGetErrorString(e));
+    done[dev].store(1, std::memory_order_release);  // racing threads set the same values
     return GS355_OK;
 }
 
@@ -874,7 +895,7 @@ int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint
     int per_group;
     const int groups = bin_groups(P, &per_group);
     const size_t lds = (size_t)f.grid_x * f.grid_y * sizeof(uint32_t);
-    int rc = set_bin_lds(reinterpret_cast<const void*>(bin_kernel<false>), lds);
+    int rc = allow_large_lds();
     if (rc) return rc;
     hipLaunchKernelGGL(bin_kernel<false>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, rects,
                        (const uint32_t*)nullptr, (const gs355_header*)nullptr, matrix, (const uint32_t*)nullptr,
@@ -904,20 +925,11 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
     int per_group;
     const int groups = bin_groups(P, &per_group);
     const size_t lds = (size_t)f.grid_x * f.grid_y * sizeof(uint32_t);
-    int rc = set_bin_lds(reinterpret_cast<const void*>(bin_kernel<true>), lds);
+    int rc = allow_large_lds();
     if (rc) return rc;
     hipLaunchKernelGGL(bin_kernel<true>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, rects, depth_bits,
                        header, const_cast<uint32_t*>(matrix), tile_base, (uint32_t*)nullptr, buckets);
     GS355_CHECK_LAUNCH("bin: scatter");
-    return GS355_OK;
-}
-
-template <typename K>
-static int allow_lds(K kernel, size_t bytes)
-{
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return set_error(GS355_EHIP, "tile sort: LDS attribute: %s", hipGetErrorString(e));
     return GS355_OK;
 }
 
@@ -931,8 +943,7 @@ int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* rang
     static_assert(S0::kCap == kTileSortCap[0] && S1::kCap == kTileSortCap[1] && S2::kCap == kTileSortCap[2] &&
                       S3::kCap == kTileSortCap[3], "size classes out of step with the layout kernel");
     int rc;
-    if ((rc = allow_lds(tile_sort_list_1024x5_kernel, S2::kBytes))) return rc;
-    if ((rc = allow_lds(tile_sort_list_kernel<1024, 10>, S3::kBytes))) return rc;
+    if ((rc = allow_large_lds())) return rc;
     const uint32_t* list0 = lists + 4;
     hipLaunchKernelGGL((tile_sort_each_kernel<256, 4>), dim3(tiles), dim3(256), S0::kBytes, s, header, ranges, buckets,
                        out_keys, out_vals);

@@ -220,19 +220,24 @@ def render_trajectory(model, cameras, in_flight: int = 2, **forward_kwargs):
         image.record_stream(caller)
         return image
 
-    with torch.no_grad():
-        for k, camera in enumerate(cameras):
-            stream = streams[k % in_flight]
-            stream.wait_stream(caller)  # whatever produced the model's inputs has been enqueued before
-            with torch.cuda.stream(stream):
-                image = model(camera, **forward_kwargs)
-                done = torch.cuda.Event()
-                done.record(stream)
-            pending.append((image, done))
-            if len(pending) >= in_flight:
+    try:
+        with torch.no_grad():
+            for k, camera in enumerate(cameras):
+                stream = streams[k % in_flight]
+                stream.wait_stream(caller)  # whatever produced the model's inputs has been enqueued before
+                with torch.cuda.stream(stream):
+                    image = model(camera, **forward_kwargs)
+                    done = torch.cuda.Event()
+                    done.record(stream)
+                pending.append((image, done))
+                if len(pending) >= in_flight:
+                    yield hand_over(pending.popleft())
+            while pending:
                 yield hand_over(pending.popleft())
-        while pending:
-            yield hand_over(pending.popleft())
+    finally:
+        from . import pipeline
+        for stream in streams:  # the streams retire with this call: so do their rasterizer workspaces
+            pipeline.release_workspace(device, stream)
 
 
 def init_inference(based_model_cls, infer_model_cls, model_config: Union[str, Path, Config, Dict, None],

@@ -12,9 +12,11 @@ the callers on either side of the rasterizer.
 They keep the reference's call sequence (visibility prefilter -> optional
 anchor decode -> settings record re-assigned on the renderer -> rasterize),
 its eval-mode gather of the visible Gaussians and its `act_cache` behaviour,
-and its parameter names so checkpoints map one to one.  Forward / eval only:
-training and densification are not part of this package; checkpoint I/O lives
-in `checkpoints.py`.
+and its parameter names so checkpoints map one to one.  The vanilla model also
+runs in training mode (every Gaussian rendered, differentiable through the
+rasterizer's backward pass, `viewspace_points` kept for densification); the
+Scaffold- / Octree-GS models are forward-only.  Optimizers and densification
+are not part of this package; checkpoint I/O lives in `checkpoints.py`.
 Activations and gathers are a handful of torch elementwise calls, as in the
 reference; everything per-Gaussian and per-pixel runs in the HIP library.
 """

@@ -7,6 +7,7 @@ HIP kernel behind `gs355_run` / `gs355_visible_filter`.
 """
 import ctypes as C
 import math
+from collections import OrderedDict
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -87,16 +88,34 @@ class Workspace:
         raise KeyError(name)
 
 
-_workspaces: Dict[Tuple[int, int], Workspace] = {}
+# One workspace per (device, stream) that rendered recently: frames on different streams may be in flight together
+# and must not share buffers.  Least recently used entries beyond _MAX_WORKSPACES are dropped (their device memory
+# goes back to torch's allocator, which orders its reuse after the work already enqueued on that stream).
+_MAX_WORKSPACES = 8
+_workspaces: "OrderedDict[Tuple[int, int], Workspace]" = OrderedDict()
+
+
+def _workspace_key(device: torch.device, stream=None) -> Tuple[int, int]:
+    stream = stream if stream is not None else torch.cuda.current_stream(device)
+    return (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
 
 
 def default_workspace(device: torch.device) -> Workspace:
-    stream = torch.cuda.current_stream(device)
-    key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    key = _workspace_key(device)
     ws = _workspaces.get(key)
     if ws is None:
         ws = _workspaces[key] = Workspace(device)
+        while len(_workspaces) > _MAX_WORKSPACES:
+            _workspaces.popitem(last=False)
+    else:
+        _workspaces.move_to_end(key)
     return ws
+
+
+def release_workspace(device: torch.device, stream=None) -> None:
+    """Drop the workspace of `stream` (default: the current stream) on `device`, e.g. when a temporary stream
+    retires.  Frames already enqueued keep their memory until they have run."""
+    _workspaces.pop(_workspace_key(device, stream), None)
 
 
 class FrameInputs:

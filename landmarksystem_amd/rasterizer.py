@@ -57,7 +57,11 @@ _INPUT_NAMES = ("means3D", "means2D", "opacities", "shs", "colors_precomp", "sca
 
 
 class _RasterizeGaussians(torch.autograd.Function):
-    """forward(): one frame in a workspace of its own, kept until backward() has read it."""
+    """forward(): one frame in a workspace of its own, kept until backward() has read it.
+
+    Memory: every graph that is still waiting for its backward pass holds the whole workspace of its frame (records,
+    keys, values, binning tables: about 0.7 GB at 6M Gaussians / 13.6M keys, 2 GB at 20M Gaussians in 4K), released
+    when backward() has run or the graph is dropped.  The backward pass can run once per forward pass."""
 
     @staticmethod
     def forward(ctx, settings, means3D, means2D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp):
@@ -87,6 +91,10 @@ class _RasterizeGaussians(torch.autograd.Function):
         needs = dict(zip(_INPUT_NAMES, ctx.needs_input_grad[1:]))
         if g_image is None and g_depth is None and g_alpha is None:
             return (None,) * 9
+        if ctx.workspace is None:
+            raise RuntimeError("the rasterizer's backward pass ran already for this frame: its workspace is released "
+                               "after the first backward pass (retain_graph=True cannot replay it); render the frame "
+                               "again")
         inputs = pipeline.FrameInputs(ctx.settings, means3D, opacities=opacities, shs=shs,
                                       colors_precomp=colors_precomp, scales=scales, rotations=rotations,
                                       cov3D_precomp=cov3D_precomp)

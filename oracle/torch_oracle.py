@@ -252,11 +252,15 @@ def frame_dict(scene, cam=None):
                 scale_modifier=1.0, sh_degree=scene.sh_degree)
 
 
-def timed_baseline(scene, blend_budget_s: float = 12.0):
+def timed_baseline(scene, blend_budget_s: float = 12.0, colors_precomp=None, extra_seconds: float = 0.0,
+                   extra_note: str = ""):
     """CPU baseline for bench.py: preprocess, key generation and the stable
     sort are timed in full on all host cores; blending is timed on every k-th
     tile (k chosen so that it fits the budget) and extrapolated by range
-    length.  Returns the cpu_baseline object of the bench line."""
+    length.  `colors_precomp` replaces the SH evaluation (the Scaffold-GS
+    call); `extra_seconds` / `extra_note` add a stage timed by the caller (the
+    anchor decode) to the frame time.  Returns the cpu_baseline object of the
+    bench line."""
     cores = os.cpu_count() or 1
     cores = min(cores, 16)
     torch.set_num_threads(cores)
@@ -265,8 +269,8 @@ def timed_baseline(scene, blend_budget_s: float = 12.0):
     gx, gy = (W + 15) // 16, (H + 15) // 16
     with torch.no_grad():
         t0 = time.perf_counter()
-        pre = preprocess(fr, scene.means3D, scene.opacities, shs=scene.shs, scales=scene.scales,
-                         rotations=scene.rotations)
+        pre = preprocess(fr, scene.means3D, scene.opacities, shs=None if colors_precomp is not None else scene.shs,
+                         colors_precomp=colors_precomp, scales=scene.scales, rotations=scene.rotations)
         t1 = time.perf_counter()
         keys, vals, _ = make_keys(pre, gx)
         t2 = time.perf_counter()
@@ -287,13 +291,13 @@ def timed_baseline(scene, blend_budget_s: float = 12.0):
                 break
         t_blend = time.perf_counter() - tb0
     blend_full = t_blend * (total_len / sample_len) if sample_len > 0 else t_blend * gx * gy / max(done_tiles, 1)
-    frame_s = (t1 - t0) + (t2 - t1) + (t3 - t2) + blend_full
+    frame_s = (t1 - t0) + (t2 - t1) + (t3 - t2) + blend_full + extra_seconds
     return {
         "value": round(1.0 / frame_s, 4),
         "unit": "frames/s",
         "cores": cores,
         "kind": "port",
-        "sample": ("PyTorch-CPU rasterizer (oracle/torch_oracle.py), same scene: preprocess %.2fs + keys %.2fs + "
+        "sample": (extra_note + "PyTorch-CPU rasterizer (oracle/torch_oracle.py), same scene: preprocess %.2fs + keys %.2fs + "
                    "stable sort/ranges %.2fs timed in full (%d Gaussians, %d keys); blend timed on %d of %d tiles "
                    "(every %dth, %.2fs) and extrapolated by tile range length to %.1fs"
                    % (t1 - t0, t2 - t1, t3 - t2, scene.P, keys.numel(), done_tiles, gx * gy, stride, t_blend,

@@ -65,6 +65,9 @@ def parse_args():
                     help="skip the model-level variants (their launches of the same kernels on other inputs would "
                          "mix into the per-kernel averages of a profiler run)")
     ap.add_argument("--no-backward", action="store_true", help="skip the backward-pass timing")
+    ap.add_argument("--spatial-order", action="store_true",
+                    help="store the scene along a Morton curve first (the checkpoint loaders' spatial_order option); "
+                         "same Gaussians, coherent memory traffic; not the headline workload")
     ap.add_argument("--two-in-flight", action="store_true",
                     help="also time the frames with two in flight on alternating streams (reported beside `value`)")
     return ap.parse_args()
@@ -349,6 +352,12 @@ def bench_vanilla(args, torch, dev):
     make = scenes.BY_INDEX[args.config]
     scene = make(args.gaussians) if args.gaussians else make()
     gen_s = time.time() - t0
+    if args.spatial_order:
+        from landmarksystem_amd.models import morton_order
+        order = morton_order(scene.means3D)
+        scene = scenes.GaussianScene(scene.name + " (Morton order)", scene.means3D[order], scene.scales[order],
+                                     scene.rotations[order], scene.opacities[order], scene.shs[order], scene.sh_degree,
+                                     scene.cameras, scene.bg)
     d = scene.to(dev)
     rast = GaussianRasterizer(settings_for(scene, dev))
     kwargs = dict(means3D=d.means3D, means2D=None, shs=d.shs, colors_precomp=None, opacities=d.opacities,
@@ -411,7 +420,7 @@ def bench_vanilla(args, torch, dev):
     stage_ms, stats = stage_breakdown(torch, pipeline, _lib, inp, n_cap, args.stage_steps)
     P, V, N = scene.P, stats["num_visible"], stats["num_keys"]
     pairs, pairs_error = (None, None) if args.no_cpu_baseline else guarded(cpu_pair_stats, scene)
-    counters = COUNTER_TRAFFIC if (args.config == 3 and not args.gaussians) else None
+    counters = COUNTER_TRAFFIC if (args.config == 3 and not args.gaussians and not args.spatial_order) else None
     stages, roofline = raster_report(stage_ms, stats, P, inp.tiles, inp.width * inp.height, 12 * scene.shs.shape[1],
                                      pairs, counters)
     if pairs and pairs["num_keys"] != N:
@@ -419,7 +428,8 @@ def bench_vanilla(args, torch, dev):
     if not args.no_backward:
         stages["backward"] = backward_report(torch, pipeline, inp, n_cap, N, V, P, scene.shs.shape[1], ms_per_step,
                                              args.stage_steps)
-    metric = "1080p frames/sec at 6M Gaussians (1 GPU)" if args.config == 3 and not args.gaussians else \
+    metric = "1080p frames/sec at 6M Gaussians (1 GPU)" if args.config == 3 and not args.gaussians \
+        and not args.spatial_order else \
         "%dx%d frames/sec at %d Gaussians (1 GPU)" % (inp.width, inp.height, P)
     result = base_line(metric, fps, ms_per_step, args, args.warmup, "f32", {
         "workload": "configs[%d]: %s, %d Gaussians, SH degree %d, %dx%d, RGB+depth+alpha" %

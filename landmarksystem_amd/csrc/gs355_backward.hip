@@ -69,14 +69,16 @@ struct PixelGrad {
 // blended its pair; otherwise lane s < 10 of each row returns in `sum` the row's total of accumulator s:
 // the moments of dL/dpower over the pixel offsets (dpow dx, dpow dy, dpow dx^2, dpow dx dy, dpow dy^2),
 // dL/dopacity, dL/d(r, g, b, depth).  T carries the forward blend's state (sign = finished).
+// b.y is log2(opacity) and `inv_opacity` its reciprocal: opacity * exp(power) is evaluated exactly as the forward
+// blend evaluates it (one multiply-add into the hardware exp2), so both passes take the same decisions.
 __device__ __forceinline__ bool backward_one(float& T, float& prefix, const PixelGrad& pg, float pxf, float pyf,
-                                             const float4 a, const float4 b, const float4 c, bool enabled, int sub,
-                                             float& sum)
+                                             const float4 a, const float4 b, const float4 c, float inv_opacity,
+                                             bool enabled, int sub, float& sum)
 {
     const float dx = a.x - pxf, dy = a.y - pyf;
     const float power = splat_exponent(dx, dy, a.z, a.w, b.x);
-    const float G = __expf(power);
-    const float alpha = fminf(0.99f, b.y * G);
+    const float raw = __builtin_amdgcn_exp2f(__builtin_fmaf(power, 1.4426950408889634f, b.y));  // opacity * exp(power)
+    const float alpha = fminf(0.99f, raw);
     const bool accept = enabled && !(power > 0.0f || alpha < 1.0f / 255.0f);
     const float test_T = T * (1.0f - alpha);
     const bool hit = accept && test_T >= 0.0001f;
@@ -88,8 +90,8 @@ __device__ __forceinline__ bool backward_one(float& T, float& prefix, const Pixe
         const float fg = b.z * pg.g0 + b.w * pg.g1 + c.x * pg.g2 + c.y * pg.g3;
         prefix += w * fg;
         const float dalpha = T * fg - (pg.R - prefix) * __builtin_amdgcn_rcpf(1.0f - alpha);
-        dop = G * dalpha;
-        dpow = b.y * dop;
+        dpow = raw * dalpha;  // the gradient passes through min(0.99, .) unchanged
+        dop = dpow * inv_opacity;
         T = test_T;
     }
     const float mx = dpow * dx, my = dpow * dy;
@@ -123,8 +125,9 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
     const uint32_t* __restrict__ first_key, float* __restrict__ key_grads)
 {
     __shared__ float4 s_a[256];  // px, py, conic_x, conic_y
-    __shared__ float4 s_b[256];  // conic_z, opacity, r, g
+    __shared__ float4 s_b[256];  // conic_z, log2(opacity), r, g
     __shared__ float4 s_c[256];  // b, depth, reach_x, reach_y
+    __shared__ float s_inv_opacity[256];
     __shared__ float s_grad[256 * kGradFloats];
     __shared__ uint32_t s_wave_done[4];
     __shared__ uint8_t s_list[4][4][256 + 4];
@@ -169,9 +172,12 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
         if (j < hi) {
             const uint32_t g = values[j];
             const float4* __restrict__ rec = reinterpret_cast<const float4*>(records + (size_t)g * kRecordFloats);
+            const float4 r1 = rec[1];
+            const float opacity = r1.y < 0.0f ? 0.0f : r1.y;  // as the forward blend: a negative opacity never blends
             s_a[tid] = rec[0];
-            s_b[tid] = rec[1];
+            s_b[tid] = make_float4(r1.x, __builtin_amdgcn_logf(opacity), r1.z, r1.w);
             s_c[tid] = rec[2];
+            s_inv_opacity[tid] = __builtin_amdgcn_rcpf(opacity);
             slot = key_slot(first_key[g], rects[g], tile_x, tile_y);
         }
         {
@@ -213,7 +219,8 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
                 const uint32_t kk = k_next;
                 k_next = mine[i + 1];
                 float sum;
-                if (backward_one(T, prefix, pg, pxf, pyf, s_a[kk], s_b[kk], s_c[kk], i < my_len, sub, sum)) {
+                if (backward_one(T, prefix, pg, pxf, pyf, s_a[kk], s_b[kk], s_c[kk], s_inv_opacity[kk], i < my_len, sub,
+                                 sum)) {
                     // lane s of each row adds accumulator s of the row's Gaussian
                     if (sub < 10 && i < my_len && sum != 0.0f) atomicAdd(&s_grad[kk * kGradFloats + sub], sum);
                 }

@@ -6,12 +6,13 @@
 // Blending: one 256-thread workgroup per 16x16 pixel tile, each of its four
 // wavefronts owning an 8x8 pixel quadrant, each group of 16 lanes a 4x4 block
 // of it.  The tile's depth-sorted Gaussians are staged through LDS in batches
-// of 256 records (48 B each); every 4x4 block gets its own list of the staged
-// Gaussians that can reach it, and the four lane groups of a wavefront walk
-// their lists side by side, so one pass of the pixel arithmetic serves four
-// different Gaussians.  A wavefront stops as soon as a ballot shows all of
-// its 64 pixels finished, and the workgroup stops fetching batches once all
-// four wavefronts have.
+// of 256 records (48 B each, rescaled while staging so that the per-pixel
+// arithmetic needs no constant multiplies); every 4x4 block gets its own list
+// of the staged Gaussians that can reach it, and the four lane groups of a
+// wavefront walk their lists side by side, four entries per round, so one
+// pass of the pixel arithmetic serves four different Gaussians.  A wavefront
+// stops as soon as a ballot shows all of its 64 pixels finished, and the
+// workgroup stops fetching batches once all four wavefronts have.
 #include "gs355_internal.h"
 
 namespace gs355 {
@@ -49,7 +50,14 @@ __global__ __launch_bounds__(256) void ranges_kernel(const gs355_header* __restr
 // One (pixel, Gaussian) pair: exponent, alpha, the three discrete tests and the
 // accumulation.  The exponent is evaluated with unfused multiplies and adds in
 // a fixed order (contraction is switched off for it), so the sign test and the
-// alpha threshold see the same value as a scalar evaluation of the formula.
+// alpha threshold see the same value as a scalar evaluation of the formula
+//     power = -0.5 * ((qx * dx) * dx + (qz * dy) * dy) - (qy * dx) * dy .
+// The staged record carries hx = -0.5 qx, hz = -0.5 qz and ny = -qy: scaling by a
+// power of two and negation commute with rounding, so
+//     ((hx * dx) * dx + (hz * dy) * dy) + (ny * dx) * dy
+// has the same bits with two instructions fewer.  The opacity enters through its
+// base-2 logarithm: alpha = min(0.99, exp2(power * log2(e) + log2(opacity))), one
+// multiply-add and the hardware exp2.
 //
 // A pixel's transmittance T stays >= 1e-4 while it is live, so the sign of T
 // carries the "finished" state: T > 0 live, T <= 0 finished with |T| the final
@@ -59,21 +67,22 @@ struct PixelState {
     float T, c0, c1, c2, depth;
 };
 
-__device__ __forceinline__ float splat_exponent(float dx, float dy, float qx, float qy, float qz)
+__device__ __forceinline__ float splat_exponent(float dx, float dy, float hx, float ny, float hz)
 {
 #pragma clang fp contract(off)
-    const float t1 = (qx * dx) * dx;
-    const float t2 = (qz * dy) * dy;
-    const float t3 = (qy * dx) * dy;
-    return -0.5f * (t1 + t2) - t3;
+    const float t1 = (hx * dx) * dx;
+    const float t2 = (hz * dy) * dy;
+    const float t3 = (ny * dx) * dy;
+    return (t1 + t2) + t3;
 }
 
+// a = px, py, hx, ny;  b = hz, log2(opacity), r, g;  c = b, depth, reach_x, reach_y
 __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, const float4 a, const float4 b,
                                           const float4 c)
 {
     const float dx = a.x - pxf, dy = a.y - pyf;
     const float power = splat_exponent(dx, dy, a.z, a.w, b.x);
-    const float alpha = fminf(0.99f, b.y * __expf(power));
+    const float alpha = fminf(0.99f, __builtin_amdgcn_exp2f(__builtin_fmaf(power, 1.4426950408889634f, b.y)));
     if (power > 0.0f || alpha < 1.0f / 255.0f) return;
     const float test_T = p.T * (1.0f - alpha);
     if (test_T >= 0.0001f) {
@@ -88,6 +97,9 @@ __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, c
     }
 }
 
+constexpr int kBatch = 256;            // records staged per round
+constexpr uint32_t kNullEntry = kBatch * 16;  // list entry of the null record (opacity 0: rejected by every pixel)
+
 // kCull: each wavefront first tests the staged Gaussians (one per lane) against
 // the four 4x4 blocks of its quadrant, using the bounding box of the
 // alpha >= 1/255 region from the record, and appends the survivors, in depth
@@ -95,6 +107,10 @@ __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, c
 // that is left out is one whose 16 pixels would all have taken the
 // `alpha < 1/255` branch, and every pixel still sees its Gaussians front to
 // back with the same arithmetic, so both variants produce identical images.
+// List entries are the byte offsets of the staged records (16 x record number);
+// the lists are padded with the null record to a common length that is a
+// multiple of four, so the walk needs no per-entry length test, reads four
+// entries at a time and checks for finished wavefronts once per four entries.
 template <bool kCull>
 __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_header* __restrict__ header,
                                                     const uint32_t* __restrict__ ranges,
@@ -102,12 +118,12 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
                                                     const float* __restrict__ records, float* __restrict__ image,
                                                     float* __restrict__ out_depth, float* __restrict__ out_alpha)
 {
-    __shared__ float4 s_a[256];  // px, py, conic_x, conic_y
-    __shared__ float4 s_b[256];  // conic_z, opacity, r, g
-    __shared__ float4 s_c[256];  // b, depth, reach_x, reach_y
+    __shared__ float4 s_a[kBatch + 1];  // px, py, -conic_x / 2, -conic_y          (+ the null record)
+    __shared__ float4 s_b[kBatch + 1];  // -conic_z / 2, log2(opacity), r, g
+    __shared__ float4 s_c[kBatch + 1];  // b, depth, reach_x, reach_y
     __shared__ uint32_t s_wave_done[4];
-    // per wavefront and 4x4 block: staged-record numbers of the Gaussians that can reach the block
-    __shared__ uint8_t s_list[kCull ? 4 : 1][4][256 + 4];
+    // per wavefront and 4x4 block: byte offsets of the staged records of the Gaussians that can reach the block
+    __shared__ __align__(8) uint16_t s_list[kCull ? 4 : 1][4][kBatch + 8];
 
     if (header->overflow) return;
     const int tile = blockIdx.x;
@@ -125,21 +141,36 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
 
     const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
     PixelState p = {inside ? 1.0f : -1.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (tid == 0) {  // the null record: zero conic and log2(opacity) = -inf give alpha = 0
+        s_a[kBatch] = make_float4(0.f, 0.f, 0.f, 0.f);
+        s_b[kBatch] = make_float4(0.f, -__builtin_inff(), 0.f, 0.f);
+        s_c[kBatch] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    const char* const rec_a = reinterpret_cast<const char*>(s_a);
+    const char* const rec_b = reinterpret_cast<const char*>(s_b);
+    const char* const rec_c = reinterpret_cast<const char*>(s_c);
+    auto blend_entry = [&](uint32_t entry) {
+        blend_one(p, pxf, pyf, *reinterpret_cast<const float4*>(rec_a + entry),
+                  *reinterpret_cast<const float4*>(rec_b + entry), *reinterpret_cast<const float4*>(rec_c + entry));
+    };
 
-    for (uint32_t base = lo; base < hi; base += 256) {
+    for (uint32_t base = lo; base < hi; base += kBatch) {
         const bool wave_done = __ballot(p.T > 0.0f) == 0ull;
         if (lane == 0) s_wave_done[wave] = wave_done ? 1u : 0u;
         const uint32_t j = base + tid;
         if (j < hi) {
             const uint32_t g = values[j];
             const float4* __restrict__ rec = reinterpret_cast<const float4*>(records + (size_t)g * kRecordFloats);
-            s_a[tid] = rec[0];
-            s_b[tid] = rec[1];
-            s_c[tid] = rec[2];
+            const float4 r0 = rec[0], r1 = rec[1], r2 = rec[2];
+            // a negative opacity gives a negative alpha, which every pixel rejects: log2(0) = -inf does the same
+            const float log2o = __builtin_amdgcn_logf(r1.y < 0.0f ? 0.0f : r1.y);
+            s_a[tid] = make_float4(r0.x, r0.y, -0.5f * r0.z, -r0.w);
+            s_b[tid] = make_float4(-0.5f * r1.x, log2o, r1.z, r1.w);
+            s_c[tid] = r2;
         }
         __syncthreads();
         if ((s_wave_done[0] & s_wave_done[1] & s_wave_done[2] & s_wave_done[3]) != 0u) break;
-        const int count = (int)min(256u, hi - base);
+        const int count = (int)min((uint32_t)kBatch, hi - base);
         if (!wave_done) {
             if (kCull) {
                 // ---- lists: which staged Gaussians reach which 4x4 block (lane = Gaussian) ----
@@ -160,27 +191,36 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
                     for (int b = 0; b < 4; ++b) {
                         const bool hit = ((b & 1) ? in_x1 : in_x0) && ((b >> 1) ? in_y1 : in_y0);
                         const uint64_t m = __ballot(hit);
-                        if (hit) s_list[wave][b][len[b] + (uint32_t)__popcll(m & lanes_below)] = (uint8_t)k;
+                        if (hit) s_list[wave][b][len[b] + (uint32_t)__popcll(m & lanes_below)] = (uint16_t)(k * 16);
                         len[b] += (uint32_t)__popcll(m);
                     }
                 }
+                const uint32_t longest = (uint32_t)__builtin_amdgcn_readfirstlane(
+                    (int)max(max(len[0], len[1]), max(len[2], len[3])));
+                const uint32_t quads = (longest + 3u) / 4u;
+                // pad every list with the null record up to the common length
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    for (uint32_t at = len[b] + (uint32_t)lane; at < quads * 4u; at += 64u)
+                        s_list[wave][b][at] = (uint16_t)kNullEntry;
                 // a wavefront's LDS operations execute in order: its list writes precede the reads below
                 wave_lds_sync();
-                // ---- the four lane groups walk their lists side by side ----
-                const uint32_t my_len = group == 0 ? len[0] : group == 1 ? len[1] : group == 2 ? len[2] : len[3];
-                const uint32_t longest = max(max(len[0], len[1]), max(len[2], len[3]));
-                const uint8_t* __restrict__ mine = s_list[wave][group];
-                uint32_t k_next = mine[0];  // read ahead by one entry (entries past the end are never used)
-                for (uint32_t i = 0; i < longest; ++i) {
-                    const uint32_t kk = k_next;
-                    k_next = mine[i + 1];
-                    if (i < my_len) blend_one(p, pxf, pyf, s_a[kk], s_b[kk], s_c[kk]);
+                // ---- the four lane groups walk their lists side by side, four entries per round ----
+                const uint2* __restrict__ mine = reinterpret_cast<const uint2*>(s_list[wave][group]);
+                uint2 next = mine[0];  // read ahead by one round (rounds past the end are never used)
+                for (uint32_t i = 0; i < quads; ++i) {
+                    const uint2 e = next;
+                    next = mine[i + 1];
+                    blend_entry(e.x & 0xFFFFu);
+                    blend_entry(e.x >> 16);
+                    blend_entry(e.y & 0xFFFFu);
+                    blend_entry(e.y >> 16);
                     if (__ballot(p.T > 0.0f) == 0ull) break;
                 }
             } else {
                 for (int k = 0; k < count; ++k) {
                     if (__ballot(p.T > 0.0f) == 0ull) break;
-                    blend_one(p, pxf, pyf, s_a[k], s_b[k], s_c[k]);
+                    blend_entry((uint32_t)k * 16u);
                 }
             }
         }

@@ -84,6 +84,11 @@ typedef struct gs355_gaussians {
     const float *scales;         /* [P,3] or NULL */
     const float *rotations;      /* [P,4] (r,x,y,z) or NULL */
     const float *cov3D_precomp;  /* [P,6] (xx,xy,xz,yy,yz,zz) or NULL */
+    /* Optional (NULL = unused): device u32 holding the number of Gaussians when only the device knows it (the
+     * output of gs355_decode).  The kernels then process min(P, *P_device) Gaussians, read when they run; P is the
+     * capacity the arrays are sized for and launches are sized by.  radii[i] is not written for i >= *P_device.
+     * Forward rendering only (gs355_run / gs355_render). */
+    const uint32_t *P_device;
 } gs355_gaussians;
 
 /* Outputs of forward().  image and radii are required for a full render;
@@ -251,20 +256,32 @@ GS355_API int gs355_render_backward(const gs355_frame *frame, const gs355_gaussi
                                     void *scratch, size_t scratch_bytes, const gs355_gradients *grads, void *stream);
 
 /* ---------------------------------------------------------------------------
- * Anchor decode for Scaffold-GS / Octree-GS: replaces AnchorDecoder.forward in eval mode
+ * Anchor decode for Scaffold-GS / Octree-GS: replaces AnchorDecoder.forward
  * (landmark/nerf_components/model_components/fields/anchor_decoder.py:108-242) and the kernels of its
  * fused twin (fused_anchor_decoder.py:69-244: fusedKernels.*, FusedMatmul.simple2layer -- an empty
- * third-party submodule in the reference tree).  Supported configuration: feat_dim 32, 1..10 offsets,
- * no feature bank, no level / appearance inputs (the Scaffold-GS model's, scaffold_gs/gs_model.py:126-134).
- * Heads are indexed 0 = opacity (tanh), 1 = covariance (7 per offset), 2 = colour (sigmoid). */
+ * third-party submodule in the reference tree).  Supported: feat_dim 32, 1..10 offsets, the feature bank
+ * (:163-177), the level input (:179-186) and the training-mode by-products (:239-242); not the appearance
+ * embedding (:204-211).  Heads are indexed 0 = opacity (tanh), 1 = covariance (7 per offset), 2 = colour
+ * (sigmoid). */
 typedef struct gs355_decoder {
     int32_t feat_dim;    /* 32 */
     int32_t n_offsets;   /* 1..10 */
-    int32_t in_dim[3];   /* 36 = [feat | view | dist], 35 = [feat | view] (the head's add_*_dist is False) */
+    int32_t in_dim[3];   /* 36 = [feat | view | dist], 35 = [feat | view] (the head's add_*_dist is False); with
+                            add_level every head takes [feat | view | level] (36), as the reference feeds it
+                            (anchor_decoder.py:181-182 drops the distance from both inputs) */
     const float *w0[3];  /* device f32[32, in_dim]   nn.Linear weight layout [out, in] */
     const float *b0[3];  /* device f32[32] */
     const float *w1[3];  /* device f32[k, 32], k = n_offsets, 7 n_offsets, 3 n_offsets */
     const float *b1[3];  /* device f32[k] */
+    int32_t add_level;   /* 1: the fourth extra input of the heads is anchors.level instead of the distance */
+    int32_t bank_in_dim; /* 0 = no feature bank; 3 = bank MLP on the view direction; 4 = on [view | level] */
+    const float *bank_w0; /* device f32[32, bank_in_dim]  mlp_feature_bank.0.weight */
+    const float *bank_b0; /* device f32[32] */
+    const float *bank_w1; /* device f32[3, 32]            mlp_feature_bank.2.weight (softmax over the 3 outputs) */
+    const float *bank_b1; /* device f32[3] */
+    int32_t fp32_features; /* 0: anchor features are fp16-representable (what fp16 checkpoints hold) and enter the
+                              matrix cores as one fp16 operand; 1: general fp32 features, carried as hi + lo fp16
+                              pairs (two more matrix instructions per head).  Weights are rounded to fp16 either way. */
 } gs355_decoder;
 
 typedef struct gs355_anchors {
@@ -275,6 +292,7 @@ typedef struct gs355_anchors {
     const float *scaling;        /* [A,6] (exp-activated; 0..2 scale offsets, 3..5 scale Gaussians) */
     const uint8_t *visible_mask; /* [A] 0/1 (a torch.bool tensor) */
     const float *campos;         /* device f32[3] */
+    const float *level;          /* [A] (the reference's [A,1]); required with add_level or bank_in_dim 4, else NULL */
 } gs355_anchors;
 
 typedef struct gs355_decoded {
@@ -283,6 +301,11 @@ typedef struct gs355_decoded {
     float *opacity; /* [G,1] */
     float *scaling; /* [G,3] */
     float *rot;     /* [G,4] */
+    /* gs355_decode only, each optional (NULL = not written): */
+    uint32_t *count;       /* device u32: G, the number of Gaussians the call emits (also when G > capacity) */
+    uint32_t *num_visible; /* device u32: visible anchors */
+    float *neural_opacity; /* [A_vis * n_offsets] tanh of every offset of the visible anchors (room for A * n) */
+    uint8_t *mask;         /* [A_vis * n_offsets] opacity > 0 (room for A * n) */
 } gs355_decoded;
 
 GS355_API int gs355_decode_scratch_bytes(int32_t A, size_t *bytes);
@@ -304,9 +327,22 @@ GS355_API int gs355_decode_count_static(const gs355_decoder *dec, const gs355_an
                                         uint32_t *offsets, void *stream);
 
 /* Pass 2: decode all heads and write the kept Gaussians in boolean-mask order (row-major over visible anchor,
- * offset) into outputs with room for `capacity` Gaussians. */
+ * offset) into outputs with room for `capacity` Gaussians.  The optional fields of `out` are ignored. */
 GS355_API int gs355_decode_emit(const gs355_decoder *dec, const gs355_anchors *an, const uint32_t *offsets, int64_t capacity,
                       const gs355_decoded *out, void *stream);
+
+/* The whole decode with nothing read back: count phase (feature bank, opacity head, kept offsets per run of
+ * anchors, a one-workgroup scan over the runs) and emit phase.  The outputs have room for `capacity` Gaussians
+ * (n_offsets per anchor always suffices); G stays on the device in out->count, where gs355_gaussians.P_device of
+ * the rasterizer can read it.  Gaussians beyond `capacity` are not written.  `phases`: both for one call; or the
+ * count phase alone (only out->count / out->num_visible are written), then -- after the caller has read G and
+ * sized its outputs -- the emit phase with the same decoder, anchors and workspace, untouched in between.  With a
+ * feature bank the mixed features of the visible anchors go through the workspace.  gs355_decode_count / _emit
+ * above do not support the feature bank. */
+enum { GS355_DECODE_COUNT = 1, GS355_DECODE_EMIT = 2, GS355_DECODE_ALL = 3 };
+GS355_API int gs355_decode_workspace_bytes(int32_t A, int32_t n_offsets, int32_t with_feature_bank, size_t *bytes);
+GS355_API int gs355_decode(const gs355_decoder *dec, const gs355_anchors *an, int64_t capacity, const gs355_decoded *out,
+                           void *workspace, size_t workspace_bytes, uint32_t phases, void *stream);
 
 #ifdef __cplusplus
 }

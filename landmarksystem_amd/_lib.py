@@ -17,10 +17,12 @@ STAGE_BLEND_PLAIN = 64
 STAGE_TILE_COUNT, STAGE_TILESORT, STAGE_TILE_SCATTER = 128, 256, 512
 PIPELINE_FAST = STAGE_PREPROCESS | STAGE_TILE_COUNT | STAGE_TILE_SCATTER | STAGE_TILESORT | STAGE_BLEND
 MAX_FAST_TILES = 36000
+DECODE_COUNT, DECODE_EMIT, DECODE_ALL = 1, 2, 3
 
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
            "gs355_visible_filter", "gs355_anchor_filter", "gs355_decode_scratch_bytes", "gs355_decode_count",
-           "gs355_decode_count_static", "gs355_decode_emit", "gs355_backward_scratch_bytes", "gs355_render_backward")
+           "gs355_decode_count_static", "gs355_decode_emit", "gs355_decode_workspace_bytes", "gs355_decode",
+           "gs355_backward_scratch_bytes", "gs355_render_backward")
 
 
 class Frame(C.Structure):
@@ -49,6 +51,7 @@ class Gaussians(C.Structure):
         ("scales", C.c_void_p),
         ("rotations", C.c_void_p),
         ("cov3D_precomp", C.c_void_p),
+        ("P_device", C.c_void_p),
     ]
 
 
@@ -100,6 +103,13 @@ class Decoder(C.Structure):
         ("b0", C.c_void_p * 3),
         ("w1", C.c_void_p * 3),
         ("b1", C.c_void_p * 3),
+        ("add_level", C.c_int32),
+        ("bank_in_dim", C.c_int32),
+        ("bank_w0", C.c_void_p),
+        ("bank_b0", C.c_void_p),
+        ("bank_w1", C.c_void_p),
+        ("bank_b1", C.c_void_p),
+        ("fp32_features", C.c_int32),
     ]
 
 
@@ -112,12 +122,14 @@ class Anchors(C.Structure):
         ("scaling", C.c_void_p),
         ("visible_mask", C.c_void_p),
         ("campos", C.c_void_p),
+        ("level", C.c_void_p),
     ]
 
 
 class Decoded(C.Structure):
     _fields_ = [("xyz", C.c_void_p), ("color", C.c_void_p), ("opacity", C.c_void_p), ("scaling", C.c_void_p),
-                ("rot", C.c_void_p)]
+                ("rot", C.c_void_p), ("count", C.c_void_p), ("num_visible", C.c_void_p),
+                ("neural_opacity", C.c_void_p), ("mask", C.c_void_p)]
 
 
 class AnchorLod(C.Structure):
@@ -180,6 +192,11 @@ def load() -> C.CDLL:
     lib.gs355_decode_emit.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_void_p, C.c_int64,
                                       C.POINTER(Decoded), C.c_void_p]
     lib.gs355_decode_emit.restype = C.c_int
+    lib.gs355_decode_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_size_t)]
+    lib.gs355_decode_workspace_bytes.restype = C.c_int
+    lib.gs355_decode.argtypes = [C.POINTER(Decoder), C.POINTER(Anchors), C.c_int64, C.POINTER(Decoded), C.c_void_p,
+                                 C.c_size_t, C.c_uint32, C.c_void_p]
+    lib.gs355_decode.restype = C.c_int
     lib.gs355_backward_scratch_bytes.argtypes = [C.c_int32, C.c_int64, C.POINTER(C.c_size_t)]
     lib.gs355_backward_scratch_bytes.restype = C.c_int
     lib.gs355_render_backward.argtypes = [C.POINTER(Frame), C.POINTER(Gaussians), C.c_void_p, C.c_size_t, C.c_int64,

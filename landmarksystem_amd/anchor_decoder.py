@@ -7,15 +7,22 @@ signature (:108-120) and 7-tuple result (:239-242), so the reference's
 component-swap map (`kernel_fusion_components_convert_map["AnchorDecoder"]`,
 landmark/nerf_components/components_convertor/convert_maps.py:40-47) can point
 at it.  Parameters keep the reference's names (`mlp_opacity.0.weight`, ...,
-cf. tests/test_module/test_util/test_gs_ckpt_transform.py:24-28) so its
-checkpoints load unchanged.
+`mlp_feature_bank.0.weight`, cf. tests/test_module/test_util/
+test_gs_ckpt_transform.py:24-28) so its checkpoints load unchanged.
 
-Forward only, eval mode; the configuration the Scaffold-GS model builds
-(no feature bank, no level / appearance inputs).  All arithmetic runs in the
-HIP kernels behind `gs355_decode_count` / `gs355_decode_emit`.
+Supported: the feature bank (`use_feat_bank`), the level input (`add_level`)
+and the training-mode by-products (`neural_opacity`, `mask`); not the
+appearance embedding (`appearance_dim > 0`: the reference's own branch
+concatenates a 1-D integer tensor to the 2-D input, anchor_decoder.py:204-211,
+and cannot run as written).  Forward only.  All arithmetic runs in the HIP
+kernels behind `gs355_decode`: one call enqueues the whole decode and the
+number of Gaussians stays on the device; `forward` waits for that one number
+(the reference's boolean-mask indexing synchronises at the same place) only to
+give its results their exact shapes, `decode_on_device` never waits.
 """
 import ctypes as C
-from typing import Optional
+from collections import OrderedDict
+from typing import NamedTuple, Optional
 
 import torch
 from torch import nn
@@ -32,34 +39,64 @@ def _f32c(t: torch.Tensor, device) -> torch.Tensor:
     return t.contiguous()
 
 
+class DeviceDecode(NamedTuple):
+    """Result of `decode_on_device`: tensors with room for A * n_offsets Gaussians, of which the first `count[0]`
+    are valid.  `counts` (int32[2], on the device) holds the number of Gaussians and of visible anchors."""
+    xyz: torch.Tensor
+    color: torch.Tensor
+    opacity: torch.Tensor
+    scaling: torch.Tensor
+    rot: torch.Tensor
+    counts: torch.Tensor
+    neural_opacity: Optional[torch.Tensor]
+    mask: Optional[torch.Tensor]
+
+    @property
+    def count(self) -> torch.Tensor:  # int32[1]: what the rasterizer takes as its device-side Gaussian count
+        return self.counts[0:1]
+
+
 class FusedAnchorDecoder(nn.Module):
     def __init__(self, use_feat_bank: bool, add_opacity_dist: bool, add_color_dist: bool, add_cov_dist: bool,
                  view_dim: int, feat_dim: int, n_offsets: int, appearance_dim: int = 0, add_level: bool = False,
                  dist2level: str = None):
         super().__init__()
-        if use_feat_bank or add_level or appearance_dim > 0:
-            raise NotImplementedError(
-                "FusedAnchorDecoder covers the Scaffold-GS configuration (use_feat_bank=False, add_level=False, "
-                "appearance_dim=0)")
+        if appearance_dim > 0:
+            raise NotImplementedError("FusedAnchorDecoder does not take an appearance embedding (appearance_dim=0 only)")
         if view_dim != 3 or feat_dim != 32 or not 1 <= n_offsets <= 10:
             raise NotImplementedError("FusedAnchorDecoder needs view_dim=3, feat_dim=32 and 1..10 offsets")
         self.use_feat_bank, self.add_level, self.dist2level = use_feat_bank, add_level, dist2level
         self.add_opacity_dist, self.add_color_dist, self.add_cov_dist = add_opacity_dist, add_color_dist, add_cov_dist
         self.view_dim, self.feat_dim, self.n_offsets, self.appearance_dim = view_dim, feat_dim, n_offsets, appearance_dim
+        level_dim = 1 if add_level else 0
 
         def head(with_dist: bool, outputs: int, last: Optional[nn.Module]):
-            layers = [nn.Linear(feat_dim + view_dim + (1 if with_dist else 0), feat_dim), nn.ReLU(True),
+            layers = [nn.Linear(feat_dim + view_dim + (1 if with_dist else 0) + level_dim, feat_dim), nn.ReLU(True),
                       nn.Linear(feat_dim, outputs)]
             if last is not None:
                 layers.append(last)
             return nn.Sequential(*layers)
 
+        if use_feat_bank:
+            self.mlp_feature_bank = nn.Sequential(nn.Linear(view_dim + level_dim, feat_dim), nn.ReLU(True),
+                                                  nn.Linear(feat_dim, 3), nn.Softmax(dim=1))
         self.mlp_opacity = head(add_opacity_dist, n_offsets, nn.Tanh())
         self.mlp_cov = head(add_cov_dist, 7 * n_offsets, None)
         self.mlp_color = head(add_color_dist, 3 * n_offsets, nn.Sigmoid())
-        self._scratch: Optional[torch.Tensor] = None
+        # device buffers the decoder keeps between calls, one set per stream that decoded recently (frames of
+        # different streams may be in flight together): "workspace" of gs355_decode, "block" of reused outputs
+        self._per_stream = OrderedDict()
+        self._marshalled = None  # (key, gs355_decoder struct, the tensors it points at)
+        self._host_count: Optional[torch.Tensor] = None  # pinned landing place of the device-side counts
+        self._feat_checked = None  # (identity of the last feature tensor, whether fp16 holds it exactly)
 
+    # ---- marshalling -----------------------------------------------------------------------------------------
     def _decoder_struct(self, device):
+        """The gs355_decoder record of the current parameters, rebuilt only when a parameter was replaced, moved or
+        modified in place (tensor identity and version), not per call."""
+        key = (device,) + tuple((id(p), p._version, p.data_ptr()) for p in self._parameter_list())
+        if self._marshalled is not None and self._marshalled[0] == key:
+            return self._marshalled[1]
         keep = []
         d = _lib.Decoder()
         d.feat_dim, d.n_offsets = self.feat_dim, self.n_offsets
@@ -68,48 +105,165 @@ class FusedAnchorDecoder(nn.Module):
             keep += [w0, b0, w1, b1]
             d.in_dim[j] = w0.shape[1]
             d.w0[j], d.b0[j], d.w1[j], d.b1[j] = w0.data_ptr(), b0.data_ptr(), w1.data_ptr(), b1.data_ptr()
-        return d, keep
+        d.add_level = 1 if self.add_level else 0
+        d.bank_in_dim = 0
+        if self.use_feat_bank:
+            mlp = self.mlp_feature_bank
+            w0, b0, w1, b1 = (_f32c(t, device) for t in (mlp[0].weight, mlp[0].bias, mlp[2].weight, mlp[2].bias))
+            keep += [w0, b0, w1, b1]
+            d.bank_in_dim = w0.shape[1]
+            d.bank_w0, d.bank_b0, d.bank_w1, d.bank_b1 = w0.data_ptr(), b0.data_ptr(), w1.data_ptr(), b1.data_ptr()
+        self._marshalled = (key, d, keep)
+        return d
 
-    @torch.no_grad()
-    def forward(self, camera_center, anchor, anchor_feat, offset, scaling, visible_mask=None, level=None,
-                prog_ratio=None, transition_mask=None, appearance_code=None):
-        """Returns (xyz[G,3], color[G,3], opacity[G,1], scaling[G,3], rot[G,4], None, None): the neural Gaussians of
-        the visible anchors whose decoded opacity is positive, in boolean-mask order."""
+    def _parameter_list(self):
+        mlps = [self.mlp_opacity, self.mlp_cov, self.mlp_color] + ([self.mlp_feature_bank] if self.use_feat_bank else [])
+        return [t for m in mlps for t in (m[0].weight, m[0].bias, m[2].weight, m[2].bias)]
+
+    def _check_level(self, level, A):
+        """The reference's behaviour for the level input (anchor_decoder.py:157-186): with add_level and a level
+        tensor every head is fed [feat | view | level]; anything else does not match the widths the heads were
+        built with and fails in its first matrix product."""
+        if not self.add_level:
+            return None
+        if level is None:
+            raise RuntimeError("add_level=True but no level was given: the heads are %d wide, the input without a level "
+                               "is not (the reference fails in mlp_opacity with a shape mismatch)"
+                               % self.mlp_opacity[0].weight.shape[1])
+        for name, flag in (("opacity", self.add_opacity_dist), ("cov", self.add_cov_dist), ("color", self.add_color_dist)):
+            if flag:
+                raise RuntimeError("add_level=True with add_%s_dist=True: the reference feeds [feat | view | level] "
+                                   "(36 columns, anchor_decoder.py:181-182) into a head built 37 wide and fails with a "
+                                   "shape mismatch" % name)
+        if level.numel() != A:
+            raise ValueError("level has %d elements, expected %d" % (level.numel(), A))
+        return level.reshape(-1)
+
+    # ---- decode ----------------------------------------------------------------------------------------------
+    def _marshal(self, camera_center, anchor, anchor_feat, offset, scaling, visible_mask, level):
         if not anchor.is_cuda:
             raise ValueError("anchor must be a tensor on the GPU (the decoder has no CPU path)")
         dev = anchor.device
         A = anchor.shape[0]
+        level = self._check_level(level, A)
         if visible_mask is None:
             visible_mask = torch.ones(A, dtype=torch.bool, device=dev)
         vis = visible_mask.to(device=dev, dtype=torch.bool).contiguous()
         an = _lib.Anchors()
-        tensors = dict(anchor=_f32c(anchor, dev), feat=_f32c(anchor_feat, dev), offset=_f32c(offset, dev),
-                       scaling=_f32c(scaling, dev), campos=_f32c(camera_center, dev))
+        tensors = [_f32c(anchor, dev), _f32c(anchor_feat, dev), _f32c(offset, dev), _f32c(scaling, dev),
+                   _f32c(camera_center, dev), vis]
         an.A = A
-        an.anchor, an.feat = tensors["anchor"].data_ptr(), tensors["feat"].data_ptr()
-        an.offset, an.scaling = tensors["offset"].data_ptr(), tensors["scaling"].data_ptr()
-        an.visible_mask, an.campos = vis.data_ptr(), tensors["campos"].data_ptr()
-        dec, keep = self._decoder_struct(dev)
-        lib = _lib.load()
-        stream = torch.cuda.current_stream(dev).cuda_stream
-
+        an.anchor, an.feat, an.offset, an.scaling = (t.data_ptr() for t in tensors[:4])
+        an.campos, an.visible_mask = tensors[4].data_ptr(), vis.data_ptr()
+        if level is not None:
+            tensors.append(_f32c(level, dev))
+            an.level = tensors[-1].data_ptr()
+        dec = self._decoder_struct(dev)
+        # features that fp16 cannot hold exactly (fp32-trained checkpoints) go through the matrix cores as hi + lo
+        # pairs; checked once per feature tensor, not per frame
+        feat_key = (id(anchor_feat), anchor_feat._version, anchor_feat.data_ptr(), tuple(anchor_feat.shape))
+        if self._feat_checked is None or self._feat_checked[0] != feat_key:
+            f32 = tensors[1]
+            self._feat_checked = (feat_key, bool(torch.equal(f32.half().float(), f32)))
+        dec.fp32_features = 0 if self._feat_checked[1] else 1
         need = C.c_size_t()
-        _lib.check(lib.gs355_decode_scratch_bytes(A, C.byref(need)))
-        if self._scratch is None or self._scratch.device != dev or self._scratch.numel() < need.value:
-            self._scratch = torch.empty(need.value, dtype=torch.uint8, device=dev)
-        counts = torch.empty(max(A, 1), dtype=torch.int32, device=dev)
-        offsets = torch.empty(max(A, 1), dtype=torch.int32, device=dev)
-        _lib.check(lib.gs355_decode_count(C.byref(dec), C.byref(an), counts.data_ptr(), offsets.data_ptr(),
-                                          self._scratch.data_ptr(), self._scratch.numel(), stream))
-        # the output shapes depend on the data: one read-back, as the reference's boolean-mask indexing does
-        G = int((offsets[A - 1] + counts[A - 1]).item()) if A > 0 else 0
-        out = dict(xyz=torch.empty((G, 3), device=dev), color=torch.empty((G, 3), device=dev),
-                   opacity=torch.empty((G, 1), device=dev), scaling=torch.empty((G, 3), device=dev),
-                   rot=torch.empty((G, 4), device=dev))
-        if G > 0:
-            o = _lib.Decoded()
-            o.xyz, o.color, o.opacity = out["xyz"].data_ptr(), out["color"].data_ptr(), out["opacity"].data_ptr()
-            o.scaling, o.rot = out["scaling"].data_ptr(), out["rot"].data_ptr()
-            _lib.check(lib.gs355_decode_emit(C.byref(dec), C.byref(an), offsets.data_ptr(), G, C.byref(o), stream))
-        del keep
-        return out["xyz"], out["color"], out["opacity"], out["scaling"], out["rot"], None, None
+        _lib.check(_lib.load().gs355_decode_workspace_bytes(A, self.n_offsets, 1 if self.use_feat_bank else 0,
+                                                            C.byref(need)))
+        kept = self._kept(dev)
+        if kept.get("workspace") is None or kept["workspace"].numel() < need.value:
+            kept["workspace"] = torch.empty(max(need.value, 256), dtype=torch.uint8, device=dev)
+        return dev, A, dec, an, tensors
+
+    def _kept(self, dev):
+        key = (dev, torch.cuda.current_stream(dev).cuda_stream)
+        kept = self._per_stream.get(key)
+        if kept is None:
+            kept = self._per_stream[key] = {}
+            while len(self._per_stream) > 4:
+                self._per_stream.popitem(last=False)
+        else:
+            self._per_stream.move_to_end(key)
+        return kept
+
+    def _run(self, dec, an, capacity, o, phases, dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        ws = self._kept(dev)["workspace"]
+        _lib.check(_lib.load().gs355_decode(C.byref(dec), C.byref(an), int(capacity), C.byref(o), ws.data_ptr(),
+                                            ws.numel(), int(phases), stream))
+
+    @torch.no_grad()
+    def decode_on_device(self, camera_center, anchor, anchor_feat, offset, scaling, visible_mask=None, level=None,
+                         want_training_outputs: bool = False, reuse_buffers: bool = False) -> DeviceDecode:
+        """The whole decode enqueued on the current stream, nothing read back.  Outputs have room for
+        A * n_offsets Gaussians; `counts` says how many are valid.  `reuse_buffers`: the outputs live in one block
+        the decoder keeps and overwrites at its next call (a render loop that consumes them at once pays no
+        per-frame allocation of the capacity-sized block)."""
+        dev, A, dec, an, tensors = self._marshal(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, level)
+        n = self.n_offsets
+        cap = A * n
+        # one block for the five outputs (14 floats per Gaussian) and the two counters, carved into views
+        kept = self._kept(dev)
+        if reuse_buffers and kept.get("block") is not None and kept["block"][0] == cap:
+            res = kept["block"][1]
+        else:
+            block = torch.empty(cap * 14 + 2, dtype=torch.float32, device=dev)
+            cut = lambda first, width: block[first * cap:(first + width) * cap].view(cap, width)  # noqa: E731
+            res = DeviceDecode(cut(0, 3), cut(3, 3), cut(6, 1), cut(7, 3), cut(10, 4), block[cap * 14:].view(torch.int32),
+                               None, None)
+            kept["block"] = (cap, res) if reuse_buffers else None
+        if want_training_outputs:
+            res = res._replace(neural_opacity=torch.empty((cap, 1), dtype=torch.float32, device=dev),
+                               mask=torch.empty(cap, dtype=torch.bool, device=dev))
+        o = _lib.Decoded()
+        if cap > 0:
+            o.xyz, o.color, o.opacity = res.xyz.data_ptr(), res.color.data_ptr(), res.opacity.data_ptr()
+            o.scaling, o.rot = res.scaling.data_ptr(), res.rot.data_ptr()
+            if want_training_outputs:
+                o.neural_opacity, o.mask = res.neural_opacity.data_ptr(), res.mask.data_ptr()
+        o.count, o.num_visible = res.counts.data_ptr(), res.counts.data_ptr() + 4
+        self._run(dec, an, cap, o, _lib.DECODE_ALL, dev)
+        del tensors  # torch's allocator keeps their memory alive for the work already enqueued on this stream
+        return res
+
+    def read_counts(self, res):
+        """(G, visible anchors) from the device-side counters of a decode: one 8-byte copy to pinned memory, waited
+        for.  `res`: a `decode_on_device` result or the int32[2] counter tensor."""
+        counts = res.counts if isinstance(res, DeviceDecode) else res
+        if self._host_count is None:
+            self._host_count = torch.zeros(2, dtype=torch.int32, pin_memory=True)
+        self._host_count.copy_(counts, non_blocking=True)
+        torch.cuda.current_stream(counts.device).synchronize()
+        return int(self._host_count[0]), int(self._host_count[1])
+
+    @torch.no_grad()
+    def forward(self, camera_center, anchor, anchor_feat, offset, scaling, visible_mask=None, level=None,
+                prog_ratio=None, transition_mask=None, appearance_code=None):
+        """Returns (xyz[G,3], color[G,3], opacity[G,1], scaling[G,3], rot[G,4], neural_opacity, mask): the neural
+        Gaussians of the visible anchors whose decoded opacity is positive, in boolean-mask order; in training mode
+        also the opacity of every offset of the visible anchors ([A_vis * n, 1]) and the mask over them, else None.
+
+        The output shapes depend on the data, so the count phase runs first and its two counters are read back
+        (the reference's boolean-mask indexing synchronises at the same place); the emit phase then writes into
+        tensors of exactly that size."""
+        if self.dist2level == "progressive" and prog_ratio is not None and transition_mask is not None:
+            raise NotImplementedError("progressive level-of-detail opacity scaling is not part of this decoder")
+        dev, A, dec, an, tensors = self._marshal(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, level)
+        counts = torch.empty(2, dtype=torch.int32, device=dev)
+        o = _lib.Decoded()
+        o.count, o.num_visible = counts.data_ptr(), counts.data_ptr() + 4
+        self._run(dec, an, 0, o, _lib.DECODE_COUNT, dev)
+        G, a_vis = self.read_counts(counts)
+        f = lambda *shape: torch.empty(shape, dtype=torch.float32, device=dev)  # noqa: E731
+        out = (f(G, 3), f(G, 3), f(G, 1), f(G, 3), f(G, 4))
+        extra = (None, None)
+        if self.training:
+            extra = (f(a_vis * self.n_offsets, 1), torch.empty(a_vis * self.n_offsets, dtype=torch.bool, device=dev))
+        if G > 0 or (self.training and a_vis > 0):
+            if G > 0:
+                o.xyz, o.color, o.opacity, o.scaling, o.rot = (t.data_ptr() for t in out)
+            if self.training and a_vis > 0:
+                o.neural_opacity, o.mask = extra[0].data_ptr(), extra[1].data_ptr()
+            o.count = o.num_visible = None
+            self._run(dec, an, G, o, _lib.DECODE_EMIT, dev)
+        del tensors
+        return out + extra

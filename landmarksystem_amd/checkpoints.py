@@ -276,13 +276,20 @@ def _decoder_state(state: Mapping[str, torch.Tensor]) -> Dict[str, torch.Tensor]
     return {k[len(pre):]: v for k, v in state.items() if k.startswith(pre)}
 
 
-def _decoder_kwargs(dec: Mapping[str, torch.Tensor], n_offsets: int, feat_dim: int) -> Dict[str, bool]:
-    # the first layer's width tells whether the camera distance is appended: feat + view(3) [+ dist(1)]
+def _decoder_kwargs(dec: Mapping[str, torch.Tensor], n_offsets: int, feat_dim: int, add_level: bool = False) -> Dict[str, bool]:
+    # the first layer's width tells whether the camera distance is appended: feat + view(3) [+ dist(1)] [+ level(1)];
+    # a feature bank shows as its own MLP, whose input width tells whether it takes the level
     out = {}
+    bank = dec.get("mlp_feature_bank.0.weight")
+    if bank is not None:
+        out["use_feat_bank"] = True
+        add_level = add_level or bank.shape[1] == 4
+    if add_level:
+        out["add_level"] = True
     for head in ("opacity", "cov", "color"):
         w = dec.get("mlp_%s.0.weight" % head)
         if w is not None:
-            out["add_%s_dist" % head] = bool(w.shape[1] == feat_dim + 4)
+            out["add_%s_dist" % head] = bool(w.shape[1] == feat_dim + 4 + (1 if add_level else 0))
     return out
 
 
@@ -337,7 +344,7 @@ def load_octree_gs(path, device="cuda", spatial_order: bool = False, **kw):
         _reorder(s, "_anchor")
     dec = _decoder_state(load_mlp_state(os.path.dirname(os.path.abspath(ply)), device))
     n_offsets, feat_dim = s["_offset"].shape[1], s["_anchor_feat"].shape[1]
-    kw = {**_decoder_kwargs(dec, n_offsets, feat_dim), **kw}
+    kw = {**_decoder_kwargs(dec, n_offsets, feat_dim, bool(kw.get("add_level", False))), **kw}
     m = OctreeGS(s["_anchor"], s["_anchor_feat"], s["_offset"], s["_scaling"], s["_rotation"], s["_level"],
                  voxel_size, standard_dist, extra_level=s["_extra_level"], opacity=s["_opacity"],
                  n_offsets=n_offsets, feat_dim=feat_dim, **kw)

@@ -163,6 +163,7 @@ FrameArgs make_args(const gs355_frame* f)
     a.projmatrix = f->projmatrix;
     a.campos = f->campos;
     a.bg = f->bg;
+    a.p_device = nullptr;
     return a;
 }
 
@@ -226,13 +227,14 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     auto* bin_visible = reinterpret_cast<uint32_t*>(ws + L.bin_visible);
     auto* tile_lists = reinterpret_cast<uint32_t*>(ws + L.tile_lists);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const FrameArgs fa = make_args(frame);
+    FrameArgs fa = make_args(frame);
+    fa.p_device = g->P_device;
     const uint32_t cap = (uint32_t)n_cap;
 
     if (stage_mask & GS355_STAGE_PREPROCESS)
         if ((rc = launch_preprocess(fa, *g, false, records, touched, rects, depth_bits, out->radii, s))) return rc;
     if (stage_mask & GS355_STAGE_SCAN)
-        if ((rc = launch_scan_offsets(touched, out->radii, g->P, offsets, scan_tmp, header, cap, s))) return rc;
+        if ((rc = launch_scan_offsets(touched, out->radii, g->P, g->P_device, offsets, scan_tmp, header, cap, s))) return rc;
     if (stage_mask & GS355_STAGE_DUPLICATE)
         if ((rc = launch_duplicate(fa, g->P, records, out->radii, offsets, header, keys[0], vals[0], s))) return rc;
     if (stage_mask & GS355_STAGE_SORT)
@@ -275,6 +277,7 @@ int gs355_visible_filter(const gs355_frame* frame, const gs355_gaussians* g, int
     if ((rc = check_frame(frame, false))) return rc;
     if ((rc = check_geometry_inputs(g))) return rc;
     if (g->P > 0 && !radii) return set_error(GS355_EINVAL, "radii is NULL");
+    if (g->P_device) return set_error(GS355_EINVAL, "visible_filter does not take a device-side Gaussian count");
     const FrameArgs fa = make_args(frame);
     return launch_preprocess(fa, *g, true, nullptr, nullptr, nullptr, nullptr, radii, static_cast<hipStream_t>(stream));
 }
@@ -315,6 +318,7 @@ int gs355_render_backward(const gs355_frame* frame, const gs355_gaussians* g, co
     if ((rc = check_frame(frame, true))) return rc;
     if ((rc = check_geometry_inputs(g))) return rc;
     if ((rc = check_colour_inputs(frame, g))) return rc;
+    if (g->P_device) return set_error(GS355_EINVAL, "the backward pass does not take a device-side Gaussian count");
     if (!in) return set_error(GS355_EINVAL, "backward inputs is NULL");
     if (!grads) return set_error(GS355_EINVAL, "gradients is NULL");
     if (!in->image || !in->dL_dimage) return set_error(GS355_EINVAL, "image / dL_dimage is NULL");
@@ -359,6 +363,7 @@ int gs355_anchor_filter(const gs355_frame* frame, const gs355_gaussians* anchors
     if ((rc = check_frame(frame, false))) return rc;
     if ((rc = check_geometry_inputs(anchors))) return rc;
     if (scale_stride < 3) return set_error(GS355_EINVAL, "scale_stride must be >= 3 (got %d)", scale_stride);
+    if (anchors->P_device) return set_error(GS355_EINVAL, "the anchor filter does not take a device-side count");
     if (anchors->P > 0 && !visible) return set_error(GS355_EINVAL, "visible is NULL");
     FilterArgs x;
     x.scale_stride = scale_stride;

@@ -48,12 +48,17 @@ __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P
     __shared__ uint32_t s_nqueue, s_visible;
 
     if (kScatter && header->overflow) return;
+    if (f.p_device) {  // the slices follow the device-side count: as many Gaussians per workgroup as on the host side
+        P = effective_count(f, P);
+        per_group = (P + (int)gridDim.x - 1) / (int)gridDim.x;
+        per_group = max(kBinThreads, (per_group + kBinThreads - 1) / kBinThreads * kBinThreads);
+    }
     const int T = f.grid_x * f.grid_y;
     const int tid = threadIdx.x, c = blockIdx.x;
     uint32_t* __restrict__ row = matrix + (size_t)c * T;
     for (int t = tid; t < T; t += kBinThreads) s_tile[t] = kScatter ? tile_base[t] + row[t] : 0u;
     if (tid == 0) s_visible = 0;
-    const int g_begin = c * per_group;
+    const int g_begin = min(P, c * per_group);
     const int g_end = min(P, g_begin + per_group);
     uint32_t visible = 0;
 

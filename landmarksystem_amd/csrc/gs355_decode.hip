@@ -54,10 +54,19 @@ struct DecodeArgs {
     const float* scaling;
     const uint8_t* visible;
     const float* campos;
+    const float* level;  // per-anchor level: the fourth fp32-only input instead of the distance (add_level), or NULL
+    int split_feat;      // features enter as hi + lo fp16 pairs (fp32 features that fp16 cannot represent)
     const float* w0[3];
     const float* b0[3];
     const float* w1[3];
     const float* b1[3];
+    // one-call decode (gs355_decode): the count pass leaves per-run totals behind, a one-workgroup scan turns
+    // them into run bases, and the emit pass (which recomputes the opacity head: matrix instructions are cheap
+    // here, registers and memory requests are not) places its Gaussians from those instead of per-anchor offsets
+    uint2* run_totals;       // [runs] (kept offsets, visible anchors) per run of kRun anchors, or NULL
+    const uint2* run_base;   // [runs] exclusive prefix of run_totals, or NULL
+    float* neural_opacity;   // [A_vis * n] tanh of every pre-activation, in visible-anchor order, or NULL
+    uint8_t* kept_mask;      // [A_vis * n] pre-activation > 0, or NULL
 };
 
 __device__ __forceinline__ half8_t to_half8(const float v[8])
@@ -124,14 +133,18 @@ __device__ __forceinline__ void load_head(const DecodeArgs& d, int head, int out
 
 // One head for one tile of 32 anchors: returns up to kTiles accumulators of the
 // second layer (rows = outputs 32r + 8b + 4*half + t, column = this lane's anchor).
-template <int kTiles>
+template <int kTiles, bool kSplit>
 __device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const float* bias0, const float* bias1,
-                                         const half8_t X[3], int half, floatx16 out[kTiles])
+                                         const half8_t X[kSplit ? 5 : 3], int half, floatx16 out[kTiles])
 {
-    // layer 1: hidden = W0 [32 x in] * X^T + b0
+    // layer 1: hidden = W0 [32 x in] * X^T + b0  (X[3], X[4]: the low parts of features that fp16 cannot hold)
     floatx16 h = bias_rows(bias0, 0, half);
 #pragma unroll
     for (int s = 0; s < 3; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w0[s], X[s], h, 0, 0, 0);
+    if constexpr (kSplit) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w0[s], X[3 + s], h, 0, 0, 0);
+    }
     // ReLU, then hi/lo split: registers 8s..8s+7 are the B operand of k-step s
     half8_t hh[2], hl[2];
 #pragma unroll
@@ -176,6 +189,7 @@ struct TileInputs {
     float4 f[4] = {};          // features 16s + 8*half .. +7 in f[2s], f[2s+1], s = 0..1
     float pos[3] = {0.f, 0.f, 0.f};
     float sc3[3] = {0.f, 0.f, 0.f};
+    float extra = 0.f;  // the anchor's level when it replaces the distance
     uint32_t first_slot = 0;
     float ofv[kCountOnly ? 1 : 5][3] = {};
 };
@@ -184,7 +198,8 @@ struct TileInputs {
 // and runs the MLPs on those only: the work follows the number of visible anchors, not of anchors.
 constexpr int kRun = 128;
 
-template <bool kCountOnly>
+// kSplit: the features enter as hi + lo fp16 pairs (general fp32 features; two more matrix instructions per head).
+template <bool kCountOnly, bool kSplit>
 __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
                                                      const uint32_t* __restrict__ offsets, uint32_t capacity,
                                                      float* __restrict__ xyz, float* __restrict__ color,
@@ -237,11 +252,23 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
       const bool v0 = a0 < d.A && d.visible[a0] != 0, v1 = a1 < d.A && d.visible[a1] != 0;
       const uint64_t m0 = __ballot(v0), m1 = __ballot(v1);
       const int n0 = __popcll(m0), nvis = n0 + __popcll(m1);
-      if (kCountOnly) {  // anchors that are not decoded keep nothing
+      if (kCountOnly && counts) {  // anchors that are not decoded keep nothing
           if (!v0 && a0 < d.A) counts[a0] = 0;
           if (!v1 && a1 < d.A) counts[a1] = 0;
       }
-      if (nvis == 0) continue;  // uniform
+      if (nvis == 0) {  // uniform
+          if (kCountOnly && d.run_totals && lane == 0) d.run_totals[run] = make_uint2(0u, 0u);
+          continue;
+      }
+      uint32_t run_kept = 0;  // count pass: this lane's share of the run's kept offsets
+      // emit pass of the one-call decode: the run's first output slot, advanced tile by tile (uniform), and the
+      // rank of its first visible anchor among all visible anchors
+      uint32_t run_slot = 0, run_rank = 0;
+      if (!kCountOnly && d.run_base) {
+          const uint2 rb = d.run_base[run];
+          run_slot = rb.x;
+          run_rank = rb.y;
+      }
       if (v0) run_list[__popcll(m0 & lanes_below)] = (uint8_t)lane;
       if (v1) run_list[n0 + __popcll(m1 & lanes_below)] = (uint8_t)(64 + lane);
       wave_lds_sync();
@@ -260,6 +287,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
             }
 #pragma unroll
             for (int k = 0; k < 3; ++k) in.pos[k] = d.anchor[3 * (size_t)a + k];
+            if (d.level) in.extra = d.level[a];
         }
         if constexpr (!kCountOnly) {
             // half 0: scaling[0..2] (offset scale), half 1: scaling[3..5] (Gaussian scale)
@@ -267,7 +295,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
 #pragma unroll
                 for (int k = 0; k < 3; ++k) in.sc3[k] = d.scaling[6 * (size_t)a + 3 * half + k];
             }
-            if (vis) in.first_slot = offsets[a];  // entry 0's value is the tile's first output slot
+            if (vis && offsets) in.first_slot = offsets[a];  // entry 0's value is the tile's first output slot
             // the learned offsets of the items this lane's position covers (item = entry * n + offset)
 #pragma unroll
             for (int r = 0; r < 5; ++r) {
@@ -281,7 +309,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
             }
         }
         // B operand: X^T, column = anchor; slots as described at HeadWeights
-        half8_t X[3];
+        half8_t X[kSplit ? 5 : 3];
         const float ax = in.pos[0], ay = in.pos[1], az = in.pos[2];
         {
             float x8[8];
@@ -290,6 +318,11 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
                 x8[0] = in.f[2 * s].x, x8[1] = in.f[2 * s].y, x8[2] = in.f[2 * s].z, x8[3] = in.f[2 * s].w;
                 x8[4] = in.f[2 * s + 1].x, x8[5] = in.f[2 * s + 1].y, x8[6] = in.f[2 * s + 1].z, x8[7] = in.f[2 * s + 1].w;
                 X[s] = to_half8(x8);  // all zero for an invisible anchor
+                if constexpr (kSplit) {  // what the fp16 rounding left over, as a second operand
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) x8[j] -= (float)X[s][j];
+                    X[3 + s] = to_half8(x8);
+                }
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) x8[j] = 0.0f;
@@ -299,7 +332,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
                 vx /= dist;
                 vy /= dist;
                 vz /= dist;
-                const float in4[4] = {vx, vy, vz, dist};
+                const float in4[4] = {vx, vy, vz, d.level ? in.extra : dist};
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const _Float16 top = (_Float16)in4[t];
@@ -311,17 +344,20 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         }
 
         // ---- opacity head ----
-        floatx16 op[1];
-        run_head<1>(w_op, s_bias, s_bias + 96, X, half, op);
         // the mask opacity > 0 is the sign of the pre-activation (tanh is odd, monotone and tanh(x) = x for the
         // smallest floats), so tanh itself is only evaluated for the offsets that are kept
-        store_rows(mine + col * stride, 0, n, 0, half, op[0]);
+        {
+            floatx16 op[1];
+            run_head<1, kSplit>(w_op, s_bias, s_bias + 96, X, half, op);
+            store_rows(mine + col * stride, 0, n, 0, half, op[0]);
+        }
         if (kCountOnly) {
             wave_lds_sync();
             if (half == 0 && vis) {
                 uint32_t kept = 0;
                 for (int m = 0; m < n; ++m) kept += mine[col * stride + m] > 0.0f ? 1u : 0u;
-                counts[a] = kept;
+                if (counts) counts[a] = kept;
+                run_kept += kept;
             }
             wave_lds_sync();
             continue;
@@ -329,11 +365,11 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
 
         // ---- covariance and colour heads ----
         floatx16 cv[3];
-        run_head<3>(w_cov, s_bias + 32, s_bias + 128, X, half, cv);
+        run_head<3, kSplit>(w_cov, s_bias + 32, s_bias + 128, X, half, cv);
 #pragma unroll
         for (int r = 0; r < 3; ++r) store_rows(mine + col * stride, n, 7 * n, 32 * r, half, cv[r]);
         floatx16 cl[1];
-        run_head<1>(w_col, s_bias + 64, s_bias + 224, X, half, cl);
+        run_head<1, kSplit>(w_col, s_bias + 64, s_bias + 224, X, half, cl);
         store_rows(mine + col * stride, 8 * n, 3 * n, 0, half, cl[0]);
         {
             float* __restrict__ extra = mine + col * stride + 11 * n;
@@ -371,7 +407,24 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         // the survivors of a tile occupy consecutive output slots from the slot of its first anchor: lanes write
         // consecutive addresses.  No global reads in here: the learned offsets sit in registers of the lane that
         // requested them (item = round * 64 + lane) and are fetched across lanes.
-        const uint32_t tile_slot = reinterpret_cast<const uint32_t*>(mine)[11 * n + 9];
+        const uint32_t tile_slot = d.run_base ? run_slot : reinterpret_cast<const uint32_t*>(mine)[11 * n + 9];
+        run_slot += total;
+        // training-mode by-products: tanh of every pre-activation of the visible anchors and the mask, indexed by
+        // (visible anchor, offset): the tile's entries are the run's visible anchors first .. first + 31
+        if (d.neural_opacity || d.kept_mask) {
+            const size_t row0 = ((size_t)run_rank + (size_t)first) * (size_t)n;
+#pragma unroll
+            for (int r = 0; r < 5; ++r) {
+                const int it = r * 64 + lane;
+                if (it >= items) break;
+                const int al = (it * inv_n) >> 16, m = it - al * n;
+                if ((any >> al) & 1ull) {
+                    const float v = mine[al * stride + m];
+                    if (d.neural_opacity) d.neural_opacity[row0 + (size_t)it] = tanhf(v);
+                    if (d.kept_mask) d.kept_mask[row0 + (size_t)it] = v > 0.0f ? 1 : 0;
+                }
+            }
+        }
         for (uint32_t s0 = 0; s0 < total; s0 += 64) {  // uniform
             const uint32_t s = s0 + lane;
             const bool live = s < total;
@@ -408,6 +461,123 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         }
         wave_lds_sync();
       }
+      if (kCountOnly && d.run_totals) {  // the run's totals: kept offsets (summed over the lanes), visible anchors
+          uint32_t t = run_kept;
+#pragma unroll
+          for (int off = 32; off > 0; off >>= 1) t += (uint32_t)__shfl_xor((int)t, off, 64);
+          if (lane == 0) d.run_totals[run] = make_uint2(t, (uint32_t)nvis);
+      }
+    }
+}
+
+// One workgroup: exclusive prefix of the per-run totals (kept offsets, visible anchors) and the grand totals.
+__global__ __launch_bounds__(1024) void run_scan_kernel(const uint2* __restrict__ totals, uint2* __restrict__ base,
+                                                        uint32_t runs, uint32_t* __restrict__ num_emitted,
+                                                        uint32_t* __restrict__ num_visible)
+{
+    __shared__ uint2 s_wave[16];
+    __shared__ uint2 s_carry;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) s_carry = make_uint2(0u, 0u);
+    __syncthreads();
+    for (uint32_t first = 0; first < runs; first += 1024) {
+        const uint32_t j = first + threadIdx.x;
+        const uint2 v = j < runs ? totals[j] : make_uint2(0u, 0u);
+        uint32_t ix = v.x, iy = v.y;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t ux = (uint32_t)__shfl_up((int)ix, d, 64), uy = (uint32_t)__shfl_up((int)iy, d, 64);
+            if (lane >= d) {
+                ix += ux;
+                iy += uy;
+            }
+        }
+        if (lane == 63) s_wave[wave] = make_uint2(ix, iy);
+        __syncthreads();
+        uint2 before = s_carry;
+        for (int w = 0; w < wave; ++w) {
+            before.x += s_wave[w].x;
+            before.y += s_wave[w].y;
+        }
+        if (j < runs) base[j] = make_uint2(before.x + ix - v.x, before.y + iy - v.y);
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = make_uint2(before.x + ix, before.y + iy);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        if (num_emitted) *num_emitted = s_carry.x;
+        if (num_visible) *num_visible = s_carry.y;
+    }
+}
+
+// Feature bank (anchor_decoder.py:163-177): a small MLP of the view direction (and the level) gives three softmax
+// weights per anchor that mix the feature vector with its 4x and 2x strided copies:
+//     feat'[j] = feat[4 (j mod 8)] w0 + feat[2 (j mod 16)] w1 + feat[j] w2 .
+// One thread per visible anchor, fp32 throughout; the decode then reads the mixed features.
+struct BankArgs {
+    int A, in_dim;  // 3 = view direction, 4 = view direction and level
+    const float* anchor;
+    const float* feat;
+    const uint8_t* visible;
+    const float* campos;
+    const float* level;
+    const float* w0;  // [32, in_dim]
+    const float* b0;  // [32]
+    const float* w1;  // [3, 32]
+    const float* b1;  // [3]
+    float* mixed;     // [A, 32]
+};
+
+__global__ __launch_bounds__(256) void feature_bank_kernel(BankArgs k)
+{
+    __shared__ float s_w0[kFeat * 4], s_b0[kFeat], s_w1[3 * kFeat], s_b1[3];
+    for (int t = threadIdx.x; t < kFeat * k.in_dim; t += 256) s_w0[t] = k.w0[t];
+    for (int t = threadIdx.x; t < 3 * kFeat; t += 256) s_w1[t] = k.w1[t];
+    if (threadIdx.x < kFeat) s_b0[threadIdx.x] = k.b0[threadIdx.x];
+    if (threadIdx.x < 3) s_b1[threadIdx.x] = k.b1[threadIdx.x];
+    __syncthreads();
+    const int a = blockIdx.x * 256 + threadIdx.x;
+    if (a >= k.A || k.visible[a] == 0) return;
+    float in[4];
+    {
+        float vx = k.anchor[3 * (size_t)a] - k.campos[0], vy = k.anchor[3 * (size_t)a + 1] - k.campos[1],
+              vz = k.anchor[3 * (size_t)a + 2] - k.campos[2];
+        const float dist = sqrtf(vx * vx + vy * vy + vz * vz);
+        in[0] = vx / dist;
+        in[1] = vy / dist;
+        in[2] = vz / dist;
+        in[3] = k.in_dim > 3 ? k.level[a] : 0.0f;
+    }
+    float logit[3] = {s_b1[0], s_b1[1], s_b1[2]};
+    for (int h = 0; h < kFeat; ++h) {
+        float v = s_b0[h];
+        for (int c = 0; c < k.in_dim; ++c) v += s_w0[h * k.in_dim + c] * in[c];
+        v = fmaxf(v, 0.0f);
+#pragma unroll
+        for (int o = 0; o < 3; ++o) logit[o] += s_w1[o * kFeat + h] * v;
+    }
+    const float top = fmaxf(logit[0], fmaxf(logit[1], logit[2]));
+    float w[3] = {expf(logit[0] - top), expf(logit[1] - top), expf(logit[2] - top)};
+    const float sum = w[0] + w[1] + w[2];
+#pragma unroll
+    for (int o = 0; o < 3; ++o) w[o] /= sum;
+    float f[kFeat];
+    const float4* __restrict__ src = reinterpret_cast<const float4*>(k.feat + (size_t)a * kFeat);
+#pragma unroll
+    for (int q = 0; q < kFeat / 4; ++q) {
+        const float4 v = src[q];
+        f[4 * q] = v.x, f[4 * q + 1] = v.y, f[4 * q + 2] = v.z, f[4 * q + 3] = v.w;
+    }
+    float4* __restrict__ dst = reinterpret_cast<float4*>(k.mixed + (size_t)a * kFeat);
+#pragma unroll
+    for (int q = 0; q < kFeat / 4; ++q) {
+        float o4[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int j = 4 * q + t;
+            o4[t] = f[4 * (j % 8)] * w[0] + f[2 * (j % 16)] * w[1] + f[j] * w[2];
+        }
+        dst[q] = make_float4(o4[0], o4[1], o4[2], o4[3]);
     }
 }
 
@@ -417,7 +587,7 @@ struct DecodeLaunch {
     DecodeArgs args;
 };
 
-static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, DecodeArgs* out)
+static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, bool allow_bank, DecodeArgs* out)
 {
     if (!dec || !an) return set_error(GS355_EINVAL, "decoder / anchors is NULL");
     if (dec->feat_dim != kFeat)
@@ -426,13 +596,30 @@ static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, DecodeAr
         return set_error(GS355_EINVAL, "anchor decode supports 1..10 offsets per anchor (got %d)", dec->n_offsets);
     if (an->A < 0) return set_error(GS355_EINVAL, "A must be >= 0 (got %d)", an->A);
     for (int j = 0; j < 3; ++j) {
-        if (dec->in_dim[j] != kFeat + 3 && dec->in_dim[j] != kFeat + 4)
+        if (dec->add_level) {
+            // the reference concatenates [feat | view | level] for every head once a level is given
+            // (anchor_decoder.py:181-182), so a head built with a distance column as well cannot be fed
+            if (dec->in_dim[j] != kFeat + 4)
+                return set_error(GS355_EINVAL, "head %d: with add_level the input is [feat | view | level], 36 wide "
+                                 "(got %d; a head with add_*_dist expects a width the reference never provides)",
+                                 j, dec->in_dim[j]);
+        } else if (dec->in_dim[j] != kFeat + 3 && dec->in_dim[j] != kFeat + 4) {
             return set_error(GS355_EINVAL, "head %d: input width must be 35 or 36 (got %d)", j, dec->in_dim[j]);
+        }
         if (!dec->w0[j] || !dec->b0[j] || !dec->w1[j] || !dec->b1[j])
             return set_error(GS355_EINVAL, "head %d: weight or bias pointer is NULL", j);
     }
+    if (dec->bank_in_dim != 0) {
+        if (!allow_bank) return set_error(GS355_EINVAL, "the feature bank is supported by gs355_decode only");
+        if (dec->bank_in_dim != 3 && dec->bank_in_dim != 4)
+            return set_error(GS355_EINVAL, "bank_in_dim must be 0, 3 or 4 (got %d)", dec->bank_in_dim);
+        if (!dec->bank_w0 || !dec->bank_b0 || !dec->bank_w1 || !dec->bank_b1)
+            return set_error(GS355_EINVAL, "feature bank: weight or bias pointer is NULL");
+    }
     if (an->A > 0 && (!an->anchor || !an->feat || !an->offset || !an->scaling || !an->visible_mask || !an->campos))
         return set_error(GS355_EINVAL, "anchor inputs must all be non-NULL");
+    if (an->A > 0 && (dec->add_level || dec->bank_in_dim == 4) && !an->level)
+        return set_error(GS355_EINVAL, "anchors.level is NULL but the decoder takes the level as an input");
     if (an->A > 0 && (reinterpret_cast<uintptr_t>(an->feat) & 15u) != 0)
         return set_error(GS355_EINVAL, "anchor features must be 16-byte aligned");
     DecodeArgs a;
@@ -444,6 +631,8 @@ static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, DecodeAr
     a.scaling = an->scaling;
     a.visible = an->visible_mask;
     a.campos = an->campos;
+    a.level = dec->add_level ? an->level : nullptr;
+    a.split_feat = (dec->fp32_features || dec->bank_in_dim != 0) ? 1 : 0;  // bank-mixed features are general floats
     for (int j = 0; j < 3; ++j) {
         a.in_dim[j] = dec->in_dim[j];
         a.w0[j] = dec->w0[j];
@@ -451,6 +640,10 @@ static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, DecodeAr
         a.w1[j] = dec->w1[j];
         a.b1[j] = dec->b1[j];
     }
+    a.run_totals = nullptr;
+    a.run_base = nullptr;
+    a.neural_opacity = nullptr;
+    a.kept_mask = nullptr;
     *out = a;
     return GS355_OK;
 }
@@ -464,6 +657,32 @@ static dim3 decode_grid(int A, int cap)
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
     return dim3(blocks);
+}
+
+// Launch the count or the emit pass in the variant the features need.
+static void launch_decode(bool count_only, dim3 grid, hipStream_t s, const DecodeArgs& a, uint32_t* counts,
+                          const uint32_t* offsets, uint32_t capacity, const gs355_decoded* out)
+{
+    float* xyz = out ? out->xyz : nullptr;
+    float* color = out ? out->color : nullptr;
+    float* opacity = out ? out->opacity : nullptr;
+    float* scaling = out ? out->scaling : nullptr;
+    float* rot = out ? out->rot : nullptr;
+    if (count_only) {
+        if (a.split_feat)
+            hipLaunchKernelGGL((decode_kernel<true, true>), grid, dim3(256), 0, s, a, counts, offsets, capacity, xyz, color,
+                               opacity, scaling, rot);
+        else
+            hipLaunchKernelGGL((decode_kernel<true, false>), grid, dim3(256), 0, s, a, counts, offsets, capacity, xyz, color,
+                               opacity, scaling, rot);
+    } else {
+        if (a.split_feat)
+            hipLaunchKernelGGL((decode_kernel<false, true>), grid, dim3(256), 0, s, a, counts, offsets, capacity, xyz, color,
+                               opacity, scaling, rot);
+        else
+            hipLaunchKernelGGL((decode_kernel<false, false>), grid, dim3(256), 0, s, a, counts, offsets, capacity, xyz, color,
+                               opacity, scaling, rot);
+    }
 }
 
 }  // namespace gs355
@@ -515,7 +734,7 @@ int gs355_decode_count(const gs355_decoder* dec, const gs355_anchors* an, uint32
                        void* scratch_buf, size_t scratch_bytes, void* stream)
 {
     DecodeArgs a;
-    int rc = fill_args(dec, an, &a);
+    int rc = fill_args(dec, an, false, &a);
     if (rc) return rc;
     if (a.A == 0) return GS355_OK;
     if (!counts || !offsets || !scratch_buf) return set_error(GS355_EINVAL, "counts / offsets / scratch is NULL");
@@ -524,8 +743,7 @@ int gs355_decode_count(const gs355_decoder* dec, const gs355_anchors* an, uint32
     if (scratch_bytes < need)
         return set_error(GS355_ENOSPC, "decode scratch has %zu bytes, %zu needed", scratch_bytes, need);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(decode_kernel<true>, decode_grid(a.A, 1024), dim3(256), 0, s, a, counts, (const uint32_t*)nullptr, 0u,
-                       (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr);
+    launch_decode(true, decode_grid(a.A, 1024), s, a, counts, nullptr, 0u, nullptr);
     GS355_CHECK_LAUNCH("decode: count");
     return launch_exclusive_scan(counts, offsets, (size_t)a.A, static_cast<uint32_t*>(scratch_buf), s);
 }
@@ -534,7 +752,7 @@ int gs355_decode_count_static(const gs355_decoder* dec, const gs355_anchors* an,
                               void* stream)
 {
     DecodeArgs a;
-    int rc = fill_args(dec, an, &a);
+    int rc = fill_args(dec, an, false, &a);
     if (rc) return rc;
     if (a.A > kStaticCountMaxAnchors)
         return set_error(GS355_ENOSPC, "gs355_decode_count_static handles at most %d anchors (got %d); use gs355_decode_count",
@@ -547,8 +765,7 @@ int gs355_decode_count_static(const gs355_decoder* dec, const gs355_anchors* an,
     uint32_t* tmp = nullptr;
     if ((rc = static_scratch(&tmp))) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(decode_kernel<true>, decode_grid(a.A, 1024), dim3(256), 0, s, a, counts, (const uint32_t*)nullptr, 0u,
-                       (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr);
+    launch_decode(true, decode_grid(a.A, 1024), s, a, counts, nullptr, 0u, nullptr);
     GS355_CHECK_LAUNCH("decode: count");
     // the scan writes every block sum before it reads it: nothing in the array has to start at zero
     return launch_exclusive_scan(counts, offsets, (size_t)a.A, tmp, s);
@@ -558,7 +775,7 @@ int gs355_decode_emit(const gs355_decoder* dec, const gs355_anchors* an, const u
                       const gs355_decoded* out, void* stream)
 {
     DecodeArgs a;
-    int rc = fill_args(dec, an, &a);
+    int rc = fill_args(dec, an, false, &a);
     if (rc) return rc;
     if (a.A == 0 || capacity == 0) return GS355_OK;
     if (capacity < 0 || capacity > 0xFFFFFFFFll)
@@ -567,8 +784,108 @@ int gs355_decode_emit(const gs355_decoder* dec, const gs355_anchors* an, const u
     if (!out || !out->xyz || !out->color || !out->opacity || !out->scaling || !out->rot)
         return set_error(GS355_EINVAL, "decoded outputs must all be non-NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(decode_kernel<false>, decode_grid(a.A, 512), dim3(256), 0, s, a, (uint32_t*)nullptr, offsets,
-                       (uint32_t)capacity, out->xyz, out->color, out->opacity, out->scaling, out->rot);
+    launch_decode(false, decode_grid(a.A, 512), s, a, nullptr, offsets, (uint32_t)capacity, out);
+    GS355_CHECK_LAUNCH("decode: emit");
+    return GS355_OK;
+}
+
+namespace {
+struct FusedLayout {
+    size_t run_totals, run_base, mixed, total;
+};
+FusedLayout fused_layout(int32_t A, int32_t n, bool bank)
+{
+    auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+    const size_t runs = ((size_t)A + kRun - 1) / kRun;
+    FusedLayout L;
+    size_t off = 0;
+    (void)n;
+    L.run_totals = off;
+    off = up(off + runs * sizeof(uint2) + 8);
+    L.run_base = off;
+    off = up(off + runs * sizeof(uint2) + 8);
+    L.mixed = off;
+    if (bank) off = up(off + (size_t)A * kFeat * sizeof(float) + 4);
+    L.total = off;
+    return L;
+}
+}  // namespace
+
+int gs355_decode_workspace_bytes(int32_t A, int32_t n_offsets, int32_t with_feature_bank, size_t* bytes)
+{
+    if (!bytes) return set_error(GS355_EINVAL, "bytes is NULL");
+    if (A < 0) return set_error(GS355_EINVAL, "A must be >= 0 (got %d)", A);
+    if (n_offsets < 1 || n_offsets > 10)
+        return set_error(GS355_EINVAL, "anchor decode supports 1..10 offsets per anchor (got %d)", n_offsets);
+    *bytes = fused_layout(A, n_offsets, with_feature_bank != 0).total;
+    return GS355_OK;
+}
+
+int gs355_decode(const gs355_decoder* dec, const gs355_anchors* an, int64_t capacity, const gs355_decoded* out,
+                 void* workspace, size_t workspace_bytes, uint32_t phases, void* stream)
+{
+    if (phases == 0 || (phases & ~(uint32_t)(GS355_DECODE_COUNT | GS355_DECODE_EMIT)) != 0)
+        return set_error(GS355_EINVAL, "phases must be GS355_DECODE_COUNT, GS355_DECODE_EMIT or both (got 0x%x)", phases);
+    const bool do_count = (phases & GS355_DECODE_COUNT) != 0, do_emit = (phases & GS355_DECODE_EMIT) != 0;
+    DecodeArgs a;
+    int rc = fill_args(dec, an, true, &a);
+    if (rc) return rc;
+    if (capacity < 0 || capacity > 0xFFFFFFFFll)
+        return set_error(GS355_EINVAL, "capacity must be in [0, 2^32) (got %lld)", (long long)capacity);
+    if (!out) return set_error(GS355_EINVAL, "decoded outputs is NULL");
+    if (do_emit && capacity > 0 && (!out->xyz || !out->color || !out->opacity || !out->scaling || !out->rot))
+        return set_error(GS355_EINVAL, "decoded outputs must all be non-NULL");
+    const bool bank = dec->bank_in_dim != 0;
+    const FusedLayout L = fused_layout(a.A, a.n, bank);
+    if (a.A > 0) {
+        if (!workspace) return set_error(GS355_EINVAL, "workspace is NULL");
+        if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+            return set_error(GS355_EINVAL, "workspace must be 256-byte aligned");
+        if (workspace_bytes < L.total)
+            return set_error(GS355_ENOSPC, "decode workspace has %zu bytes, %zu needed", workspace_bytes, L.total);
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (a.A == 0) {
+        if (do_count && out->count && (rc = launch_fill_u32(out->count, 1, 0u, s))) return rc;
+        if (do_count && out->num_visible && (rc = launch_fill_u32(out->num_visible, 1, 0u, s))) return rc;
+        return GS355_OK;
+    }
+    char* ws = static_cast<char*>(workspace);
+    const uint32_t runs = (uint32_t)(((size_t)a.A + kRun - 1) / kRun);
+    if (bank) a.feat = reinterpret_cast<float*>(ws + L.mixed);  // written by the count phase, read by both passes
+    uint2* run_base = reinterpret_cast<uint2*>(ws + L.run_base);
+    if (do_count) {
+        if (bank) {
+            BankArgs b;
+            b.A = a.A;
+            b.in_dim = dec->bank_in_dim;
+            b.anchor = a.anchor;
+            b.feat = an->feat;
+            b.visible = a.visible;
+            b.campos = a.campos;
+            b.level = an->level;
+            b.w0 = dec->bank_w0;
+            b.b0 = dec->bank_b0;
+            b.w1 = dec->bank_w1;
+            b.b1 = dec->bank_b1;
+            b.mixed = reinterpret_cast<float*>(ws + L.mixed);
+            hipLaunchKernelGGL(feature_bank_kernel, dim3((a.A + 255) / 256), dim3(256), 0, s, b);
+            GS355_CHECK_LAUNCH("decode: feature bank");
+        }
+        a.run_totals = reinterpret_cast<uint2*>(ws + L.run_totals);
+        launch_decode(true, decode_grid(a.A, 1024), s, a, nullptr, nullptr, 0u, nullptr);
+        GS355_CHECK_LAUNCH("decode: count");
+        hipLaunchKernelGGL(run_scan_kernel, dim3(1), dim3(1024), 0, s, a.run_totals, run_base, runs, out->count,
+                           out->num_visible);
+        GS355_CHECK_LAUNCH("decode: run scan");
+    }
+    if (!do_emit) return GS355_OK;
+    if (capacity == 0 && !out->neural_opacity && !out->mask) return GS355_OK;
+    a.run_totals = nullptr;
+    a.run_base = run_base;
+    a.neural_opacity = out->neural_opacity;
+    a.kept_mask = out->mask;
+    launch_decode(false, decode_grid(a.A, 512), s, a, nullptr, nullptr, (uint32_t)capacity, out);
     GS355_CHECK_LAUNCH("decode: emit");
     return GS355_OK;
 }

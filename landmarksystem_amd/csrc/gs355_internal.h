@@ -33,7 +33,16 @@ struct FrameArgs {  // by-value kernel argument
     const float* projmatrix;
     const float* campos;
     const float* bg;
+    const uint32_t* p_device;  // optional device-side number of Gaussians (gs355_gaussians.P_device)
 };
+
+// Number of Gaussians a kernel processes: the host's P, or the device-side count when there is one.
+__device__ __forceinline__ int effective_count(const FrameArgs& f, int P)
+{
+    if (!f.p_device) return P;
+    const uint32_t n = *f.p_device;
+    return n < (uint32_t)P ? (int)n : P;
+}
 
 // Extras of the radii-only preprocess when it serves the anchor prefilter (by-value kernel argument).
 struct FilterArgs {
@@ -76,8 +85,8 @@ __device__ __forceinline__ Rect tile_rect(float px, float py, int radius, int gr
 // stage launchers (each returns a gs355_status)
 int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_only, float* records,
                       uint32_t* tiles_touched, uint64_t* rects, uint32_t* depth_bits, int32_t* radii, hipStream_t s);
-int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int32_t P, uint32_t* offsets,
-                        uint32_t* scan_tmp, gs355_header* header, uint32_t n_cap, hipStream_t s);
+int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int32_t P, const uint32_t* p_device,
+                        uint32_t* offsets, uint32_t* scan_tmp, gs355_header* header, uint32_t n_cap, hipStream_t s);
 int launch_anchor_filter(const FrameArgs& f, const gs355_gaussians& g, const FilterArgs& x, int32_t* radii, hipStream_t s);
 int launch_duplicate(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
                      const uint32_t* offsets, const gs355_header* header, uint64_t* keys, uint32_t* values,

@@ -180,7 +180,7 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
     __shared__ int s_alive[4];
 
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    const bool valid = i < g.P;
+    const bool valid = i < effective_count(f, g.P);
     const float* __restrict__ V = f.viewmatrix;
     const float* __restrict__ M = f.projmatrix;
 
@@ -391,8 +391,10 @@ __global__ __launch_bounds__(256) void duplicate_kernel(FrameArgs f, int32_t P, 
     __shared__ int s_x0[256], s_y0[256], s_w[256];
 
     if (header->overflow) return;  // capacity too small: the caller redoes the frame
+    P = effective_count(f, P);
     const int t = threadIdx.x;
     const int g0 = blockIdx.x * 256;
+    if (g0 >= P) return;  // uniform
     const int i = g0 + t;
     const uint32_t begin = g0 == 0 ? 0u : offsets[g0 - 1];
     uint32_t end_i = begin;

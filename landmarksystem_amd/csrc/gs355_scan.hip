@@ -52,14 +52,17 @@ __device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t v, uint32_t* s
 }
 
 // ---- tile sums -----------------------------------------------------------
+// `n_device` (optional): device-side element count; elements at and beyond it count as zero.
 template <bool kCountVisible>
 __global__ __launch_bounds__(kScanThreads) void tile_sum_kernel(const uint32_t* __restrict__ in,
                                                                 const int32_t* __restrict__ radii, size_t n,
+                                                                const uint32_t* __restrict__ n_device,
                                                                 uint64_t* __restrict__ sums,
                                                                 uint32_t* __restrict__ visible)
 {
     __shared__ uint64_t s_sum[4];
     __shared__ uint32_t s_vis[4];
+    if (n_device && (size_t)*n_device < n) n = *n_device;
     const size_t base = (size_t)blockIdx.x * kScanTile;
     uint64_t acc = 0;
     uint32_t vis = 0;
@@ -131,10 +134,12 @@ __global__ __launch_bounds__(256) void scan_sums_kernel(uint64_t* __restrict__ s
 // ---- rescan each tile with its prefix --------------------------------------
 template <bool kInclusive>
 __global__ __launch_bounds__(kScanThreads) void tile_scan_kernel(const uint32_t* in, size_t n,
+                                                                 const uint32_t* __restrict__ n_device,
                                                                  const uint64_t* __restrict__ sums,
                                                                  uint32_t* out /* may alias in */)
 {
     __shared__ uint32_t s_wave[4];
+    if (n_device && (size_t)*n_device < n) n = *n_device;
     const size_t base = (size_t)blockIdx.x * kScanTile;
     // blocked arrangement: thread t owns items [t*kScanItems, (t+1)*kScanItems)
     uint32_t v[kScanItems];
@@ -168,22 +173,22 @@ size_t scan_tmp_words(size_t n)
     return nb * 3 + 8;  // u64 sum + u32 visible per tile
 }
 
-int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int32_t P, uint32_t* offsets,
-                        uint32_t* scan_tmp, gs355_header* header, uint32_t n_cap, hipStream_t s)
+int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int32_t P, const uint32_t* p_device,
+                        uint32_t* offsets, uint32_t* scan_tmp, gs355_header* header, uint32_t n_cap, hipStream_t s)
 {
     const uint32_t nb = (uint32_t)(((size_t)P + kScanTile - 1) / kScanTile);
     uint64_t* sums = reinterpret_cast<uint64_t*>(scan_tmp);
     uint32_t* visible = scan_tmp + 2 * (size_t)(nb ? nb : 1);
     if (nb) {
         hipLaunchKernelGGL(tile_sum_kernel<true>, dim3(nb), dim3(kScanThreads), 0, s, tiles_touched, radii, (size_t)P,
-                           sums, visible);
+                           p_device, sums, visible);
         GS355_CHECK_LAUNCH("scan: tile sums");
     }
     hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, s, sums, visible, nb, header, n_cap);
     GS355_CHECK_LAUNCH("scan: sums");
     if (nb) {
-        hipLaunchKernelGGL(tile_scan_kernel<true>, dim3(nb), dim3(kScanThreads), 0, s, tiles_touched, (size_t)P, sums,
-                           offsets);
+        hipLaunchKernelGGL(tile_scan_kernel<true>, dim3(nb), dim3(kScanThreads), 0, s, tiles_touched, (size_t)P,
+                           p_device, sums, offsets);
         GS355_CHECK_LAUNCH("scan: tiles");
     }
     return GS355_OK;
@@ -194,13 +199,14 @@ int launch_exclusive_scan(const uint32_t* in, uint32_t* out, size_t n, uint32_t*
     if (n == 0) return GS355_OK;
     const uint32_t nb = (uint32_t)((n + kScanTile - 1) / kScanTile);
     uint64_t* sums = reinterpret_cast<uint64_t*>(tmp);
-    hipLaunchKernelGGL(tile_sum_kernel<false>, dim3(nb), dim3(kScanThreads), 0, s, in, (const int32_t*)nullptr, n, sums,
-                       (uint32_t*)nullptr);
+    hipLaunchKernelGGL(tile_sum_kernel<false>, dim3(nb), dim3(kScanThreads), 0, s, in, (const int32_t*)nullptr, n,
+                       (const uint32_t*)nullptr, sums, (uint32_t*)nullptr);
     GS355_CHECK_LAUNCH("scan: tile sums");
     hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, s, sums, (const uint32_t*)nullptr, nb,
                        (gs355_header*)nullptr, 0u);
     GS355_CHECK_LAUNCH("scan: sums");
-    hipLaunchKernelGGL(tile_scan_kernel<false>, dim3(nb), dim3(kScanThreads), 0, s, in, n, sums, out);
+    hipLaunchKernelGGL(tile_scan_kernel<false>, dim3(nb), dim3(kScanThreads), 0, s, in, n, (const uint32_t*)nullptr, sums,
+                       out);
     GS355_CHECK_LAUNCH("scan: tiles");
     return GS355_OK;
 }

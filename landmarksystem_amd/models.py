@@ -317,17 +317,20 @@ class ScaffoldGS(nn.Module):
     """Scaffold-GS: anchors decoded into neural Gaussians per frame."""
 
     _ckpt_kind = "scaffold"
-    _decoder_options = (("use_feat_bank", False), ("view_dim", 3))
+    _decoder_options = (("view_dim", 3),)
 
     def __init__(self, anchor=None, anchor_feat=None, offset=None, scaling=None, rotation=None, n_offsets: int = 10,
                  feat_dim: int = 32, add_opacity_dist: bool = True, add_cov_dist: bool = True,
                  add_color_dist: bool = True, white_bkgd: bool = False, act_cache: bool = False, opacity=None,
-                 config=None, scene_manager=None, fuse_prefilter: bool = False):
+                 config=None, scene_manager=None, fuse_prefilter: bool = False, use_feat_bank: bool = False,
+                 add_level: bool = False, appearance_dim: int = 0):
         super().__init__()
         # fuse_prefilter: the anchor-level prefilter (for Octree-GS including the level-of-detail mask, its gather
-        # of the selected anchors and the scatter of the result) runs as one kernel over all anchors.  Same masks,
-        # except that an anchor whose predicted level sits within rounding of a .5 boundary may fall on the other
-        # side (the level-of-detail formula is evaluated in the kernel instead of by a chain of torch operations).
+        # of the selected anchors and the scatter of the result) runs as one kernel over all anchors, and the
+        # number of decoded Gaussians stays on the device: decode and rasterizer are enqueued back to back without
+        # a read-back in between (`visibility_filter` reads it when asked for).  Same masks, except that an anchor
+        # whose predicted level sits within rounding of a .5 boundary may fall on the other side (the
+        # level-of-detail formula is evaluated in the kernel instead of by a chain of torch operations).
         self.fuse_prefilter = fuse_prefilter
         if anchor is not None and not torch.is_tensor(anchor):  # the reference's signature: (config, scene_manager)
             config, anchor = anchor, None
@@ -338,9 +341,13 @@ class ScaffoldGS(nn.Module):
             add_color_dist = _cfg(config, "add_color_dist", add_color_dist)
             white_bkgd, act_cache = _cfg(config, "white_bkgd", white_bkgd), _cfg(config, "act_cache", act_cache)
             self.fuse_prefilter = _cfg(config, "fuse_prefilter", fuse_prefilter)
+            use_feat_bank = _cfg(config, "use_feat_bank", use_feat_bank)
             # the options the reference's model hands to its AnchorDecoder: scaffold_gs/gs_model.py:126-134 passes
             # neither add_level nor appearance_dim (its config's add_level=True default never reaches the decoder);
             # octree_gs/gs_model.py:165-176 passes both
+            if self._ckpt_kind == "octree":
+                add_level = _cfg(config, "add_level", add_level)
+                appearance_dim = _cfg(config, "appearance_dim", appearance_dim)
             for name, allowed in self._decoder_options:
                 if _cfg(config, name, allowed) != allowed:
                     raise NotImplementedError("%s=%r: the fused anchor decode supports %s=%r only"
@@ -360,12 +367,29 @@ class ScaffoldGS(nn.Module):
         self._rotation = nn.Parameter(rotation, requires_grad=False)  # [A,4]
         self.act_cache = act_cache
         self.anchor_decoder = FusedAnchorDecoder(
-            use_feat_bank=False, add_opacity_dist=add_opacity_dist, add_color_dist=add_color_dist,
-            add_cov_dist=add_cov_dist, view_dim=3, feat_dim=feat_dim, n_offsets=n_offsets)
+            use_feat_bank=use_feat_bank, add_opacity_dist=add_opacity_dist, add_color_dist=add_color_dist,
+            add_cov_dist=add_cov_dist, view_dim=3, feat_dim=feat_dim, n_offsets=n_offsets,
+            appearance_dim=appearance_dim, add_level=add_level)
         self.register_buffer("background", torch.tensor([1.0, 1.0, 1.0] if white_bkgd else [0.0, 0.0, 0.0]))
         self.renderer = _placeholder_renderer(self.background)
         self._cache = {}
-        self.visibility_filter = self.voxel_visible_mask = None
+        self._visibility_filter = self.voxel_visible_mask = None
+        self._pending = None  # (decode result, radii sized for its capacity) of a frame whose count is still on the device
+
+    # `visibility_filter` (bool[G] over the decoded Gaussians) is a by-product the reference leaves on the model.
+    # A frame rendered without reading the number of Gaussians back derives it when it is asked for.
+    @property
+    def visibility_filter(self):
+        if self._visibility_filter is None and self._pending is not None:
+            res, radii = self._pending
+            G, _ = self.anchor_decoder.read_counts(res)
+            self._visibility_filter = radii[:G] > 0
+            self._pending = None
+        return self._visibility_filter
+
+    @visibility_filter.setter
+    def visibility_filter(self, value):
+        self._visibility_filter, self._pending = value, None
 
     @classmethod
     def from_scene(cls, scene, **kw):
@@ -470,6 +494,9 @@ class ScaffoldGS(nn.Module):
     def _before_prefilter(self, viewpoint_camera):
         pass
 
+    def _decoder_level(self):
+        return None  # Scaffold-GS anchors carry no level
+
     @torch.no_grad()
     def forward(self, viewpoint_camera, scaling_modifier=1.0, retain_grad=False, render_exclude_filter=None):
         viewpoint_camera = viewpoint_camera.to(self._anchor.device)
@@ -477,10 +504,21 @@ class ScaffoldGS(nn.Module):
         voxel_visible_mask = self.prefilter_voxel(viewpoint_camera)
         if render_exclude_filter is not None:
             voxel_visible_mask = voxel_visible_mask & render_exclude_filter
-        xyz, color, opacity, scaling, rot, _, _ = self.anchor_decoder(
-            camera_center=viewpoint_camera.camera_center, anchor=self.get_anchor, anchor_feat=self.get_anchor_feat,
-            offset=self.get_offset, scaling=self.get_scaling, visible_mask=voxel_visible_mask)
         self.renderer.raster_settings = _settings(viewpoint_camera, self.background, scaling_modifier, 1)
+        decode = dict(camera_center=viewpoint_camera.camera_center, anchor=self.get_anchor,
+                      anchor_feat=self.get_anchor_feat, offset=self.get_offset, scaling=self.get_scaling,
+                      visible_mask=voxel_visible_mask, level=self._decoder_level())
+        if self.fuse_prefilter and not self.training:
+            # nothing is read back: the decode leaves the number of Gaussians on the device, the rasterizer takes it
+            # from there and works over tensors sized for the most the anchors can emit
+            res = self.anchor_decoder.decode_on_device(**decode, reuse_buffers=True)
+            rendered_image, radii, _ = self.renderer(
+                means3D=res.xyz, means2D=None, shs=None, colors_precomp=res.color, opacities=res.opacity,
+                scales=res.scaling, rotations=res.rot, cov3D_precomp=None, count=res.count)
+            self._visibility_filter, self._pending = None, (res, radii)
+            self.voxel_visible_mask = voxel_visible_mask
+            return rendered_image
+        xyz, color, opacity, scaling, rot, _, _ = self.anchor_decoder(**decode)
         rendered_image, radii, _ = self.renderer(
             means3D=xyz, means2D=None, shs=None, colors_precomp=color, opacities=opacity, scales=scaling,
             rotations=rot, cov3D_precomp=None)
@@ -492,7 +530,7 @@ class OctreeGS(ScaffoldGS):
     """Octree-GS: Scaffold-GS plus a per-frame level-of-detail mask over the anchors."""
 
     _ckpt_kind = "octree"
-    _decoder_options = ScaffoldGS._decoder_options + (("appearance_dim", 0), ("add_level", False))
+    _decoder_options = ScaffoldGS._decoder_options + (("appearance_dim", 0),)
     _encoding_keys = ScaffoldGS._encoding_keys + ("_level", "_extra_level")
 
     def __init__(self, anchor=None, anchor_feat=None, offset=None, scaling=None, rotation=None, level=None,
@@ -559,6 +597,12 @@ class OctreeGS(ScaffoldGS):
         # ape_code selects an appearance embedding in the reference (octree_gs/gs_model.py:254-260); without
         # appearance inputs (appearance_dim = 0, all this decode supports) it has no effect
         return super().forward(viewpoint_camera, scaling_modifier, retain_grad, render_exclude_filter)
+
+    def _decoder_level(self):
+        # the reference's model hands its decoder `gaussian_encoding.levels`, the number of levels
+        # (octree_gs/gs_model.py:268), where the decoder indexes a per-anchor tensor (anchor_decoder.py:157-158): with
+        # add_level that call cannot run.  The per-anchor level is what the decoder's input is built for.
+        return self._level if self.anchor_decoder.add_level else None
 
     def _level_span_value(self) -> int:
         if self._level_span is None or self._level_span[0] is not self._level:

@@ -122,7 +122,10 @@ class FrameInputs:
     """The tensors of one rasterizer call, validated and marshalled."""
 
     def __init__(self, settings, means3D, opacities=None, shs=None, colors_precomp=None, scales=None, rotations=None,
-                 cov3D_precomp=None, need_colour: bool = True):
+                 cov3D_precomp=None, need_colour: bool = True, count: Optional[torch.Tensor] = None):
+        """`count`: optional one-element int32 tensor on the device holding the number of Gaussians (the anchor
+        decode leaves it there); the tensors are then sized for a capacity and only the first `count` rows are
+        rendered, without the host ever reading the number."""
         if need_colour:
             if (shs is None and colors_precomp is None) or (shs is not None and colors_precomp is not None):
                 raise Exception("Please provide excatly one of either SHs or precomputed colors!")
@@ -171,6 +174,13 @@ class FrameInputs:
         g.means3D, g.shs, g.colors_precomp = _ptr(self.means3D), _ptr(self.shs), _ptr(self.colors_precomp)
         g.opacities, g.scales, g.rotations = _ptr(self.opacities), _ptr(self.scales), _ptr(self.rotations)
         g.cov3D_precomp = _ptr(self.cov3D_precomp)
+        self.count = None
+        if count is not None:
+            if not (isinstance(count, torch.Tensor) and count.device == dev and count.numel() == 1
+                    and count.dtype in (torch.int32, torch.uint32)):
+                raise ValueError("count must be a one-element int32 tensor on the Gaussians' device")
+            self.count = count
+            g.P_device = count.data_ptr()
         self.gaussians = g
 
     @property

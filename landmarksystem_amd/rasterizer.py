@@ -133,8 +133,11 @@ class GaussianRasterizer(nn.Module):
         return pipeline.visible_filter(inputs)
 
     def forward(self, means3D, means2D=None, opacities=None, shs=None, colors_precomp=None, scales=None,
-                rotations=None, cov3D_precomp=None):
+                rotations=None, cov3D_precomp=None, count=None):
         """Returns (image f32[3,H,W], radii i32[P], depth f32[1,H,W]).
+        `count` (an extension of the reference's signature): one-element int32 device tensor with the number of
+        Gaussians when only the device knows it (the anchor decode's output); the inputs are then sized for a
+        capacity P, rows at and beyond `count` are ignored and their radii are not written.  Inference only.
         `means2D` takes no part in the forward pass; when it requires grad it
         receives the screen-space gradient (normalised device units, third
         component zero).  Alpha (1 - final transmittance, f32[1,H,W]) is left
@@ -143,12 +146,14 @@ class GaussianRasterizer(nn.Module):
             raise ValueError("opacities is required")
         tensors = (means3D, means2D, opacities, shs, colors_precomp, scales, rotations, cov3D_precomp)
         if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors):
+            if count is not None:
+                raise ValueError("a device-side Gaussian count cannot be combined with gradients")
             image, radii, depth, alpha = _RasterizeGaussians.apply(self.raster_settings, *tensors)
             self.last_depth, self.last_alpha, self.last_num_keys = depth, alpha, 0
             return image, radii, depth
         inputs = pipeline.FrameInputs(self.raster_settings, means3D, opacities=opacities, shs=shs,
                                       colors_precomp=colors_precomp, scales=scales, rotations=rotations,
-                                      cov3D_precomp=cov3D_precomp)
+                                      cov3D_precomp=cov3D_precomp, count=count)
         out = pipeline.render(inputs)
         self.last_depth, self.last_alpha, self.last_num_keys = out.depth, out.alpha, out.num_keys
         return out.image, out.radii, out.depth

@@ -30,7 +30,7 @@ def test_struct_sizes_match_the_header():
     # 64-byte header; pointers are 8 bytes; the layout struct mirrors include/gs355.h field by field
     assert C.sizeof(_lib.Header) == 64
     assert C.sizeof(_lib.Frame) == 7 * 4 + 4 + 4 * 8  # 7 scalars, padding to 8, 4 pointers
-    assert C.sizeof(_lib.Gaussians) == 8 + 7 * 8
+    assert C.sizeof(_lib.Gaussians) == 8 + 8 * 8  # P (padded to 8), 7 tensors, the optional device-side count
     assert C.sizeof(_lib.Outputs) == 4 * 8
     assert C.sizeof(_lib.Layout) == 18 * 8 + 4 * 4
     assert C.sizeof(_lib.AnchorLod) == 2 * 8 + 4 * 4 + 2 * 4

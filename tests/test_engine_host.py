@@ -92,8 +92,9 @@ def test_config_built_models_load_their_checkpoints(tmp_path):
     assert all(torch.equal(a, b) for a, b in zip(s.parameters(), empty.parameters()))
     with pytest.raises(ValueError, match="only found keys"):
         ScaffoldGS(config={}).load_from_state_dict({"gaussian_encoding._anchor": torch.zeros(2, 3)})
-    with pytest.raises(NotImplementedError, match="use_feat_bank"):
-        ScaffoldGS(config=dict(use_feat_bank=True))
+    banked = ScaffoldGS(config=dict(use_feat_bank=True))  # the feature bank is a fourth MLP of the decoder
+    assert banked.anchor_decoder.mlp_feature_bank[0].weight.shape == (32, 3)
+    assert banked.anchor_decoder.mlp_feature_bank[2].weight.shape == (3, 32)
 
     o = _anchor_model(OctreeGS, g, level=torch.tensor([0, 1, 2, 0, 1, 2]), voxel_size=0.25, standard_dist=40.0,
                       extra_level=torch.randn(6, generator=g), add_opacity_dist=False, add_cov_dist=False,
@@ -109,9 +110,21 @@ def test_config_built_models_load_their_checkpoints(tmp_path):
         OctreeGS(dict(appearance_dim=32))
     # the Scaffold-GS model never hands add_level / appearance_dim to its decoder (scaffold_gs/gs_model.py:126-134),
     # so its config's add_level=True default (:33) must be accepted
-    ScaffoldGS(dict(n_offsets=10, feat_dim=32, add_level=True, appearance_dim=32))
-    with pytest.raises(NotImplementedError, match="use_feat_bank"):
-        ScaffoldGS(dict(use_feat_bank=True))
+    plain = ScaffoldGS(dict(n_offsets=10, feat_dim=32, add_level=True, appearance_dim=32))
+    assert plain.anchor_decoder.mlp_opacity[0].weight.shape == (32, 36) and not plain.anchor_decoder.add_level
+    # Octree-GS does hand them over (octree_gs/gs_model.py:165-176): the level widens every head and the bank's input
+    levelled = OctreeGS(dict(n_offsets=10, feat_dim=32, add_level=True, use_feat_bank=True))
+    assert levelled.anchor_decoder.add_level and levelled.anchor_decoder.mlp_opacity[0].weight.shape == (32, 36)
+    assert levelled.anchor_decoder.mlp_feature_bank[0].weight.shape == (32, 4)
+    # a checkpoint with a feature bank and a level input loads into a decoder of the same shape
+    ob = _anchor_model(OctreeGS, g, level=torch.tensor([0, 1, 2, 0, 1, 2]), voxel_size=0.25, standard_dist=40.0,
+                       add_opacity_dist=False, add_cov_dist=False, add_color_dist=False, use_feat_bank=True,
+                       add_level=True)
+    ck.save_model(ob, tmp_path / "ob")
+    back = ck.load_octree_gs(tmp_path / "ob", device="cpu")
+    assert back.anchor_decoder.use_feat_bank and back.anchor_decoder.add_level
+    assert not back.anchor_decoder.add_opacity_dist
+    assert all(torch.equal(a, b) for a, b in zip(ob.anchor_decoder.parameters(), back.anchor_decoder.parameters()))
 
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU error")

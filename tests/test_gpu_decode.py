@@ -115,8 +115,168 @@ def test_decode_nothing_visible_and_default_mask(gpu_device):
 
 def test_unsupported_configurations_are_refused():
     with pytest.raises(NotImplementedError):
-        FusedAnchorDecoder(True, True, True, True, 3, 32, 10)
-    with pytest.raises(NotImplementedError):
-        FusedAnchorDecoder(False, True, True, True, 3, 32, 10, add_level=True)
+        FusedAnchorDecoder(False, True, True, True, 3, 32, 10, appearance_dim=32)
     with pytest.raises(NotImplementedError):
         FusedAnchorDecoder(False, True, True, True, 3, 64, 10)
+
+
+def decoder_with(sc, device, g, use_feat_bank, add_level, add_dist):
+    """A decoder with the given options and random weights of the right shapes; returns it with the oracle's view
+    of the same weights."""
+    dec = FusedAnchorDecoder(use_feat_bank=use_feat_bank, add_opacity_dist=add_dist[0], add_color_dist=add_dist[2],
+                             add_cov_dist=add_dist[1], view_dim=3, feat_dim=32, n_offsets=sc.n_offsets,
+                             add_level=add_level)
+    with torch.no_grad():
+        for p in dec.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) * (0.5 if p.dim() == 1 else p.shape[1] ** -0.5)).half().float())
+    mlp = {}
+    for name, head in (("mlp_opacity", "opacity"), ("mlp_cov", "cov"), ("mlp_color", "color")):
+        m = getattr(dec, name)
+        mlp[head] = tuple(t.detach().clone() for t in (m[0].weight, m[0].bias, m[2].weight, m[2].bias))
+    bank = None
+    if use_feat_bank:
+        m = dec.mlp_feature_bank
+        bank = tuple(t.detach().clone() for t in (m[0].weight, m[0].bias, m[2].weight, m[2].bias))
+    return dec.to(device).eval(), mlp, bank
+
+
+@pytest.mark.parametrize("use_feat_bank,add_level", [(True, False), (False, True), (True, True)])
+def test_decode_with_feature_bank_and_level(gpu_device, use_feat_bank, add_level):
+    """The feature bank (anchor_decoder.py:163-177) and the level input (:179-186): with a level every head reads
+    [feat | view | level], so the heads are built without distance inputs (the Octree-GS defaults)."""
+    A = 20_000
+    sc = scenes.config5(A=A)
+    g = torch.Generator().manual_seed(7 + 2 * use_feat_bank + add_level)
+    add_dist = (False, False, False) if add_level else (True, False, True)
+    dec, mlp, bank = decoder_with(sc, gpu_device, g, use_feat_bank, add_level, add_dist)
+    vis = torch.rand(A, generator=g) < 0.6
+    level = torch.randint(0, 5, (A, 1), generator=g).float()
+    cam = sc.camera.camera_center
+    got = dec(camera_center=cam.to(gpu_device), anchor=sc.anchor.to(gpu_device), anchor_feat=sc.anchor_feat.to(gpu_device),
+              offset=sc.offset.to(gpu_device), scaling=sc.scaling.to(gpu_device), visible_mask=vis.to(gpu_device),
+              level=level.to(gpu_device))
+    redo = lambda keep=None: ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, mlp, sc.n_offsets,  # noqa: E731
+                                       add_dist=add_dist, keep_override=keep, level=level, add_level=add_level, bank=bank)
+    compare(got, redo(), redo)
+    assert got[0].shape[0] > A  # a real decode, not an empty one
+
+
+def test_features_that_fp16_cannot_hold(gpu_device):
+    """Anchor features of an fp32-trained checkpoint are general floats: they enter the matrix cores as hi + lo
+    fp16 pairs, so the decode still meets the fp32 bar (weights remain fp16-representable here)."""
+    A = 12_000
+    sc = scenes.config5(A=A)
+    g = torch.Generator().manual_seed(12)
+    sc.anchor_feat = torch.randn(A, 32, generator=g) * 0.5  # not rounded to fp16
+    assert not torch.equal(sc.anchor_feat.half().float(), sc.anchor_feat)
+    dec = build_decoder(sc, gpu_device)
+    vis = torch.rand(A, generator=g) < 0.8
+    cam = sc.camera.camera_center
+    got = dec(cam.to(gpu_device), sc.anchor.to(gpu_device), sc.anchor_feat.to(gpu_device), sc.offset.to(gpu_device),
+              sc.scaling.to(gpu_device), vis.to(gpu_device))
+    redo = lambda keep=None: ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp,  # noqa: E731
+                                       sc.n_offsets, keep_override=keep)
+    compare(got, redo(), redo)
+
+
+def test_level_input_follows_the_reference_quirks(gpu_device):
+    sc = scenes.config5(A=64)
+    g = torch.Generator().manual_seed(1)
+    args = [t.to(gpu_device) for t in (sc.camera.camera_center, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling)]
+    level = torch.zeros(64, 1, device=gpu_device)
+    # a head built with a distance column as well (37 wide) cannot be fed by the reference's forward
+    dec, _, _ = decoder_with(sc, gpu_device, g, False, True, (True, False, False))
+    assert dec.mlp_opacity[0].weight.shape == (32, 37)
+    with pytest.raises(RuntimeError, match="shape mismatch"):
+        dec(*args, None, level)
+    # add_level without a level tensor: the input lacks the column the heads were built for
+    dec, _, _ = decoder_with(sc, gpu_device, g, False, True, (False, False, False))
+    with pytest.raises(RuntimeError, match="no level was given"):
+        dec(*args, None, None)
+    # without add_level a level tensor is ignored
+    dec, mlp, _ = decoder_with(sc, gpu_device, g, False, False, (True, True, True))
+    a, b = dec(*args, None, level), dec(*args, None, None)
+    assert all(torch.equal(x, y) for x, y in zip(a[:5], b[:5]))
+
+
+def test_training_mode_returns_every_opacity_and_the_mask(gpu_device):
+    """anchor_decoder.py:239-242: in training mode the 7-tuple also carries the opacity of every offset of the
+    visible anchors and the mask that selected the Gaussians."""
+    A = 9000
+    sc = scenes.config5(A=A)
+    dec = build_decoder(sc, gpu_device).train()
+    vis = torch.rand(A, generator=torch.Generator().manual_seed(4)) < 0.5
+    cam = sc.camera.camera_center
+    out = dec(cam.to(gpu_device), sc.anchor.to(gpu_device), sc.anchor_feat.to(gpu_device), sc.offset.to(gpu_device),
+              sc.scaling.to(gpu_device), vis.to(gpu_device))
+    ref = ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp, sc.n_offsets)
+    neural_opacity, mask = out[5], out[6]
+    a_vis = int(vis.sum())
+    assert neural_opacity.shape == (a_vis * 10, 1) and mask.shape == (a_vis * 10,) and mask.dtype == torch.bool
+    want = ref["neural_opacity"].numpy()
+    assert float(np.abs(neural_opacity.cpu().numpy() - want).max()) <= TOL
+    sure = np.abs(ref["raw_opacity"].numpy()) > UNSURE
+    np.testing.assert_array_equal(mask.cpu().numpy()[sure], ref["mask"].numpy()[sure])
+    assert torch.equal(neural_opacity[mask], out[2]) and int(mask.sum()) == out[0].shape[0]
+    redo = lambda keep=None: ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp,  # noqa: E731
+                                       sc.n_offsets, keep_override=keep)
+    compare(out[:5] + (None, None), ref, redo)
+    assert dec.eval()(cam.to(gpu_device), sc.anchor.to(gpu_device), sc.anchor_feat.to(gpu_device),
+                      sc.offset.to(gpu_device), sc.scaling.to(gpu_device), vis.to(gpu_device))[5] is None
+
+
+def test_decode_on_device_and_the_two_pass_entry_points_agree(gpu_device):
+    """gs355_decode (one call, count kept on the device) against gs355_decode_count + gs355_decode_emit (per-anchor
+    offsets, exact output size) through the C ABI: the same Gaussians bit for bit."""
+    import ctypes as C
+
+    from landmarksystem_amd import _lib
+    A = 70_001
+    sc = scenes.config5(A=A)
+    dec = build_decoder(sc, gpu_device)
+    vis = (torch.rand(A, generator=torch.Generator().manual_seed(8)) < 0.4).to(gpu_device)
+    t = [x.to(gpu_device).contiguous() for x in (sc.camera.camera_center, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling)]
+    res = dec.decode_on_device(*t, vis)
+    G, a_vis = dec.read_counts(res)
+    assert a_vis == int(vis.sum()) and 0 < G < a_vis * 10 and res.xyz.shape[0] == A * 10
+    exact = dec(*t, vis)
+    assert exact[0].shape[0] == G
+    lib = _lib.load()
+    d = dec._decoder_struct(gpu_device)
+    an = _lib.Anchors()
+    an.A, an.campos, an.anchor, an.feat, an.offset, an.scaling = A, *(x.data_ptr() for x in t)
+    an.visible_mask = vis.data_ptr()
+    need = C.c_size_t()
+    _lib.check(lib.gs355_decode_scratch_bytes(A, C.byref(need)))
+    scratch = torch.empty(need.value, dtype=torch.uint8, device=gpu_device)
+    counts = torch.empty(A, dtype=torch.int32, device=gpu_device)
+    offsets = torch.empty(A, dtype=torch.int32, device=gpu_device)
+    stream = torch.cuda.current_stream(gpu_device).cuda_stream
+    _lib.check(lib.gs355_decode_count(C.byref(d), C.byref(an), counts.data_ptr(), offsets.data_ptr(), scratch.data_ptr(),
+                                      scratch.numel(), stream))
+    assert int(offsets[-1] + counts[-1]) == G
+    outs = [torch.empty((G, k), device=gpu_device) for k in (3, 3, 1, 3, 4)]
+    o = _lib.Decoded()
+    o.xyz, o.color, o.opacity, o.scaling, o.rot = (x.data_ptr() for x in outs)
+    _lib.check(lib.gs355_decode_emit(C.byref(d), C.byref(an), offsets.data_ptr(), G, C.byref(o), stream))
+    torch.cuda.synchronize()
+    for name, two_pass, one_call, sliced in zip(("xyz", "color", "opacity", "scaling", "rot"), outs, exact[:5],
+                                                (res.xyz, res.color, res.opacity, res.scaling, res.rot)):
+        assert torch.equal(two_pass, one_call), name
+        assert torch.equal(sliced[:G], one_call), name
+
+
+def test_model_frames_without_reading_the_gaussian_count_back(gpu_device):
+    """Scaffold- / Octree-GS with the fused path: the decode leaves the number of Gaussians on the device and the
+    rasterizer takes it from there.  Same frame as the sequence that reads it back, also through the classic
+    stages (images beyond the tile-bucket limit), and the by-products appear when they are asked for."""
+    from landmarksystem_amd.models import ScaffoldGS
+    for width, height in ((640, 360), (4000, 2400)):
+        scene = scenes.config5(A=30_000, width=width, height=height)
+        plain = ScaffoldGS.from_scene(scene).to(gpu_device).eval()
+        fused = ScaffoldGS.from_scene(scene, fuse_prefilter=True).to(gpu_device).eval()
+        a, b = plain(scene.camera), fused(scene.camera)
+        assert torch.equal(a, b) and float(a.max()) > 0.1
+        assert fused._pending is not None  # nothing was read back yet
+        assert torch.equal(plain.visibility_filter, fused.visibility_filter) and fused._pending is None
+        assert torch.equal(plain(scene.camera), fused(scene.camera))  # a second frame over the same buffers

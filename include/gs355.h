@@ -125,7 +125,7 @@ typedef struct gs355_layout {
     size_t sort_hist;     /* u32[...] per-block digit histograms of the radix sort */
     size_t ranges;        /* u32[tiles][2] */
     size_t bin_matrix;    /* u32[slices][tiles] pairs per (slice of Gaussians, tile), then their prefix over slices */
-    size_t tile_base;     /* u32[tiles]      first slot of each tile's bucket */
+    size_t tile_base;     /* u32[2][tiles]   first slot of each tile's bucket; its next free slot during the scatter */
     size_t bin_visible;   /* u32[slices]     visible Gaussians per slice */
     size_t tile_lists;    /* u32[4+4*tiles]  counts and lists of the buckets of each larger sorter size class */
     size_t total_bytes;
@@ -148,12 +148,14 @@ enum {
      * (no per-block culling).  Produces the same image as GS355_STAGE_BLEND; not part of GS355_STAGE_ALL. */
     GS355_STAGE_BLEND_PLAIN = 64,
     /* Tile-bucketed equivalent of SCAN + DUPLICATE + SORT + RANGES: same sorted keys, values, ranges and
-     * header, far less memory traffic, no global atomics.
+     * header, far less memory traffic.
      *   TILE_COUNT    pairs per (slice of Gaussians, tile) in LDS-private counters; prefix over slices; tile
-     *                 bases = ranges; header (key count, overflow, visible count)
-     *   TILE_SCATTER  (depth bits << 32 | index) pairs into their tile's bucket
+     *                 bases = ranges; header (key count, overflow, visible count).  Beyond 36000 tiles the
+     *                 slices count per bin of 16 consecutive tiles and the tiles' totals are summed with
+     *                 global atomics.
+     *   TILE_SCATTER  (depth bits << 32 | index) pairs into bins of 16 tiles, then into their tile's bucket
      *   TILESORT      every bucket sorted by (depth bits, index) in LDS
-     * Needs tiles <= 36000 (the counters of one workgroup live in LDS); larger images use the classic stages. */
+     * Needs tiles <= 576000 (every 8K image and beyond) and P <= 2^28; otherwise use the classic stages. */
     GS355_STAGE_TILE_COUNT = 128,
     GS355_STAGE_TILESORT = 256,
     GS355_STAGE_TILE_SCATTER = 512,

@@ -16,7 +16,8 @@ STAGE_ALL = 63
 STAGE_BLEND_PLAIN = 64
 STAGE_TILE_COUNT, STAGE_TILESORT, STAGE_TILE_SCATTER = 128, 256, 512
 PIPELINE_FAST = STAGE_PREPROCESS | STAGE_TILE_COUNT | STAGE_TILE_SCATTER | STAGE_TILESORT | STAGE_BLEND
-MAX_FAST_TILES = 36000
+MAX_FAST_TILES = 36000 * 16  # limits of the tile-bucketed stages (the classic stages have neither)
+MAX_FAST_GAUSSIANS = 1 << 28
 DECODE_COUNT, DECODE_EMIT, DECODE_ALL = 1, 2, 3
 
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",

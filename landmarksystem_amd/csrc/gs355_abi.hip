@@ -85,9 +85,8 @@ int make_layout(int32_t P, int64_t n_cap, int32_t W, int32_t H, gs355_layout* L)
     L->values[1] = take(n * sizeof(uint32_t));
     L->sort_hist = take(hist_words * sizeof(uint32_t));
     L->ranges = take(tiles * 2 * sizeof(uint32_t));
-    const size_t slices = tiles <= (size_t)kBinMaxTiles ? (size_t)kBinMaxGroups : 0;
-    L->bin_matrix = take(slices * tiles * sizeof(uint32_t));
-    L->tile_base = take(tiles * sizeof(uint32_t));
+    L->bin_matrix = take((tiles <= (size_t)kBinMaxTilesWide ? bin_matrix_words(tiles) : 0) * sizeof(uint32_t));
+    L->tile_base = take(2 * tiles * sizeof(uint32_t));
     L->bin_visible = take((size_t)kBinMaxGroups * sizeof(uint32_t));
     L->tile_lists = take((4 + 4 * tiles) * sizeof(uint32_t));
     L->total_bytes = off;
@@ -199,10 +198,14 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     if ((stage_mask & (GS355_STAGE_BLEND | GS355_STAGE_BLEND_PLAIN)) && !out->image) return set_error(GS355_EINVAL, "outputs.image is NULL");
     gs355_layout L;
     if ((rc = make_layout(g->P, n_cap, frame->image_width, frame->image_height, &L))) return rc;
-    if ((stage_mask & (GS355_STAGE_TILE_COUNT | GS355_STAGE_TILE_SCATTER | GS355_STAGE_TILESORT)) &&
-        (int64_t)((frame->image_width + kTile - 1) / kTile) * ((frame->image_height + kTile - 1) / kTile) > kBinMaxTiles)
-        return set_error(GS355_EINVAL, "the tile-bucketed stages support at most %d tiles; use the classic stages",
-                         kBinMaxTiles);
+    if (stage_mask & (GS355_STAGE_TILE_COUNT | GS355_STAGE_TILE_SCATTER | GS355_STAGE_TILESORT)) {
+        if ((int64_t)((frame->image_width + kTile - 1) / kTile) * ((frame->image_height + kTile - 1) / kTile) > kBinMaxTilesWide)
+            return set_error(GS355_EINVAL, "the tile-bucketed stages support at most %d tiles; use the classic stages",
+                             kBinMaxTilesWide);
+        if (g->P > kCoarseMaxGaussians)
+            return set_error(GS355_EINVAL, "the tile-bucketed stages support at most %d Gaussians; use the classic stages",
+                             kCoarseMaxGaussians);
+    }
     if (!workspace) return set_error(GS355_EINVAL, "workspace is NULL");
     if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
         return set_error(GS355_EINVAL, "workspace must be 256-byte aligned");
@@ -252,7 +255,9 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
             return rc;
     }
     if (stage_mask & GS355_STAGE_TILE_SCATTER)
-        if ((rc = launch_tile_scatter(fa, g->P, rects, depth_bits, header, bin_matrix, tile_base, buckets, s)))
+        // (the buffer the sorted keys will go to is free until the sort: it holds the coarse level of the scatter)
+        if ((rc = launch_tile_scatter(fa, g->P, rects, depth_bits, header, bin_matrix, bin_visible, cap, tile_base, ranges,
+                                      tile_lists, buckets, keys[L.sorted_buffer], s)))
             return rc;
     if (stage_mask & GS355_STAGE_TILESORT)
         if ((rc = launch_tile_sort(header, tiles, ranges, tile_lists, buckets, keys[L.sorted_buffer],

@@ -26,53 +26,155 @@ constexpr int kInlineTiles = 32;  // splats touching more tiles than this are ex
 constexpr int kBinItems = 4;      // Gaussians per thread and round of the binning walk
 
 // ---------------------------------------------------------------------------
-// Binning.  Workgroup c owns Gaussians [c * per_group, (c+1) * per_group) and a
-// private array of per-tile counters in LDS, so no global atomic is ever issued:
-//   count:   s_tile[t] = pairs of this slice that fall in tile t  -> matrix[c][t]
-//   scatter: s_tile[t] = first free slot of tile t for this slice (tile base +
-//            the slices before it), bumped per pair -> buckets[slot]
-// A thread walks the tile rectangle of its own Gaussian; rectangles of more
-// than kInlineTiles tiles are queued and walked by all threads together.
-template <bool kScatter>
-__global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P, int per_group,
-                                                          const uint64_t* __restrict__ rects,
-                                                          const uint32_t* __restrict__ depth_bits,
-                                                          const gs355_header* __restrict__ header,
-                                                          uint32_t* __restrict__ matrix,
-                                                          const uint32_t* __restrict__ tile_base,
-                                                          uint32_t* __restrict__ group_visible,
-                                                          uint64_t* __restrict__ buckets)
+// Counting.  Workgroup c owns Gaussians [c * per_group, (c+1) * per_group) and a private array of counters in LDS.
+//   up to kBinMaxTiles tiles:  one counter per tile; matrix[c][t] = pairs of this slice that fall in tile t.  No
+//                              global atomic is issued anywhere on this path.
+//   more tiles (kWide):        one counter per coarse bin of kCoarseTiles consecutive tiles, matrix[c][b]; the
+//                              tiles' own totals are counted later, from the pairs of each bin (fine_count_kernel).
+// A thread walks the tile rectangle of its own Gaussian; rectangles of more than kInlineTiles tiles are queued and
+// walked by all threads together.
+template <bool kWide>
+__global__ __launch_bounds__(kBinThreads) void tile_count_kernel(FrameArgs f, int32_t P, int per_group,
+                                                                 const uint64_t* __restrict__ rects,
+                                                                 uint32_t* __restrict__ matrix,
+                                                                 uint32_t* __restrict__ group_visible)
 {
-    extern __shared__ uint32_t s_tile[];  // [tiles]
+    extern __shared__ uint32_t s_count[];  // [tiles], or [coarse bins] when kWide
     __shared__ uint32_t s_queue[kBinItems * kBinThreads];
     __shared__ uint32_t s_nqueue, s_visible;
 
-    if (kScatter && header->overflow) return;
     if (f.p_device) {  // the slices follow the device-side count: as many Gaussians per workgroup as on the host side
         P = effective_count(f, P);
         per_group = (P + (int)gridDim.x - 1) / (int)gridDim.x;
         per_group = max(kBinThreads, (per_group + kBinThreads - 1) / kBinThreads * kBinThreads);
     }
     const int T = f.grid_x * f.grid_y;
+    const int counters = kWide ? (T + kCoarseTiles - 1) >> kCoarseShift : T;
     const int tid = threadIdx.x, c = blockIdx.x;
-    uint32_t* __restrict__ row = matrix + (size_t)c * T;
-    for (int t = tid; t < T; t += kBinThreads) s_tile[t] = kScatter ? tile_base[t] + row[t] : 0u;
+    for (int t = tid; t < counters; t += kBinThreads) s_count[t] = 0u;
     if (tid == 0) s_visible = 0;
     const int g_begin = min(P, c * per_group);
     const int g_end = min(P, g_begin + per_group);
     uint32_t visible = 0;
+    auto add = [&](int t) { atomicAdd(&s_count[kWide ? t >> kCoarseShift : t], 1u); };
 
     for (int base = g_begin; base < g_end; base += kBinItems * kBinThreads) {
         if (tid == 0) s_nqueue = 0;
         __syncthreads();
-        // a thread's Gaussians of this round: their rectangles (and depths) are requested together
+        // a thread's Gaussians of this round: their rectangles are requested together
+        uint64_t rr[kBinItems];
+#pragma unroll
+        for (int u = 0; u < kBinItems; ++u) rr[u] = rects[min(base + u * kBinThreads + tid, g_end - 1)];
+#pragma unroll
+        for (int u = 0; u < kBinItems; ++u) {
+            const int i = base + u * kBinThreads + tid;
+            if (i < g_end) {
+                const uint64_t r = rr[u];
+                const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
+                          y1 = (int)(r >> 48);
+                const int area = (x1 - x0) * (y1 - y0);
+                if (area > 0) {
+                    ++visible;
+                    if (area > kInlineTiles) {
+                        s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
+                    } else {
+                        for (int ty = y0; ty < y1; ++ty)
+                            for (int tx = x0; tx < x1; ++tx) add(ty * f.grid_x + tx);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const uint32_t nq = s_nqueue;
+        for (uint32_t k = 0; k < nq; ++k) {
+            const uint64_t r = rects[s_queue[k]];
+            const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
+                      y1 = (int)(r >> 48);
+            const int w = x1 - x0, area = w * (y1 - y0);
+            for (int e = tid; e < area; e += kBinThreads) add((y0 + e / w) * f.grid_x + x0 + e % w);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) visible += __shfl_down(visible, d, 64);
+    if ((tid & 63) == 0 && visible) atomicAdd(&s_visible, visible);
+    __syncthreads();
+    uint32_t* __restrict__ row = matrix + (size_t)c * counters;
+    for (int t = tid; t < counters; t += kBinThreads) row[t] = s_count[t];
+    if (tid == 0) group_visible[c] = s_visible;
+}
+
+// ---------------------------------------------------------------------------
+// Two-level scatter.  Writing every pair straight into its tile's bucket spreads
+// a workgroup's stores over thousands of buckets: each 8-byte store then costs a
+// whole 32-byte sector of memory traffic.  Instead the pairs go first into
+// coarse bins of kCoarseTiles consecutive tiles (a workgroup keeps a few hundred
+// write streams going, which the L2 merges into full lines), then one workgroup
+// per coarse bin reads its bin back (contiguous) and spreads it over the bin's
+// 16 buckets (16 write streams).  The coarse bin of tiles [16 b, 16 b + 16) is
+// the concatenation of their buckets, so the same slot arithmetic serves both
+// levels: a slice's pairs of bin b start at tile_base[16 b] plus the sum of the
+// slice prefixes of the bin's tiles.  A coarse pair carries the tile's position
+// within its bin in the low four bits of the index word.
+
+// First level: the walk of the binning kernels with one cursor per coarse bin.  The tiles of one rectangle row are
+// consecutive, so a row takes one slot request per coarse bin it crosses instead of one per tile.  (Two variants
+// were measured slower: staging each round in LDS ordered by bin, so that consecutive lanes store consecutive
+// pairs, walks the rectangles twice; walking a thread's rectangles side by side to keep several slot requests in
+// flight costs more in bookkeeping than the latency it hides.)
+template <bool kWide>
+__global__ __launch_bounds__(kBinThreads) void coarse_scatter_kernel(FrameArgs f, int32_t P, int per_group,
+                                                                     const uint64_t* __restrict__ rects,
+                                                                     const uint32_t* __restrict__ depth_bits,
+                                                                     const gs355_header* __restrict__ header,
+                                                                     const uint32_t* __restrict__ matrix,
+                                                                     const uint32_t* __restrict__ base,
+                                                                     uint64_t* __restrict__ coarse)
+{
+    extern __shared__ uint32_t s_bin[];  // [coarse bins] next free slot of this slice in each bin
+    __shared__ uint32_t s_queue[kBinItems * kBinThreads];
+    __shared__ uint32_t s_nqueue;
+
+    if (header->overflow) return;
+    if (f.p_device) {
+        P = effective_count(f, P);
+        per_group = (P + (int)gridDim.x - 1) / (int)gridDim.x;
+        per_group = max(kBinThreads, (per_group + kBinThreads - 1) / kBinThreads * kBinThreads);
+    }
+    const int T = f.grid_x * f.grid_y, bins = (T + kCoarseTiles - 1) >> kCoarseShift;
+    const int tid = threadIdx.x, c = blockIdx.x, wave = tid >> 6, lane = tid & 63;
+    // a bin's first slot for this slice: the bin's base (kWide: base[b]; else the base of the bin's first tile)
+    // plus what the earlier slices put into it (the matrix holds that per bin when kWide, else per tile)
+    const uint32_t* __restrict__ row = matrix + (size_t)c * (kWide ? bins : T);
+    for (int b = tid; b < bins; b += kBinThreads) s_bin[b] = kWide ? base[b] + row[b] : base[b << kCoarseShift];
+    if (!kWide) {
+        __syncthreads();
+        for (int t = tid; t < T; t += kBinThreads) {
+            const uint32_t before = row[t];
+            if (before) atomicAdd(&s_bin[t >> kCoarseShift], before);
+        }
+    }
+    const int g_begin = min(P, c * per_group);
+    const int g_end = min(P, g_begin + per_group);
+    // the tiles [ta, tb) of one rectangle row, cut where they cross into the next bin
+    auto emit_row = [&](int ta, int tb, uint64_t payload) {
+        while (ta < tb) {
+            const int stop = min(tb, ((ta >> kCoarseShift) + 1) << kCoarseShift);
+            uint32_t slot = atomicAdd(&s_bin[ta >> kCoarseShift], (uint32_t)(stop - ta));
+            for (; ta < stop; ++ta) coarse[slot++] = payload | (uint64_t)(ta & (kCoarseTiles - 1));
+        }
+    };
+
+    for (int base = g_begin; base < g_end; base += kBinItems * kBinThreads) {
+        if (tid == 0) s_nqueue = 0;
+        __syncthreads();
         uint64_t rr[kBinItems];
         uint32_t dd[kBinItems];
 #pragma unroll
         for (int u = 0; u < kBinItems; ++u) {
             const int i = min(base + u * kBinThreads + tid, g_end - 1);
             rr[u] = rects[i];
-            dd[u] = kScatter ? depth_bits[i] : 0u;
+            dd[u] = depth_bits[i];
         }
 #pragma unroll
         for (int u = 0; u < kBinItems; ++u) {
@@ -81,47 +183,182 @@ __global__ __launch_bounds__(kBinThreads) void bin_kernel(FrameArgs f, int32_t P
                 const uint64_t r = rr[u];
                 const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
                           y1 = (int)(r >> 48);
-                const int w = x1 - x0, area = w * (y1 - y0);
-                if (area > 0) {
-                    ++visible;
-                    if (area > kInlineTiles) {
-                        s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
-                    } else {
-                        const uint64_t payload = kScatter ? ((uint64_t)dd[u] << 32) | (uint64_t)(uint32_t)i : 0ull;
-                        for (int ty = y0; ty < y1; ++ty)
-                            for (int tx = x0; tx < x1; ++tx) {
-                                const uint32_t slot = atomicAdd(&s_tile[ty * f.grid_x + tx], 1u);
-                                if (kScatter) buckets[slot] = payload;
-                            }
-                    }
+                const int area = (x1 - x0) * (y1 - y0);
+                if (area > kInlineTiles) {
+                    s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
+                } else if (area > 0) {
+                    const uint64_t payload = ((uint64_t)dd[u] << 32) | ((uint64_t)(uint32_t)i << kCoarseShift);
+                    for (int ty = y0; ty < y1; ++ty) emit_row(ty * f.grid_x + x0, ty * f.grid_x + x1, payload);
                 }
             }
         }
         __syncthreads();
+        // large rectangles: one per wavefront at a time, 64 tiles per step
         const uint32_t nq = s_nqueue;
-        for (uint32_t k = 0; k < nq; ++k) {
+        for (uint32_t k = wave; k < nq; k += kBinThreads / 64) {
             const uint32_t gi = s_queue[k];
             const uint64_t r = rects[gi];
             const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
                       y1 = (int)(r >> 48);
             const int w = x1 - x0, area = w * (y1 - y0);
-            const uint64_t payload = kScatter ? ((uint64_t)depth_bits[gi] << 32) | (uint64_t)gi : 0ull;
-            for (int e = tid; e < area; e += kBinThreads) {
-                const int ty = y0 + e / w, tx = x0 + e % w;
-                const uint32_t slot = atomicAdd(&s_tile[ty * f.grid_x + tx], 1u);
-                if (kScatter) buckets[slot] = payload;
+            const uint64_t payload = ((uint64_t)depth_bits[gi] << 32) | ((uint64_t)gi << kCoarseShift);
+            for (int e = lane; e < area; e += 64) {
+                const int t = (y0 + e / w) * f.grid_x + x0 + e % w;
+                const uint32_t slot = atomicAdd(&s_bin[t >> kCoarseShift], 1u);
+                coarse[slot] = payload | (uint64_t)(t & (kCoarseTiles - 1));
             }
         }
         __syncthreads();
     }
-    if (!kScatter) {
-#pragma unroll
-        for (int d = 32; d > 0; d >>= 1) visible += __shfl_down(visible, d, 64);
-        if ((tid & 63) == 0 && visible) atomicAdd(&s_visible, visible);
+}
+
+// Second level: the pairs of a coarse bin (contiguous) go to the buckets of the bin's tiles.  kFineSplit workgroups
+// share a bin, each taking every kFineSplit-th chunk of it (bins differ in size by a factor of several, and one
+// workgroup per bin would leave the largest for last).  A chunk is split by tile inside LDS first (wave-level ranking
+// by the four tile bits, a scan over the 8 x 16 per-wave counts), the workgroup reserves a run of slots per bucket
+// with one global atomic each, and consecutive lanes then store consecutive pairs of one bucket: full-line writes
+// instead of one memory transaction per pair.  Order inside a bucket is arbitrary, as the sort expects.
+constexpr int kFineThreads = 512;
+constexpr int kFineWaves = kFineThreads / 64;
+constexpr int kFineItems = 8;                             // pairs per thread and chunk
+constexpr int kFineChunk = kFineThreads * kFineItems;  // 4096 pairs = 32 KB of LDS
+constexpr int kFineSplit = 1 << (kCoarseShift - 1);  // workgroups per bin
+__global__ __launch_bounds__(kFineThreads) void fine_scatter_kernel(const gs355_header* __restrict__ header,
+                                                                    const uint32_t* __restrict__ tile_base,
+                                                                    uint32_t* __restrict__ cursor, int T,
+                                                                    const uint64_t* __restrict__ coarse,
+                                                                    uint64_t* __restrict__ buckets)
+{
+    __shared__ uint64_t s_stage[kFineChunk];
+    __shared__ uint32_t s_count[kFineWaves][kCoarseTiles];  // pairs per (wavefront, tile) of the chunk, then their offsets
+    __shared__ uint32_t s_start[kCoarseTiles + 1];          // first staged position of each tile's pairs
+    __shared__ uint32_t s_slot[kCoarseTiles];               // first reserved slot of each bucket for this chunk
+    if (header->overflow) return;
+    const int t0 = ((int)blockIdx.x / kFineSplit) << kCoarseShift;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const uint32_t begin = tile_base[t0];
+    const uint32_t end = t0 + kCoarseTiles < T ? tile_base[t0 + kCoarseTiles] : header->num_keys;
+    const uint64_t lanes_below = (1ull << lane) - 1ull;
+    for (uint32_t j0 = begin + (blockIdx.x % kFineSplit) * (uint32_t)kFineChunk; j0 < end;
+         j0 += (uint32_t)(kFineSplit * kFineChunk)) {
+        for (int k = tid; k < kFineWaves * kCoarseTiles; k += kFineThreads) (&s_count[0][0])[k] = 0;
         __syncthreads();
-        for (int t = tid; t < T; t += kBinThreads) row[t] = s_tile[t];
-        if (tid == 0) group_visible[c] = s_visible;
+        const uint32_t n = min((uint32_t)kFineChunk, end - j0);
+        // a wavefront owns kFineItems x 64 consecutive pairs of the chunk
+        uint64_t v[kFineItems];
+        uint32_t rank[kFineItems];
+#pragma unroll
+        for (int u = 0; u < kFineItems; ++u) {
+            const uint32_t p = (uint32_t)(wave * kFineItems + u) * 64u + lane;
+            v[u] = p < n ? coarse[j0 + p] : 0ull;
+        }
+#pragma unroll
+        for (int u = 0; u < kFineItems; ++u) {
+            const uint32_t p = (uint32_t)(wave * kFineItems + u) * 64u + lane;
+            const bool valid = p < n;
+            const uint32_t d = (uint32_t)v[u] & (kCoarseTiles - 1);
+            uint64_t peers = __ballot(valid);
+#pragma unroll
+            for (int bit = 0; bit < kCoarseShift; ++bit) {
+                const bool one = (d >> bit) & 1u;
+                const uint64_t m = __ballot(one);
+                peers &= one ? m : ~m;
+            }
+            uint32_t before = 0;
+            if (valid) {
+                const int leader = __ffsll((unsigned long long)peers) - 1;
+                if (lane == leader) before = atomicAdd(&s_count[wave][d], (uint32_t)__popcll(peers));
+                before = __shfl(before, leader, 64);
+            }
+            rank[u] = before + (uint32_t)__popcll(peers & lanes_below);
+        }
+        __syncthreads();
+        if (tid < kCoarseTiles) {  // per tile: its total in the chunk, and the slots it gets in its bucket
+            uint32_t total = 0;
+#pragma unroll
+            for (int w = 0; w < kFineWaves; ++w) {
+                const uint32_t c = s_count[w][tid];
+                s_count[w][tid] = total;  // pairs of this tile in earlier wavefronts
+                total += c;
+            }
+            s_start[tid + 1] = total;
+            s_slot[tid] = total && t0 + tid < T ? atomicAdd(&cursor[t0 + tid], total) : 0u;
+        }
+        __syncthreads();
+        if (tid < 64) {  // exclusive scan of the tiles' totals (at most 64 tiles per bin)
+            const uint32_t c = tid < kCoarseTiles ? s_start[tid + 1] : 0u;
+            uint32_t inc = c;
+#pragma unroll
+            for (int d = 1; d < kCoarseTiles; d <<= 1) {
+                const uint32_t up = __shfl_up(inc, d, 64);
+                if (lane >= d) inc += up;
+            }
+            if (tid < kCoarseTiles) s_start[tid] = inc - c;  // (the reads above are this wavefront's own, already done)
+            if (tid == kCoarseTiles - 1) s_start[kCoarseTiles] = inc;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < kFineItems; ++u) {
+            const uint32_t p = (uint32_t)(wave * kFineItems + u) * 64u + lane;
+            if (p < n) {
+                const uint32_t d = (uint32_t)v[u] & (kCoarseTiles - 1);
+                s_stage[s_start[d] + s_count[wave][d] + rank[u]] = v[u];
+            }
+        }
+        __syncthreads();
+        for (uint32_t p = tid; p < n; p += kFineThreads) {
+            const uint64_t pair = s_stage[p];
+            const uint32_t low = (uint32_t)pair, d = low & (kCoarseTiles - 1);
+            const uint32_t slot = s_slot[d] + (p - s_start[d]);
+            // (a slot outside the bin cannot happen with pairs the coarse level wrote; the test keeps corrupted input
+            // from reaching other memory)
+            if (slot >= begin && slot < end) buckets[slot] = (pair & 0xFFFFFFFF00000000ull) | (uint64_t)(low >> kCoarseShift);
+        }
+        __syncthreads();
     }
+}
+
+// Pairs per tile, counted from the coarse bins (images of more tiles than a slice can count in LDS): same chunks
+// as the fine scatter, a wavefront-level count by the four tile bits, one global atomic per tile and chunk.
+// `bin_base` [bins]: first pair of each bin; `totals` [T] cleared beforehand.
+__global__ __launch_bounds__(kFineThreads) void fine_count_kernel(const gs355_header* __restrict__ header,
+                                                                  const uint32_t* __restrict__ bin_base, int bins,
+                                                                  int T, const uint64_t* __restrict__ coarse,
+                                                                  uint32_t* __restrict__ totals)
+{
+    __shared__ uint32_t s_count[kCoarseTiles];
+    if (header->overflow) return;
+    const int b = (int)blockIdx.x / kFineSplit, t0 = b << kCoarseShift;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const uint32_t begin = bin_base[b];
+    const uint32_t end = b + 1 < bins ? bin_base[b + 1] : header->num_keys;
+    if (tid < kCoarseTiles) s_count[tid] = 0;
+    __syncthreads();
+    for (uint32_t j0 = begin + (blockIdx.x % kFineSplit) * (uint32_t)kFineChunk; j0 < end;
+         j0 += (uint32_t)(kFineSplit * kFineChunk)) {
+        const uint32_t n = min((uint32_t)kFineChunk, end - j0);
+        uint64_t v[kFineItems];
+#pragma unroll
+        for (int u = 0; u < kFineItems; ++u) {
+            const uint32_t p = (uint32_t)(u * kFineThreads + tid);
+            v[u] = p < n ? coarse[j0 + p] : 0ull;
+        }
+#pragma unroll
+        for (int u = 0; u < kFineItems; ++u) {
+            const bool valid = (uint32_t)(u * kFineThreads + tid) < n;
+            const uint32_t d = (uint32_t)v[u] & (kCoarseTiles - 1);
+            uint64_t peers = __ballot(valid);
+#pragma unroll
+            for (int bit = 0; bit < kCoarseShift; ++bit) {
+                const bool one = (d >> bit) & 1u;
+                const uint64_t m = __ballot(one);
+                peers &= one ? m : ~m;
+            }
+            if (valid && lane == __ffsll((unsigned long long)peers) - 1) atomicAdd(&s_count[d], (uint32_t)__popcll(peers));
+        }
+    }
+    __syncthreads();
+    if (tid < kCoarseTiles && t0 + tid < T && s_count[tid]) atomicAdd(&totals[t0 + tid], s_count[tid]);
 }
 
 // Exclusive prefix of every tile's counts over the slices (in place) and the
@@ -169,20 +406,24 @@ __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict_
             }
         }
     }
-    if (live && part == 0) totals[t] = total;
+    if (live && part == 0 && totals) totals[t] = total;
 }
 
 // One workgroup: tile totals -> tile bases, ranges, the frame header and the
 // lists of buckets too large for the small sorter.  `totals` and `tile_base`
-// may be the same array.
+// may be the same array.  With kTiles false the columns are coarse bins: only
+// their bases (tile_base[0, tiles)) and the header are written.
+template <bool kTiles>
 __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* totals, uint32_t tiles,
                                                            const uint32_t* __restrict__ group_visible, int groups,
                                                            uint32_t n_cap, gs355_header* __restrict__ header,
-                                                           uint32_t* tile_base, uint32_t* __restrict__ ranges,
-                                                           uint32_t* __restrict__ lists)
+                                                           bool header_known, uint32_t* tile_base,
+                                                           uint32_t* __restrict__ ranges, uint32_t* __restrict__ lists)
 {
     __shared__ uint64_t s_wave[16];
     __shared__ uint32_t s_nlist[4], s_vis;
+    // (second layout of a frame, by tile after the one by coarse bin: the header stands; nothing to do on overflow)
+    if (header_known && header->overflow) return;
     if (threadIdx.x == 0) {
         s_nlist[0] = s_nlist[1] = s_nlist[2] = s_nlist[3] = 0;
         s_vis = 0;
@@ -227,7 +468,7 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
         total += s_wave[w];
     }
     const bool overflow = total > (uint64_t)n_cap;
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0 && !header_known) {
         header->num_keys_total = total;
         header->num_keys = overflow ? n_cap : (uint32_t)total;
         header->overflow = overflow ? 1u : 0u;
@@ -244,9 +485,14 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
       for (int k = 0; k < 8; ++k) {
         const uint32_t t = tb + k, v = batch[k];
         if (t >= t1) break;
+        tile_base[t] = first;
+        if (!kTiles) {
+            first += v;
+            continue;
+        }
         ranges[2 * t] = v ? first : 0u;
         ranges[2 * t + 1] = v ? first + v : 0u;
-        tile_base[t] = first;
+        tile_base[tiles + t] = first;  // the bucket's next free slot during the scatter
         // buckets beyond the smallest sorter's capacity go on the list of their size class
         int cls = -1;
         if (v > (uint32_t)kTileSortCap[3]) cls = 3;
@@ -258,7 +504,7 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
       }
     }
     __syncthreads();
-    if (threadIdx.x < 4) lists[threadIdx.x] = s_nlist[threadIdx.x];
+    if (kTiles && threadIdx.x < 4) lists[threadIdx.x] = s_nlist[threadIdx.x];
 }
 
 constexpr int kThreads = 256;
@@ -885,8 +1131,9 @@ static int allow_large_lds()
     if (dev < 0 || dev >= kMaxDevices) return set_error(GS355_EINVAL, "device index %d is outside [0, %d)", dev, kMaxDevices);
     if (done[dev].load(std::memory_order_acquire)) return GS355_OK;
     const size_t bin_bytes = (size_t)kBinMaxTiles * sizeof(uint32_t);
-    if ((e = raise_lds_limit(bin_kernel<false>, bin_bytes)) != hipSuccess ||
-        (e = raise_lds_limit(bin_kernel<true>, bin_bytes)) != hipSuccess ||
+    if ((e = raise_lds_limit(tile_count_kernel<false>, bin_bytes)) != hipSuccess ||
+        (e = raise_lds_limit(tile_count_kernel<true>, bin_bytes)) != hipSuccess ||
+        (e = raise_lds_limit(coarse_scatter_kernel<true>, bin_bytes)) != hipSuccess ||
         (e = raise_lds_limit(tile_sort_list_1024x5_kernel, LdsSorter<1024, 5>::kBytes)) != hipSuccess ||
         (e = raise_lds_limit(tile_sort_list_kernel<1024, 10>, LdsSorter<1024, 10>::kBytes)) != hipSuccess)
         return set_error(GS355_EHIP, "LDS limit of the binning / tile sort kernels: %s", hipGetErrorString(e));
@@ -894,47 +1141,83 @@ static int allow_large_lds()
     return GS355_OK;
 }
 
+static inline int coarse_bins(int tiles) { return (tiles + kCoarseTiles - 1) >> kCoarseShift; }
+
 int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint32_t* matrix, uint32_t* group_visible,
                       hipStream_t s)
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
-    const size_t lds = (size_t)f.grid_x * f.grid_y * sizeof(uint32_t);
+    const int T = f.grid_x * f.grid_y;
     int rc = allow_large_lds();
     if (rc) return rc;
-    hipLaunchKernelGGL(bin_kernel<false>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, rects,
-                       (const uint32_t*)nullptr, (const gs355_header*)nullptr, matrix, (const uint32_t*)nullptr,
-                       group_visible, (uint64_t*)nullptr);
+    if (T <= kBinMaxTiles)
+        hipLaunchKernelGGL(tile_count_kernel<false>, dim3(groups), dim3(kBinThreads), (size_t)T * sizeof(uint32_t), s, f,
+                           P, per_group, rects, matrix, group_visible);
+    else
+        hipLaunchKernelGGL(tile_count_kernel<true>, dim3(groups), dim3(kBinThreads),
+                           (size_t)coarse_bins(T) * sizeof(uint32_t), s, f, P, per_group, rects, matrix, group_visible);
     GS355_CHECK_LAUNCH("bin: count");
     return GS355_OK;
 }
 
+// Up to kBinMaxTiles tiles: everything the later stages need (tile bases, cursors, ranges, size-class lists,
+// header).  Beyond: the header and the coarse bins' bases (in tile_cursor[0, bins)); the per-tile layout follows
+// in launch_tile_scatter once the pairs of each bin can be counted by tile.
 int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visible, int tiles, uint32_t n_cap,
                        gs355_header* header, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s)
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
-    hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(256), 0, s, matrix, groups, tiles,
-                       tile_base);
-    GS355_CHECK_LAUNCH("bin: slice prefix");
-    hipLaunchKernelGGL(tile_layout_kernel, dim3(1), dim3(1024), 0, s, tile_base, (uint32_t)tiles, group_visible, groups,
-                       n_cap, header, tile_base, ranges, lists);
+    if (tiles <= kBinMaxTiles) {
+        hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(256), 0, s, matrix, groups, tiles,
+                           tile_base);
+        GS355_CHECK_LAUNCH("bin: slice prefix");
+        hipLaunchKernelGGL(tile_layout_kernel<true>, dim3(1), dim3(1024), 0, s, tile_base, (uint32_t)tiles,
+                           group_visible, groups, n_cap, header, false, tile_base, ranges, lists);
+    } else {
+        const int bins = coarse_bins(tiles);
+        uint32_t* bin_base = tile_base + tiles;
+        hipLaunchKernelGGL(slice_prefix_kernel, dim3((bins + 63) / 64), dim3(256), 0, s, matrix, groups, bins, bin_base);
+        GS355_CHECK_LAUNCH("bin: slice prefix");
+        hipLaunchKernelGGL(tile_layout_kernel<false>, dim3(1), dim3(1024), 0, s, bin_base, (uint32_t)bins,
+                           group_visible, groups, n_cap, header, false, bin_base, ranges, lists);
+    }
     GS355_CHECK_LAUNCH("bin: layout");
     return GS355_OK;
 }
 
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
-                        const gs355_header* header, const uint32_t* matrix, const uint32_t* tile_base,
-                        uint64_t* buckets, hipStream_t s)
+                        gs355_header* header, const uint32_t* matrix, const uint32_t* group_visible, uint32_t n_cap,
+                        uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, uint64_t* buckets, uint64_t* coarse,
+                        hipStream_t s)
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
-    const size_t lds = (size_t)f.grid_x * f.grid_y * sizeof(uint32_t);
+    const int T = f.grid_x * f.grid_y, bins = coarse_bins(T);
+    uint32_t* tile_cursor = tile_base + T;
     int rc = allow_large_lds();
     if (rc) return rc;
-    hipLaunchKernelGGL(bin_kernel<true>, dim3(groups), dim3(kBinThreads), lds, s, f, P, per_group, rects, depth_bits,
-                       header, const_cast<uint32_t*>(matrix), tile_base, (uint32_t*)nullptr, buckets);
-    GS355_CHECK_LAUNCH("bin: scatter");
+    if (T <= kBinMaxTiles) {
+        hipLaunchKernelGGL(coarse_scatter_kernel<false>, dim3(groups), dim3(kBinThreads), (size_t)bins * sizeof(uint32_t),
+                           s, f, P, per_group, rects, depth_bits, header, matrix, tile_base, coarse);
+        GS355_CHECK_LAUNCH("bin: coarse scatter");
+    } else {
+        const uint32_t* bin_base = tile_cursor;  // (replaced by the tiles' cursors once the coarse level is done)
+        hipLaunchKernelGGL(coarse_scatter_kernel<true>, dim3(groups), dim3(kBinThreads), (size_t)bins * sizeof(uint32_t),
+                           s, f, P, per_group, rects, depth_bits, header, matrix, bin_base, coarse);
+        GS355_CHECK_LAUNCH("bin: coarse scatter");
+        if ((rc = launch_fill_u32(tile_base, (size_t)T, 0u, s))) return rc;
+        hipLaunchKernelGGL(fine_count_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, bin_base, bins,
+                           T, coarse, tile_base);
+        GS355_CHECK_LAUNCH("bin: fine count");
+        hipLaunchKernelGGL(tile_layout_kernel<true>, dim3(1), dim3(1024), 0, s, tile_base, (uint32_t)T, group_visible,
+                           groups, n_cap, header, true, tile_base, ranges, lists);
+        GS355_CHECK_LAUNCH("bin: layout");
+    }
+    hipLaunchKernelGGL(fine_scatter_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, tile_base,
+                       tile_cursor, T, coarse, buckets);
+    GS355_CHECK_LAUNCH("bin: fine scatter");
     return GS355_OK;
 }
 

@@ -119,15 +119,30 @@ int launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t s);
 // tile-bucketed path
 constexpr int kBinThreads = 1024;       // threads per binning workgroup
 constexpr int kBinMaxGroups = 256;      // binning workgroups (each owns a contiguous slice of the Gaussians)
-constexpr int kBinMaxTiles = 36000;     // per-tile counters of one workgroup must fit in LDS (4 B each)
+constexpr int kBinMaxTiles = 36000;     // counters of one workgroup that fit in LDS (4 B each)
+constexpr int kCoarseShift = 4;         // the scatter's first level: bins of 16 consecutive tiles
+constexpr int kCoarseTiles = 1 << kCoarseShift;
+// up to kBinMaxTiles tiles a slice counts per tile; beyond, per coarse bin (tile totals counted from the bins)
+constexpr int kBinMaxTilesWide = kBinMaxTiles * kCoarseTiles;
+constexpr int kCoarseMaxGaussians = 1 << (32 - kCoarseShift);  // a coarse pair's index shares its word with the tile bits
 int bin_groups(int32_t P, int* per_group);
+// words of the slice matrix: [slices][tiles], or [slices][coarse bins] beyond kBinMaxTiles tiles
+inline size_t bin_matrix_words(size_t tiles)
+{
+    const size_t columns = tiles <= (size_t)kBinMaxTiles ? tiles : (tiles + kCoarseTiles - 1) >> kCoarseShift;
+    return (size_t)kBinMaxGroups * columns;
+}
+// tile_base: u32[2][tiles] (bases, then the scatter's cursors).  Beyond kBinMaxTiles tiles launch_tile_layout
+// publishes the header and the coarse bins' bases only; ranges, lists and tile bases follow in launch_tile_scatter.
 int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint32_t* matrix, uint32_t* group_visible,
                       hipStream_t s);
 int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visible, int tiles, uint32_t n_cap,
                        gs355_header* header, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s);
+// `coarse`: a second buffer of the buckets' size (first level of the scatter)
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
-                        const gs355_header* header, const uint32_t* matrix, const uint32_t* tile_base,
-                        uint64_t* buckets, hipStream_t s);
+                        gs355_header* header, const uint32_t* matrix, const uint32_t* group_visible, uint32_t n_cap,
+                        uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, uint64_t* buckets, uint64_t* coarse,
+                        hipStream_t s);
 int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, const uint32_t* lists,
                      uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, hipStream_t s);
 

@@ -262,8 +262,9 @@ def run_stages(inputs: FrameInputs, outputs: FrameOutputs, ws: Workspace, n_cap:
 
 
 def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True,
-           ws: Optional[Workspace] = None) -> FrameOutputs:
-    """All stages of one frame.
+           ws: Optional[Workspace] = None, classic: bool = False) -> FrameOutputs:
+    """All stages of one frame (`classic`: through scan / duplicate / radix sort / ranges even where the
+    tile-bucketed stages apply; same results).
 
     The key count is only known on the device after the scan.  The header is
     copied to pinned host memory right after the scan and the remaining stages
@@ -275,10 +276,10 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
     out = FrameOutputs(inputs, want_depth, want_alpha)
     if ws.key_capacity == 0:
         ws.key_capacity = max(1 << 20, 4 * inputs.P)
-    if inputs.tiles <= _lib.MAX_FAST_TILES:
+    if not classic and inputs.tiles <= _lib.MAX_FAST_TILES and inputs.P <= _lib.MAX_FAST_GAUSSIANS:
         front = _lib.STAGE_PREPROCESS | _lib.STAGE_TILE_COUNT
         back = _lib.STAGE_TILE_SCATTER | _lib.STAGE_TILESORT | _lib.STAGE_BLEND
-    else:  # per-tile counters would not fit in LDS: classic duplicate / radix sort / ranges
+    else:  # beyond the bucketed stages' limits (images past 8K): classic duplicate / radix sort / ranges
         front = _lib.STAGE_PREPROCESS | _lib.STAGE_SCAN
         back = _lib.STAGE_DUPLICATE | _lib.STAGE_SORT | _lib.STAGE_RANGES | _lib.STAGE_BLEND
     for attempt in range(3):

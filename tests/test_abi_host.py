@@ -51,6 +51,11 @@ def test_workspace_layout_is_aligned_ordered_and_sized():
     tiles = 120 * 68
     assert L.bin_matrix - L.ranges >= tiles * 8 and L.total_bytes - L.tile_lists >= (4 + 4 * tiles) * 4
     assert L.tile_base - L.bin_matrix >= 256 * tiles * 4
+    assert L.bin_visible - L.tile_base >= 2 * tiles * 4  # bases, then the scatter's cursors
+    # beyond 36000 tiles the slices count per coarse bin of 16 tiles
+    Lw = _lib.workspace_layout(10, 10, 7680, 4320)
+    wide_tiles = 480 * 270
+    assert 256 * (wide_tiles // 16) * 4 <= Lw.tile_base - Lw.bin_matrix < 256 * (wide_tiles // 16) * 4 + 256
     assert L.sort_bits == 32 + 13 and L.sort_passes == 6 and L.sorted_buffer == 0
     L4k = _lib.workspace_layout(10, 10, 3840, 2160)
     assert L4k.sort_bits == 47 and L4k.sort_passes == 6
@@ -132,6 +137,12 @@ def test_run_validates_before_any_hip_call():
     msg = _err(_lib.GS355_ENOSPC, run, f, g, 0x1000, 1024, 100, out, _lib.STAGE_ALL)
     assert "needed" in msg
     assert "32-bit" in _err(_lib.GS355_EOVERFLOW, run, f, g, 0x1000, 1 << 30, 1 << 33, out, _lib.STAGE_ALL)
+    # limits of the tile-bucketed stages: 576000 tiles (16 x 36000), 2^28 Gaussians; the classic stages have neither
+    wide = _frame(W=16 * 1000, H=16 * 577)
+    assert "at most 576000 tiles" in _err(_lib.GS355_EINVAL, run, wide, g, 0x1000, 1 << 30, 100, out, _lib.PIPELINE_FAST)
+    assert "needed" in _err(_lib.GS355_ENOSPC, run, wide, g, 0x1000, 1024, 100, out, _lib.STAGE_ALL)
+    assert "Gaussians; use the classic" in _err(_lib.GS355_EINVAL, run, f, _gauss(P=(1 << 28) + 1), 0x1000, 1 << 30, 100,
+                                                 out, _lib.PIPELINE_FAST)
     no_img = _lib.Outputs()
     no_img.radii = 0x1000
     assert "image is NULL" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, no_img, _lib.STAGE_BLEND)

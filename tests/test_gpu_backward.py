@@ -53,7 +53,8 @@ def oracle_backward(scene, gi, gd=None, ga=None, colors=None, cov=None, sh_degre
                               None if ga is None else ga.numpy()[0]), fwd
 
 
-def abi_backward(scene, device, gi, gd=None, ga=None, colors=None, cov=None, sh_degree=None, want=pipeline.GRAD_NAMES):
+def abi_backward(scene, device, gi, gd=None, ga=None, colors=None, cov=None, sh_degree=None, want=pipeline.GRAD_NAMES,
+                 classic=False):
     """Forward and backward through pipeline.render / pipeline.render_backward (thin ctypes calls of the C ABI)."""
     s = settings_for(scene, device, sh_degree=sh_degree)
     dev = lambda t: None if t is None else t.to(device)  # noqa: E731
@@ -62,7 +63,7 @@ def abi_backward(scene, device, gi, gd=None, ga=None, colors=None, cov=None, sh_
                                scales=None if cov is not None else dev(scene.scales),
                                rotations=None if cov is not None else dev(scene.rotations), cov3D_precomp=dev(cov))
     ws = pipeline.Workspace(device)
-    out = pipeline.render(inp, ws=ws)
+    out = pipeline.render(inp, ws=ws, classic=classic)
     grads = pipeline.render_backward(inp, out, ws.buffer, dev(gi), dev(gd), dev(ga), want=want)
     torch.cuda.synchronize()
     return {k: v.cpu().numpy() for k, v in grads.items()}, out
@@ -234,15 +235,16 @@ def test_full_size_headline_frame_backward_equals_the_oracle(gpu_device):
         assert np.abs(value - again[name]).max() <= 1e-5 * scale, name
 
 
-def test_backward_after_the_classic_pipeline(gpu_device):
-    """More than 36000 tiles: the forward frame goes through scan / duplicate / radix sort / ranges; the backward
-    pass reads the same workspace arrays either way."""
+@pytest.mark.parametrize("classic", [True, False])
+def test_backward_after_either_pipeline_on_a_large_image(gpu_device, classic):
+    """More than 36000 tiles, forward through scan / duplicate / radix sort / ranges or through the bucketed stages
+    (which count per coarse bin at this size): the backward pass reads the same workspace arrays either way."""
     scene = scenes.config2(P=20_000, width=4000, height=2400)  # 250 x 150 = 37500 tiles
     # Splats up to 90 px in radius: thousands of pixels per sum.  Cotangents of one sign, as a smooth loss gives
     # them; with random signs the fp32 sums cancel to 1/100 of their terms and lose the digits the bar asks for.
     gi, gd, _ = (t.abs() for t in cotangents(scene, 4))
     ref, fwd = oracle_backward(scene, gi, gd)
-    got, out = abi_backward(scene, gpu_device, gi, gd)
+    got, out = abi_backward(scene, gpu_device, gi, gd, classic=classic)
     assert out.num_keys == fwd["num_keys"]
     for name, value in got.items():
         assert_grad_close(value, ref[name], name)

@@ -445,25 +445,41 @@ def test_splats_whose_extent_lands_on_a_tile_edge(gpu_device):
         np.testing.assert_array_equal(fast[name], ref[name], err_msg=name)
 
 
-def test_images_beyond_the_tile_bucket_limit(gpu_device):
-    """More than 36000 tiles: the per-tile counters of the bucketed stages no longer fit in LDS.  The C entry point
-    says so; the Python driver renders such frames through the classic stages, with the same result contract."""
-    scene = scenes.config2(P=20_000, width=4000, height=2400)  # 250 x 150 = 37500 tiles
+def test_images_beyond_the_lds_tile_counters(gpu_device):
+    """More than 36000 tiles: a slice's per-tile counters no longer fit in LDS, so the bucketed stages count per
+    coarse bin and sum the tiles' totals in global memory.  Same contract: keys, values and ranges bit-exact.  The
+    classic stages on the same frame give the same arrays."""
+    scene = scenes.config2(P=60_000, width=4000, height=2400)  # 250 x 150 = 37500 tiles
+    ref = oracle_render(scene)
+    fast = run_fast_path(scene, gpu_device)
+    assert fast["num_keys"] == ref["num_keys"]
+    for name in ("radii", "ranges", "sorted_keys", "sorted_values"):
+        np.testing.assert_array_equal(fast[name], ref[name], err_msg=name)
+    check_images(fast, ref, "37500 tiles, bucketed")
+    classic = run_all_stages(scene, gpu_device)
+    for name in ("ranges", "sorted_keys", "sorted_values"):
+        np.testing.assert_array_equal(classic[name], ref[name], err_msg="classic " + name)
+    # the Python driver takes the bucketed stages here
     s = settings_for(scene, gpu_device)
     d = scene.to(gpu_device)
     inp = pipeline.FrameInputs(s, d.means3D, opacities=d.opacities, shs=d.shs, scales=d.scales, rotations=d.rotations)
-    assert inp.tiles > _lib.MAX_FAST_TILES
-    out = pipeline.FrameOutputs(inp)
+    assert _lib.MAX_FAST_TILES >= inp.tiles > 36000
     ws = pipeline.Workspace(gpu_device)
-    with pytest.raises(_lib.Gs355Error, match="tiles"):
-        pipeline.run_stages(inp, out, ws, 1 << 20, _lib.PIPELINE_FAST)
+    ws.key_capacity = 4096  # far too small: the frame is redone once with the count the header reports
     got = pipeline.render(inp, ws=ws)
     torch.cuda.synchronize()
-    ref = co.render(oracle_frame(scene), oracle_gaussians(scene))
-    assert got.num_keys == ref["num_keys"]
-    np.testing.assert_array_equal(got.radii.cpu().numpy(), ref["radii"])
-    check_images(dict(image=got.image.cpu().numpy(), depth=got.depth.cpu().numpy(), alpha=got.alpha.cpu().numpy()),
-                 ref, "beyond the bucket limit")
+    assert ws.overflows == 1 and got.num_keys == ref["num_keys"]
+    np.testing.assert_array_equal(got.image.cpu().numpy(), fast["image"])
+
+
+def test_8k_frame_through_the_bucketed_stages(gpu_device):
+    """7680 x 4320 (129600 tiles): sorted keys, values and ranges against the oracle."""
+    scene = scenes.config2(P=150_000, width=7680, height=4320)
+    ref = oracle_render(scene)
+    fast = run_fast_path(scene, gpu_device)
+    for name in ("radii", "ranges", "sorted_keys", "sorted_values"):
+        np.testing.assert_array_equal(fast[name], ref[name], err_msg=name)
+    check_images(fast, ref, "8K")
 
 
 def test_non_finite_and_degenerate_inputs(gpu_device):

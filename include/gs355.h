@@ -151,14 +151,16 @@ enum {
      * header, far less memory traffic.
      *   TILE_COUNT    pairs per (slice of Gaussians, tile) in LDS-private counters; prefix over slices; tile
      *                 bases = ranges; header (key count, overflow, visible count).  Beyond 36000 tiles the
-     *                 slices count per bin of 16 consecutive tiles and the tiles' totals are summed with
-     *                 global atomics.
-     *   TILE_SCATTER  (depth bits << 32 | index) pairs into bins of 16 tiles, then into their tile's bucket
+     *                 slices count per bin of 16 consecutive tiles, and ranges follow with TILE_SCATTER.
+     *   TILE_SCATTER  (depth bits << 32 | index) pairs into their tile's bucket: straight for frames of fewer
+     *                 than 6 * 2^20 pairs, through bins of 16 consecutive tiles beyond (decided on the device;
+     *                 always beyond 36000 tiles, or with GS355_STAGE_TILE_SCATTER_TWO_LEVEL set as well)
      *   TILESORT      every bucket sorted by (depth bits, index) in LDS
      * Needs tiles <= 576000 (every 8K image and beyond) and P <= 2^28; otherwise use the classic stages. */
     GS355_STAGE_TILE_COUNT = 128,
     GS355_STAGE_TILESORT = 256,
     GS355_STAGE_TILE_SCATTER = 512,
+    GS355_STAGE_TILE_SCATTER_TWO_LEVEL = 1024, /* modifier of TILE_SCATTER: the two-level scatter whatever the key count */
     GS355_PIPELINE_FAST = 1 | 128 | 512 | 256 | 32
 };
 

@@ -15,6 +15,7 @@ STAGE_PREPROCESS, STAGE_SCAN, STAGE_DUPLICATE, STAGE_SORT, STAGE_RANGES, STAGE_B
 STAGE_ALL = 63
 STAGE_BLEND_PLAIN = 64
 STAGE_TILE_COUNT, STAGE_TILESORT, STAGE_TILE_SCATTER = 128, 256, 512
+STAGE_TILE_SCATTER_TWO_LEVEL = 1024  # modifier: the two-level scatter whatever the key count
 PIPELINE_FAST = STAGE_PREPROCESS | STAGE_TILE_COUNT | STAGE_TILE_SCATTER | STAGE_TILESORT | STAGE_BLEND
 MAX_FAST_TILES = 36000 * 16  # limits of the tile-bucketed stages (the classic stages have neither)
 MAX_FAST_GAUSSIANS = 1 << 28

@@ -105,80 +105,90 @@ __global__ __launch_bounds__(kBinThreads) void tile_count_kernel(FrameArgs f, in
 }
 
 // ---------------------------------------------------------------------------
-// Two-level scatter.  Writing every pair straight into its tile's bucket spreads
-// a workgroup's stores over thousands of buckets: each 8-byte store then costs a
-// whole 32-byte sector of memory traffic.  Instead the pairs go first into
-// coarse bins of kCoarseTiles consecutive tiles (a workgroup keeps a few hundred
-// write streams going, which the L2 merges into full lines), then one workgroup
-// per coarse bin reads its bin back (contiguous) and spreads it over the bin's
-// 16 buckets (16 write streams).  The coarse bin of tiles [16 b, 16 b + 16) is
-// the concatenation of their buckets, so the same slot arithmetic serves both
-// levels: a slice's pairs of bin b start at tile_base[16 b] plus the sum of the
-// slice prefixes of the bin's tiles.  A coarse pair carries the tile's position
-// within its bin in the low four bits of the index word.
+// Scatter.  Writing every pair straight into its tile's bucket spreads a
+// workgroup's stores over thousands of buckets: each 8-byte store then costs a
+// whole 32-byte sector of memory traffic.  Frames of many pairs therefore take
+// two levels: the pairs go first into coarse bins of kCoarseTiles consecutive
+// tiles (a workgroup keeps a few hundred write streams going, which the L2
+// merges into full lines), then workgroups read each bin back (contiguous)
+// and spread it over the bin's 16 buckets in line-sized runs.  The coarse bin of
+// tiles [16 b, 16 b + 16) is the concatenation of their buckets, so the same
+// slot arithmetic serves both levels: a slice's pairs of bin b start at
+// tile_base[16 b] plus the sum of the slice prefixes of the bin's tiles.  A
+// coarse pair carries the tile's position within its bin in the low four bits
+// of the index word.  The two launches of the second level cost some 40 us
+// whatever the frame holds, so frames below kTwoLevelMinKeys pairs scatter in
+// one level; the key count is only known on the device, so both variants are
+// launched and each returns at once when the other one applies.
+constexpr uint32_t kTwoLevelMinKeys = 6u << 20;
 
-// First level: the walk of the binning kernels with one cursor per coarse bin.  The tiles of one rectangle row are
-// consecutive, so a row takes one slot request per coarse bin it crosses instead of one per tile.  (Two variants
-// were measured slower: staging each round in LDS ordered by bin, so that consecutive lanes store consecutive
-// pairs, walks the rectangles twice; walking a thread's rectangles side by side to keep several slot requests in
-// flight costs more in bookkeeping than the latency it hides.)
-template <bool kWide>
-__global__ __launch_bounds__(kBinThreads) void coarse_scatter_kernel(FrameArgs f, int32_t P, int per_group,
-                                                                     const uint64_t* __restrict__ rects,
-                                                                     const uint32_t* __restrict__ depth_bits,
-                                                                     const gs355_header* __restrict__ header,
-                                                                     const uint32_t* __restrict__ matrix,
-                                                                     const uint32_t* __restrict__ base,
-                                                                     uint64_t* __restrict__ coarse)
+// The walk of the counting kernel with one cursor per column: a coarse bin (kShift = kCoarseShift) or a tile
+// (kShift = 0, straight into the buckets).  The tiles of one rectangle row are consecutive, so a row takes one slot
+// request per coarse bin it crosses instead of one per tile.  Runs only when min_keys <= pairs of the frame <
+// max_keys.  (Two variants were measured slower: staging each round in LDS ordered by bin, so that consecutive
+// lanes store consecutive pairs, walks the rectangles twice; walking a thread's rectangles side by side to keep
+// several slot requests in flight costs more in bookkeeping than the latency it hides.)
+template <int kShift, bool kWide>
+__global__ __launch_bounds__(kBinThreads) void scatter_kernel(FrameArgs f, int32_t P, int per_group,
+                                                              const uint64_t* __restrict__ rects,
+                                                              const uint32_t* __restrict__ depth_bits,
+                                                              const gs355_header* __restrict__ header,
+                                                              uint32_t min_keys, uint32_t max_keys,
+                                                              const uint32_t* __restrict__ matrix,
+                                                              const uint32_t* __restrict__ bases,
+                                                              uint64_t* __restrict__ dst)
 {
-    extern __shared__ uint32_t s_bin[];  // [coarse bins] next free slot of this slice in each bin
+    static_assert(!kWide || kShift > 0, "beyond kBinMaxTiles tiles only coarse bins fit in LDS");
+    extern __shared__ uint32_t s_bin[];  // [columns] next free slot of this slice in each column
     __shared__ uint32_t s_queue[kBinItems * kBinThreads];
     __shared__ uint32_t s_nqueue;
 
-    if (header->overflow) return;
+    if (header->overflow || header->num_keys < min_keys || header->num_keys >= max_keys) return;
     if (f.p_device) {
         P = effective_count(f, P);
         per_group = (P + (int)gridDim.x - 1) / (int)gridDim.x;
         per_group = max(kBinThreads, (per_group + kBinThreads - 1) / kBinThreads * kBinThreads);
     }
-    const int T = f.grid_x * f.grid_y, bins = (T + kCoarseTiles - 1) >> kCoarseShift;
+    constexpr int kSpan = 1 << kShift;
+    const int T = f.grid_x * f.grid_y, bins = (T + kSpan - 1) >> kShift;
     const int tid = threadIdx.x, c = blockIdx.x, wave = tid >> 6, lane = tid & 63;
-    // a bin's first slot for this slice: the bin's base (kWide: base[b]; else the base of the bin's first tile)
+    // a column's first slot for this slice: the column's base (kWide: bases[b]; else the base of its first tile)
     // plus what the earlier slices put into it (the matrix holds that per bin when kWide, else per tile)
     const uint32_t* __restrict__ row = matrix + (size_t)c * (kWide ? bins : T);
-    for (int b = tid; b < bins; b += kBinThreads) s_bin[b] = kWide ? base[b] + row[b] : base[b << kCoarseShift];
-    if (!kWide) {
+    for (int b = tid; b < bins; b += kBinThreads)
+        s_bin[b] = kWide ? bases[b] + row[b] : kShift ? bases[b << kShift] : bases[b] + row[b];
+    if (!kWide && kShift) {
         __syncthreads();
         for (int t = tid; t < T; t += kBinThreads) {
             const uint32_t before = row[t];
-            if (before) atomicAdd(&s_bin[t >> kCoarseShift], before);
+            if (before) atomicAdd(&s_bin[t >> kShift], before);
         }
     }
     const int g_begin = min(P, c * per_group);
     const int g_end = min(P, g_begin + per_group);
-    // the tiles [ta, tb) of one rectangle row, cut where they cross into the next bin
+    // the tiles [ta, tb) of one rectangle row, cut where they cross into the next column
     auto emit_row = [&](int ta, int tb, uint64_t payload) {
         while (ta < tb) {
-            const int stop = min(tb, ((ta >> kCoarseShift) + 1) << kCoarseShift);
-            uint32_t slot = atomicAdd(&s_bin[ta >> kCoarseShift], (uint32_t)(stop - ta));
-            for (; ta < stop; ++ta) coarse[slot++] = payload | (uint64_t)(ta & (kCoarseTiles - 1));
+            const int stop = min(tb, ((ta >> kShift) + 1) << kShift);
+            uint32_t slot = atomicAdd(&s_bin[ta >> kShift], (uint32_t)(stop - ta));
+            for (; ta < stop; ++ta) dst[slot++] = payload | (uint64_t)(ta & (kSpan - 1));
         }
     };
 
-    for (int base = g_begin; base < g_end; base += kBinItems * kBinThreads) {
+    for (int first = g_begin; first < g_end; first += kBinItems * kBinThreads) {
         if (tid == 0) s_nqueue = 0;
         __syncthreads();
         uint64_t rr[kBinItems];
         uint32_t dd[kBinItems];
 #pragma unroll
         for (int u = 0; u < kBinItems; ++u) {
-            const int i = min(base + u * kBinThreads + tid, g_end - 1);
+            const int i = min(first + u * kBinThreads + tid, g_end - 1);
             rr[u] = rects[i];
             dd[u] = depth_bits[i];
         }
 #pragma unroll
         for (int u = 0; u < kBinItems; ++u) {
-            const int i = base + u * kBinThreads + tid;
+            const int i = first + u * kBinThreads + tid;
             if (i < g_end) {
                 const uint64_t r = rr[u];
                 const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
@@ -187,7 +197,7 @@ __global__ __launch_bounds__(kBinThreads) void coarse_scatter_kernel(FrameArgs f
                 if (area > kInlineTiles) {
                     s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
                 } else if (area > 0) {
-                    const uint64_t payload = ((uint64_t)dd[u] << 32) | ((uint64_t)(uint32_t)i << kCoarseShift);
+                    const uint64_t payload = ((uint64_t)dd[u] << 32) | ((uint64_t)(uint32_t)i << kShift);
                     for (int ty = y0; ty < y1; ++ty) emit_row(ty * f.grid_x + x0, ty * f.grid_x + x1, payload);
                 }
             }
@@ -201,11 +211,11 @@ __global__ __launch_bounds__(kBinThreads) void coarse_scatter_kernel(FrameArgs f
             const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
                       y1 = (int)(r >> 48);
             const int w = x1 - x0, area = w * (y1 - y0);
-            const uint64_t payload = ((uint64_t)depth_bits[gi] << 32) | ((uint64_t)gi << kCoarseShift);
+            const uint64_t payload = ((uint64_t)depth_bits[gi] << 32) | ((uint64_t)gi << kShift);
             for (int e = lane; e < area; e += 64) {
                 const int t = (y0 + e / w) * f.grid_x + x0 + e % w;
-                const uint32_t slot = atomicAdd(&s_bin[t >> kCoarseShift], 1u);
-                coarse[slot] = payload | (uint64_t)(t & (kCoarseTiles - 1));
+                const uint32_t slot = atomicAdd(&s_bin[t >> kShift], 1u);
+                dst[slot] = payload | (uint64_t)(t & (kSpan - 1));
             }
         }
         __syncthreads();
@@ -222,8 +232,9 @@ constexpr int kFineThreads = 512;
 constexpr int kFineWaves = kFineThreads / 64;
 constexpr int kFineItems = 8;                             // pairs per thread and chunk
 constexpr int kFineChunk = kFineThreads * kFineItems;  // 4096 pairs = 32 KB of LDS
-constexpr int kFineSplit = 1 << (kCoarseShift - 1);  // workgroups per bin
+constexpr int kFineSplit = 8;   // workgroups per bin
 __global__ __launch_bounds__(kFineThreads) void fine_scatter_kernel(const gs355_header* __restrict__ header,
+                                                                    uint32_t min_keys,
                                                                     const uint32_t* __restrict__ tile_base,
                                                                     uint32_t* __restrict__ cursor, int T,
                                                                     const uint64_t* __restrict__ coarse,
@@ -233,7 +244,7 @@ __global__ __launch_bounds__(kFineThreads) void fine_scatter_kernel(const gs355_
     __shared__ uint32_t s_count[kFineWaves][kCoarseTiles];  // pairs per (wavefront, tile) of the chunk, then their offsets
     __shared__ uint32_t s_start[kCoarseTiles + 1];          // first staged position of each tile's pairs
     __shared__ uint32_t s_slot[kCoarseTiles];               // first reserved slot of each bucket for this chunk
-    if (header->overflow) return;
+    if (header->overflow || header->num_keys < min_keys) return;
     const int t0 = ((int)blockIdx.x / kFineSplit) << kCoarseShift;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const uint32_t begin = tile_base[t0];
@@ -1133,7 +1144,8 @@ static int allow_large_lds()
     const size_t bin_bytes = (size_t)kBinMaxTiles * sizeof(uint32_t);
     if ((e = raise_lds_limit(tile_count_kernel<false>, bin_bytes)) != hipSuccess ||
         (e = raise_lds_limit(tile_count_kernel<true>, bin_bytes)) != hipSuccess ||
-        (e = raise_lds_limit(coarse_scatter_kernel<true>, bin_bytes)) != hipSuccess ||
+        (e = raise_lds_limit(scatter_kernel<0, false>, bin_bytes)) != hipSuccess ||
+        (e = raise_lds_limit(scatter_kernel<kCoarseShift, true>, bin_bytes)) != hipSuccess ||
         (e = raise_lds_limit(tile_sort_list_1024x5_kernel, LdsSorter<1024, 5>::kBytes)) != hipSuccess ||
         (e = raise_lds_limit(tile_sort_list_kernel<1024, 10>, LdsSorter<1024, 10>::kBytes)) != hipSuccess)
         return set_error(GS355_EHIP, "LDS limit of the binning / tile sort kernels: %s", hipGetErrorString(e));
@@ -1190,22 +1202,30 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
                         gs355_header* header, const uint32_t* matrix, const uint32_t* group_visible, uint32_t n_cap,
                         uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, uint64_t* buckets, uint64_t* coarse,
-                        hipStream_t s)
+                        bool two_level, hipStream_t s)
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
     const int T = f.grid_x * f.grid_y, bins = coarse_bins(T);
     uint32_t* tile_cursor = tile_base + T;
+    const size_t coarse_lds = (size_t)bins * sizeof(uint32_t);
     int rc = allow_large_lds();
     if (rc) return rc;
+    uint32_t min_keys = 0;  // pairs from which the two levels run
     if (T <= kBinMaxTiles) {
-        hipLaunchKernelGGL(coarse_scatter_kernel<false>, dim3(groups), dim3(kBinThreads), (size_t)bins * sizeof(uint32_t),
-                           s, f, P, per_group, rects, depth_bits, header, matrix, tile_base, coarse);
+        if (!two_level) {
+            min_keys = kTwoLevelMinKeys;
+            hipLaunchKernelGGL((scatter_kernel<0, false>), dim3(groups), dim3(kBinThreads), (size_t)T * sizeof(uint32_t), s,
+                               f, P, per_group, rects, depth_bits, header, 0u, min_keys, matrix, tile_base, buckets);
+            GS355_CHECK_LAUNCH("bin: scatter");
+        }
+        hipLaunchKernelGGL((scatter_kernel<kCoarseShift, false>), dim3(groups), dim3(kBinThreads), coarse_lds, s, f, P,
+                           per_group, rects, depth_bits, header, min_keys, UINT32_MAX, matrix, tile_base, coarse);
         GS355_CHECK_LAUNCH("bin: coarse scatter");
     } else {
         const uint32_t* bin_base = tile_cursor;  // (replaced by the tiles' cursors once the coarse level is done)
-        hipLaunchKernelGGL(coarse_scatter_kernel<true>, dim3(groups), dim3(kBinThreads), (size_t)bins * sizeof(uint32_t),
-                           s, f, P, per_group, rects, depth_bits, header, matrix, bin_base, coarse);
+        hipLaunchKernelGGL((scatter_kernel<kCoarseShift, true>), dim3(groups), dim3(kBinThreads), coarse_lds, s, f, P,
+                           per_group, rects, depth_bits, header, 0u, UINT32_MAX, matrix, bin_base, coarse);
         GS355_CHECK_LAUNCH("bin: coarse scatter");
         if ((rc = launch_fill_u32(tile_base, (size_t)T, 0u, s))) return rc;
         hipLaunchKernelGGL(fine_count_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, bin_base, bins,
@@ -1215,8 +1235,8 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
                            groups, n_cap, header, true, tile_base, ranges, lists);
         GS355_CHECK_LAUNCH("bin: layout");
     }
-    hipLaunchKernelGGL(fine_scatter_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, tile_base,
-                       tile_cursor, T, coarse, buckets);
+    hipLaunchKernelGGL(fine_scatter_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, min_keys,
+                       tile_base, tile_cursor, T, coarse, buckets);
     GS355_CHECK_LAUNCH("bin: fine scatter");
     return GS355_OK;
 }

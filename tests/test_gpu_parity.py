@@ -223,8 +223,9 @@ def test_block_culling_is_result_neutral(gpu_device, make):
     assert float(out.alpha.max()) > 0.5
 
 
-def run_fast_path(scene, device):
-    """PREPROCESS | TILE_COUNT | TILE_SCATTER | TILESORT | BLEND over an exactly sized workspace."""
+def run_fast_path(scene, device, two_level=False):
+    """PREPROCESS | TILE_COUNT | TILE_SCATTER | TILESORT | BLEND over an exactly sized workspace (`two_level`: the
+    scatter through coarse bins, which frames of few pairs otherwise skip)."""
     s = settings_for(scene, device)
     inp = pipeline.FrameInputs(s, scene.means3D.to(device), opacities=scene.opacities.to(device),
                                shs=scene.shs.to(device), scales=scene.scales.to(device),
@@ -235,7 +236,7 @@ def run_fast_path(scene, device):
     lay = pipeline.run_stages(inp, out, ws, 0, _lib.STAGE_PREPROCESS | _lib.STAGE_TILE_COUNT)
     torch.cuda.synchronize()
     n = int(ws.view(lay, "header", P, 0, tiles)[0].item())
-    lay = pipeline.run_stages(inp, out, ws, n, _lib.PIPELINE_FAST)
+    lay = pipeline.run_stages(inp, out, ws, n, _lib.PIPELINE_FAST | (_lib.STAGE_TILE_SCATTER_TWO_LEVEL if two_level else 0))
     torch.cuda.synchronize()
     return dict(sorted_keys=u64(ws.view(lay, "sorted_keys", P, n, tiles)),
                 sorted_values=u32(ws.view(lay, "sorted_values", P, n, tiles)),
@@ -275,6 +276,11 @@ def test_tile_bucketed_path_equals_oracle(gpu_device, make, label):
     np.testing.assert_array_equal(got["ranges"], ref["ranges"], err_msg=label + " ranges")
     np.testing.assert_array_equal(got["sorted_keys"], ref["sorted_keys"], err_msg=label + " sorted keys")
     np.testing.assert_array_equal(got["sorted_values"], ref["sorted_values"], err_msg=label + " sorted values")
+    # frames this small scatter in one level; the two-level scatter (chosen on the device for frames of many pairs)
+    # gives the same arrays and, the blend reading the same lists, the same image bits
+    two = run_fast_path(scene, gpu_device, two_level=True)
+    for name in ("ranges", "sorted_keys", "sorted_values", "image", "depth", "alpha"):
+        np.testing.assert_array_equal(two[name], got[name], err_msg=label + " two-level " + name)
     # the crowded scenes are made of faint Gaussians (opacity 0.004 .. 0.024 around the 1/255 threshold)
     check_images(got, ref, label, max_fragile_frac=0.5 if "ties" in label else 0.02)
     if "ties" in label:

@@ -125,9 +125,10 @@ typedef struct gs355_layout {
     size_t sort_hist;     /* u32[...] per-block digit histograms of the radix sort */
     size_t ranges;        /* u32[tiles][2] */
     size_t bin_matrix;    /* u32[slices][tiles] pairs per (slice of Gaussians, tile), then their prefix over slices */
-    size_t tile_base;     /* u32[2][tiles]   first slot of each tile's bucket; its next free slot during the scatter */
+    size_t tile_base;     /* u32[2][tiles]   first slot of each tile's bucket; its next free slot during the scatter;
+                           * then u64[ceil(tiles/64)], the first slot of each block of 64 tiles */
     size_t bin_visible;   /* u32[slices]     visible Gaussians per slice */
-    size_t tile_lists;    /* u32[4+4*tiles]  counts and lists of the buckets of each larger sorter size class */
+    size_t tile_lists;    /* u32[8+4*tiles]  counts, work counters and lists of the buckets of each larger sorter size class */
     size_t total_bytes;
     int32_t unsorted_buffer; /* which keys/values buffer the duplicate stage writes (0) */
     int32_t sorted_buffer;   /* which buffer holds the sorted pairs after the sort stage */

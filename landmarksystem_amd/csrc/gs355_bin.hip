@@ -331,11 +331,13 @@ __global__ __launch_bounds__(kFineThreads) void fine_scatter_kernel(const gs355_
 
 // Pairs per tile, counted from the coarse bins (images of more tiles than a slice can count in LDS): same chunks
 // as the fine scatter, a wavefront-level count by the four tile bits, one global atomic per tile and chunk.
-// `bin_base` [bins]: first pair of each bin; `totals` [T] cleared beforehand.
+// `bin_base` [bins]: first pair of each bin; `totals` [T] and `block_sums` [T / 64] (pairs per 64 tiles) cleared
+// beforehand.
 __global__ __launch_bounds__(kFineThreads) void fine_count_kernel(const gs355_header* __restrict__ header,
                                                                   const uint32_t* __restrict__ bin_base, int bins,
                                                                   int T, const uint64_t* __restrict__ coarse,
-                                                                  uint32_t* __restrict__ totals)
+                                                                  uint32_t* __restrict__ totals,
+                                                                  uint64_t* __restrict__ block_sums)
 {
     __shared__ uint32_t s_count[kCoarseTiles];
     if (header->overflow) return;
@@ -369,16 +371,20 @@ __global__ __launch_bounds__(kFineThreads) void fine_count_kernel(const gs355_he
         }
     }
     __syncthreads();
-    if (tid < kCoarseTiles && t0 + tid < T && s_count[tid]) atomicAdd(&totals[t0 + tid], s_count[tid]);
+    if (tid < kCoarseTiles && t0 + tid < T && s_count[tid]) {
+        atomicAdd(&totals[t0 + tid], s_count[tid]);
+        atomicAdd(reinterpret_cast<unsigned long long*>(&block_sums[(t0 + tid) >> 6]), (unsigned long long)s_count[tid]);
+    }
 }
 
-// Exclusive prefix of every tile's counts over the slices (in place) and the
-// tile's total.  A workgroup covers 64 tiles; its four wavefronts take a
+// Exclusive prefix of every tile's counts over the slices (in place), the
+// tile's total and the total of the workgroup's tiles.  A workgroup covers 64 tiles; its four wavefronts take a
 // quarter of the slices each (loads of a thread are issued in batches, so many
 // are in flight), exchange their quarter sums through LDS and write the
 // prefixes shifted by the quarters before them.
 __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict__ matrix, int groups, int tiles,
-                                                           uint32_t* __restrict__ totals)
+                                                           uint32_t* __restrict__ totals,
+                                                           uint64_t* __restrict__ block_sums)
 {
     __shared__ uint32_t s_part[4][64];
     const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
@@ -417,48 +423,40 @@ __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict_
             }
         }
     }
-    if (live && part == 0 && totals) totals[t] = total;
+    if (part == 0) {
+        if (live) totals[t] = total;
+        uint64_t sum64 = live ? total : 0u;  // the 64 tiles of this workgroup are one block of the layout's scan
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) sum64 += __shfl_down(sum64, d, 64);
+        if (lane == 0) block_sums[blockIdx.x] = sum64;
+    }
 }
 
-// One workgroup: tile totals -> tile bases, ranges, the frame header and the
-// lists of buckets too large for the small sorter.  `totals` and `tile_base`
-// may be the same array.  With kTiles false the columns are coarse bins: only
-// their bases (tile_base[0, tiles)) and the header are written.
-template <bool kTiles>
-__global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* totals, uint32_t tiles,
-                                                           const uint32_t* __restrict__ group_visible, int groups,
-                                                           uint32_t n_cap, gs355_header* __restrict__ header,
-                                                           bool header_known, uint32_t* tile_base,
-                                                           uint32_t* __restrict__ ranges, uint32_t* __restrict__ lists)
+// Layout of the buckets from the tiles' totals, in two steps.  First one workgroup turns the totals of the blocks of
+// 64 tiles into block bases (exclusive scan, in place) and writes the frame header; the grand total decides overflow
+// before anything else is published.  `header_known`: second layout of a frame (by tile, after the one by coarse
+// bin): the header stands, and nothing is done on overflow.
+__global__ __launch_bounds__(1024) void block_scan_kernel(uint64_t* __restrict__ blocks, uint32_t n_blocks,
+                                                          const uint32_t* __restrict__ group_visible, int groups,
+                                                          uint32_t n_cap, gs355_header* __restrict__ header,
+                                                          bool header_known, uint32_t* __restrict__ lists)
 {
     __shared__ uint64_t s_wave[16];
-    __shared__ uint32_t s_nlist[4], s_vis;
-    // (second layout of a frame, by tile after the one by coarse bin: the header stands; nothing to do on overflow)
+    __shared__ uint32_t s_vis;
     if (header_known && header->overflow) return;
-    if (threadIdx.x == 0) {
-        s_nlist[0] = s_nlist[1] = s_nlist[2] = s_nlist[3] = 0;
-        s_vis = 0;
-    }
+    if (threadIdx.x == 0) s_vis = 0;
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    // Every thread owns a run of consecutive tiles, so one scan over the 1024 run sums (one barrier) places
-    // them all.  The grand total decides overflow before any range is published.
-    const uint32_t per = (tiles + 1023u) / 1024u;
-    const uint32_t t0 = min(threadIdx.x * per, tiles), t1 = min(t0 + per, tiles);
-    uint64_t mine = 0;
-    uint32_t head[8];  // the run's first 8 totals stay in registers for the second pass (all of them up to 8192 tiles)
+    // every thread owns a run of consecutive blocks (9 at most for the largest image), so one scan over the 1024 run
+    // sums places them all
+    constexpr uint32_t kRun = (kBinMaxTilesWide / 64 + 1023) / 1024;
+    const uint32_t per = (n_blocks + 1023u) / 1024u;
+    const uint32_t b0 = min(threadIdx.x * per, n_blocks), b1 = min(b0 + per, n_blocks);
+    uint64_t v[kRun], mine = 0;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) head[k] = 0;
-    for (uint32_t t = t0; t < t1; t += 8) {  // 8 loads in flight (the last batch re-reads the run's last tile)
-        uint32_t v[8];
-#pragma unroll
-        for (int k = 0; k < 8; ++k) v[k] = totals[min(t + k, t1 - 1)];
-#pragma unroll
-        for (int k = 0; k < 8; ++k) mine += t + k < t1 ? v[k] : 0u;
-        if (t == t0) {
-#pragma unroll
-            for (int k = 0; k < 8; ++k) head[k] = v[k];
-        }
+    for (uint32_t k = 0; k < kRun; ++k) {
+        v[k] = b0 + k < b1 ? blocks[b0 + k] : 0ull;
+        mine += v[k];
     }
     uint32_t vis = 0;
     for (int c = threadIdx.x; c < groups; c += 1024) vis += group_visible[c];
@@ -485,37 +483,63 @@ __global__ __launch_bounds__(1024) void tile_layout_kernel(const uint32_t* total
         header->overflow = overflow ? 1u : 0u;
         header->num_visible = s_vis;
     }
-    // bases, ranges and size-class lists of the thread's own tiles (skipped on overflow: later stages do nothing)
-    uint32_t first = (uint32_t)(before + inc - mine);
-    for (uint32_t tb = t0; tb < t1 && !overflow; tb += 8) {
-      // the batch's totals are read before any of its tile_base words (possibly the same words) is written
-      uint32_t batch[8];
+    if (threadIdx.x < 4) lists[threadIdx.x] = 0u;  // the size-class lists are filled by tile_publish_kernel
+    uint64_t first = before + inc - mine;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) batch[k] = tb == t0 ? head[k] : totals[min(tb + k, t1 - 1)];
+    for (uint32_t k = 0; k < kRun; ++k) {
+        if (b0 + k < b1) blocks[b0 + k] = first;
+        first += v[k];
+    }
+}
+
+// Second step, one wavefront per block of 64 tiles: tile bases (and, with kTiles, the scatter's cursors, the ranges
+// and the lists of buckets too large for the small sorter).  `totals` and `tile_base` may be the same array.  With
+// kTiles false the columns are coarse bins and only their bases are written.
+template <bool kTiles>
+__global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* totals, uint32_t tiles,
+                                                           const uint64_t* __restrict__ block_base,
+                                                           const gs355_header* __restrict__ header,
+                                                           uint32_t* tile_base, uint32_t* __restrict__ ranges,
+                                                           uint32_t* __restrict__ lists)
+{
+    if (header->overflow) return;  // later stages do nothing either
+    const int lane = threadIdx.x & 63;
+    const uint32_t block = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint32_t t = block * 64u + (uint32_t)lane;
+    const bool live = t < tiles;
+    const uint32_t v = live ? totals[t] : 0u;
+    uint32_t inc = v;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const uint32_t t = tb + k, v = batch[k];
-        if (t >= t1) break;
-        tile_base[t] = first;
-        if (!kTiles) {
-            first += v;
-            continue;
-        }
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = __shfl_up(inc, d, 64);
+        if (lane >= d) inc += up;
+    }
+    if (block * 64u >= tiles) return;  // (uniform per wavefront)
+    const uint32_t first = (uint32_t)block_base[block] + inc - v;
+    if (live) tile_base[t] = first;
+    if (!kTiles) return;
+    if (live) {
         ranges[2 * t] = v ? first : 0u;
         ranges[2 * t + 1] = v ? first + v : 0u;
         tile_base[tiles + t] = first;  // the bucket's next free slot during the scatter
-        // buckets beyond the smallest sorter's capacity go on the list of their size class
-        int cls = -1;
-        if (v > (uint32_t)kTileSortCap[3]) cls = 3;
-        else if (v > (uint32_t)kTileSortCap[2]) cls = 2;
-        else if (v > (uint32_t)kTileSortCap[1]) cls = 1;
-        else if (v > (uint32_t)kTileSortCap[0]) cls = 0;
-        if (cls >= 0) lists[4 + (size_t)cls * tiles + atomicAdd(&s_nlist[cls], 1u)] = t;
-        first += v;
-      }
     }
-    __syncthreads();
-    if (kTiles && threadIdx.x < 4) lists[threadIdx.x] = s_nlist[threadIdx.x];
+    // buckets beyond the smallest sorter's capacity go on the list of their size class (order within a list is free):
+    // one request per wavefront and class
+    int cls = -1;
+    if (v > (uint32_t)kTileSortCap[3]) cls = 3;
+    else if (v > (uint32_t)kTileSortCap[2]) cls = 2;
+    else if (v > (uint32_t)kTileSortCap[1]) cls = 1;
+    else if (v > (uint32_t)kTileSortCap[0]) cls = 0;
+    const uint64_t lanes_below = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint64_t m = __ballot(cls == c);
+        if (m == 0ull) continue;
+        uint32_t at = 0;
+        if (lane == __ffsll((unsigned long long)m) - 1) at = atomicAdd(&lists[c], (uint32_t)__popcll(m));
+        at = __shfl(at, __ffsll((unsigned long long)m) - 1, 64);
+        if (cls == c) lists[kListHeader + (size_t)c * tiles + at + (uint32_t)__popcll(m & lanes_below)] = t;
+    }
 }
 
 constexpr int kThreads = 256;
@@ -1035,38 +1059,53 @@ __global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* 
                                                             const uint32_t* __restrict__ ranges,
                                                             const uint64_t* __restrict__ buckets,
                                                             uint64_t* __restrict__ out_keys,
-                                                            uint32_t* __restrict__ out_vals)
+                                                            uint32_t* __restrict__ out_vals,
+                                                            uint32_t* __restrict__ list_work)
 {
     extern __shared__ uint32_t s_dyn[];
+    if (blockIdx.x == 0 && threadIdx.x < 4) list_work[threadIdx.x] = 0u;  // for the list kernels launched after this one
     if (header->overflow) return;
     const LdsSorter<kT, kR> sorter(s_dyn);
     sorter.run(blockIdx.x, ranges, buckets, out_keys, out_vals);
 }
 
-// Larger size classes: persistent workgroups over the class list made by tile_layout_kernel.
+// Larger size classes: persistent workgroups over the class list made by tile_layout_kernel.  A workgroup starts
+// with the list entry of its own number and then takes the next one nobody has taken (`work`, a counter cleared by
+// tile_sort_each_kernel): buckets of one class differ in size by a factor of two and more, and a fixed assignment
+// leaves most of the chip waiting for the workgroups that drew the large ones.  The request for the next entry is
+// issued before the current bucket is sorted, so its latency is not waited for.
 template <int kT, int kR>
 __device__ __forceinline__ void tile_sort_list_body(const gs355_header* __restrict__ header,
                                                     const uint32_t* __restrict__ ranges,
                                                     const uint32_t* __restrict__ list,
-                                                    const uint32_t* __restrict__ list_count,
+                                                    const uint32_t* __restrict__ list_count, uint32_t* __restrict__ work,
                                                     const uint64_t* __restrict__ buckets,
                                                     uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals,
                                                     uint32_t* lds)
 {
+    __shared__ uint32_t s_next;
     if (header->overflow) return;
     const LdsSorter<kT, kR> sorter(lds);
     const uint32_t count = *list_count;
-    for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) sorter.run(list[k], ranges, buckets, out_keys, out_vals);
+    uint32_t k = blockIdx.x;
+    while (k < count) {
+        uint32_t next = 0;
+        if (threadIdx.x == 0) next = atomicAdd(work, 1u) + gridDim.x;
+        sorter.run(list[k], ranges, buckets, out_keys, out_vals);  // (ends with a barrier)
+        if (threadIdx.x == 0) s_next = next;
+        __syncthreads();
+        k = s_next;  // the next write of s_next comes after the barriers of the next run
+    }
 }
 
 // 1024 threads x 5 rounds, held to 64 VGPRs so that two workgroups share a CU
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void tile_sort_list_1024x5_kernel(
     const gs355_header* __restrict__ header, const uint32_t* __restrict__ ranges, const uint32_t* __restrict__ list,
-    const uint32_t* __restrict__ list_count, const uint64_t* __restrict__ buckets, uint64_t* __restrict__ out_keys,
-    uint32_t* __restrict__ out_vals)
+    const uint32_t* __restrict__ list_count, uint32_t* __restrict__ work, const uint64_t* __restrict__ buckets,
+    uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals)
 {
     extern __shared__ uint32_t s_dyn[];
-    tile_sort_list_body<1024, 5>(header, ranges, list, list_count, buckets, out_keys, out_vals, s_dyn);
+    tile_sort_list_body<1024, 5>(header, ranges, list, list_count, work, buckets, out_keys, out_vals, s_dyn);
 }
 
 template <int kT, int kR>
@@ -1074,12 +1113,13 @@ __global__ __launch_bounds__(kT) void tile_sort_list_kernel(const gs355_header* 
                                                             const uint32_t* __restrict__ ranges,
                                                             const uint32_t* __restrict__ list,
                                                             const uint32_t* __restrict__ list_count,
+                                                            uint32_t* __restrict__ work,
                                                             const uint64_t* __restrict__ buckets,
                                                             uint64_t* __restrict__ out_keys,
                                                             uint32_t* __restrict__ out_vals)
 {
     extern __shared__ uint32_t s_dyn[];
-    tile_sort_list_body<kT, kR>(header, ranges, list, list_count, buckets, out_keys, out_vals, s_dyn);
+    tile_sort_list_body<kT, kR>(header, ranges, list, list_count, work, buckets, out_keys, out_vals, s_dyn);
 }
 
 // Buckets beyond the LDS capacity: the same passes through global memory,
@@ -1098,7 +1138,7 @@ __global__ __launch_bounds__(kThreads) void tile_sort_huge_kernel(const gs355_he
     const SortScratch sc = {s_hist, s_cnt, s_flags};
     const uint32_t count = lists[3];
     for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) {
-        const uint32_t tile = lists[4 + 3 * (size_t)tiles + k];
+        const uint32_t tile = lists[kListHeader + 3 * (size_t)tiles + k];
         const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
         const GlobalPairs A = {buckets + lo}, B = {out_keys + lo};
         const bool in_b = sort_pairs(A, B, n, sc);
@@ -1173,6 +1213,22 @@ int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint
     return GS355_OK;
 }
 
+// Bases of `columns` buckets from their totals (block sums already in `blocks`), and the per-tile outputs with kTiles.
+template <bool kTiles>
+static int launch_layout(uint32_t* totals_and_bases, int columns, uint64_t* blocks, const uint32_t* group_visible,
+                         int groups, uint32_t n_cap, gs355_header* header, bool header_known, uint32_t* ranges,
+                         uint32_t* lists, hipStream_t s)
+{
+    const int n_blocks = (columns + 63) / 64;
+    hipLaunchKernelGGL(block_scan_kernel, dim3(1), dim3(1024), 0, s, blocks, (uint32_t)n_blocks, group_visible, groups,
+                       n_cap, header, header_known, lists);
+    GS355_CHECK_LAUNCH("bin: block scan");
+    hipLaunchKernelGGL(tile_publish_kernel<kTiles>, dim3((n_blocks + 3) / 4), dim3(256), 0, s, totals_and_bases,
+                       (uint32_t)columns, blocks, header, totals_and_bases, ranges, lists);
+    GS355_CHECK_LAUNCH("bin: layout");
+    return GS355_OK;
+}
+
 // Up to kBinMaxTiles tiles: everything the later stages need (tile bases, cursors, ranges, size-class lists,
 // header).  Beyond: the header and the coarse bins' bases (in tile_cursor[0, bins)); the per-tile layout follows
 // in launch_tile_scatter once the pairs of each bin can be counted by tile.
@@ -1181,22 +1237,20 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
+    uint64_t* blocks = reinterpret_cast<uint64_t*>(tile_base + 2 * (size_t)tiles);
     if (tiles <= kBinMaxTiles) {
         hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(256), 0, s, matrix, groups, tiles,
-                           tile_base);
+                           tile_base, blocks);
         GS355_CHECK_LAUNCH("bin: slice prefix");
-        hipLaunchKernelGGL(tile_layout_kernel<true>, dim3(1), dim3(1024), 0, s, tile_base, (uint32_t)tiles,
-                           group_visible, groups, n_cap, header, false, tile_base, ranges, lists);
-    } else {
-        const int bins = coarse_bins(tiles);
-        uint32_t* bin_base = tile_base + tiles;
-        hipLaunchKernelGGL(slice_prefix_kernel, dim3((bins + 63) / 64), dim3(256), 0, s, matrix, groups, bins, bin_base);
-        GS355_CHECK_LAUNCH("bin: slice prefix");
-        hipLaunchKernelGGL(tile_layout_kernel<false>, dim3(1), dim3(1024), 0, s, bin_base, (uint32_t)bins,
-                           group_visible, groups, n_cap, header, false, bin_base, ranges, lists);
+        return launch_layout<true>(tile_base, tiles, blocks, group_visible, groups, n_cap, header, false, ranges, lists,
+                                   s);
     }
-    GS355_CHECK_LAUNCH("bin: layout");
-    return GS355_OK;
+    const int bins = coarse_bins(tiles);
+    uint32_t* bin_base = tile_base + tiles;
+    hipLaunchKernelGGL(slice_prefix_kernel, dim3((bins + 63) / 64), dim3(256), 0, s, matrix, groups, bins, bin_base,
+                       blocks);
+    GS355_CHECK_LAUNCH("bin: slice prefix");
+    return launch_layout<false>(bin_base, bins, blocks, group_visible, groups, n_cap, header, false, ranges, lists, s);
 }
 
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
@@ -1227,13 +1281,14 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
         hipLaunchKernelGGL((scatter_kernel<kCoarseShift, true>), dim3(groups), dim3(kBinThreads), coarse_lds, s, f, P,
                            per_group, rects, depth_bits, header, 0u, UINT32_MAX, matrix, bin_base, coarse);
         GS355_CHECK_LAUNCH("bin: coarse scatter");
+        uint64_t* blocks = reinterpret_cast<uint64_t*>(tile_base + 2 * (size_t)T);
         if ((rc = launch_fill_u32(tile_base, (size_t)T, 0u, s))) return rc;
+        if ((rc = launch_fill_u32(reinterpret_cast<uint32_t*>(blocks), 2 * (size_t)((T + 63) / 64), 0u, s))) return rc;
         hipLaunchKernelGGL(fine_count_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, bin_base, bins,
-                           T, coarse, tile_base);
+                           T, coarse, tile_base, blocks);
         GS355_CHECK_LAUNCH("bin: fine count");
-        hipLaunchKernelGGL(tile_layout_kernel<true>, dim3(1), dim3(1024), 0, s, tile_base, (uint32_t)T, group_visible,
-                           groups, n_cap, header, true, tile_base, ranges, lists);
-        GS355_CHECK_LAUNCH("bin: layout");
+        if ((rc = launch_layout<true>(tile_base, T, blocks, group_visible, groups, n_cap, header, true, ranges, lists, s)))
+            return rc;
     }
     hipLaunchKernelGGL(fine_scatter_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, min_keys,
                        tile_base, tile_cursor, T, coarse, buckets);
@@ -1241,8 +1296,8 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
     return GS355_OK;
 }
 
-int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, const uint32_t* lists,
-                     uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, hipStream_t s)
+int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, uint32_t* lists, uint64_t* buckets,
+                     uint64_t* out_keys, uint32_t* out_vals, hipStream_t s)
 {
     using S0 = LdsSorter<256, 4>;    // <= 1024 pairs, one workgroup per tile
     using S1 = LdsSorter<512, 4>;    // <= 2048
@@ -1252,19 +1307,20 @@ int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* rang
                       S3::kCap == kTileSortCap[3], "size classes out of step with the layout kernel");
     int rc;
     if ((rc = allow_large_lds())) return rc;
-    const uint32_t* list0 = lists + 4;
+    const uint32_t* list0 = lists + kListHeader;
+    uint32_t* work = lists + 4;  // next untaken entry of each class list
     hipLaunchKernelGGL((tile_sort_each_kernel<256, 4>), dim3(tiles), dim3(256), S0::kBytes, s, header, ranges, buckets,
-                       out_keys, out_vals);
+                       out_keys, out_vals, work);
     GS355_CHECK_LAUNCH("tile sort: class 0");
     auto grid = [&](int want) { return dim3(tiles < want ? tiles : want); };
     hipLaunchKernelGGL((tile_sort_list_kernel<512, 4>), grid(1024), dim3(512), S1::kBytes, s, header, ranges, list0,
-                       lists + 0, buckets, out_keys, out_vals);
+                       lists + 0, work + 0, buckets, out_keys, out_vals);
     GS355_CHECK_LAUNCH("tile sort: class 1");
     hipLaunchKernelGGL(tile_sort_list_1024x5_kernel, grid(512), dim3(1024), S2::kBytes, s, header, ranges,
-                       list0 + (size_t)tiles, lists + 1, buckets, out_keys, out_vals);
+                       list0 + (size_t)tiles, lists + 1, work + 1, buckets, out_keys, out_vals);
     GS355_CHECK_LAUNCH("tile sort: class 2");
     hipLaunchKernelGGL((tile_sort_list_kernel<1024, 10>), grid(256), dim3(1024), S3::kBytes, s, header, ranges,
-                       list0 + 2 * (size_t)tiles, lists + 2, buckets, out_keys, out_vals);
+                       list0 + 2 * (size_t)tiles, lists + 2, work + 2, buckets, out_keys, out_vals);
     GS355_CHECK_LAUNCH("tile sort: class 3");
     hipLaunchKernelGGL(tile_sort_huge_kernel, grid(256), dim3(kThreads), 0, s, header, ranges, lists, (uint32_t)tiles,
                        buckets, out_keys, out_vals);

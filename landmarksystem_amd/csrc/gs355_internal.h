@@ -132,7 +132,7 @@ inline size_t bin_matrix_words(size_t tiles)
     const size_t columns = tiles <= (size_t)kBinMaxTiles ? tiles : (tiles + kCoarseTiles - 1) >> kCoarseShift;
     return (size_t)kBinMaxGroups * columns;
 }
-// tile_base: u32[2][tiles] (bases, then the scatter's cursors).  Beyond kBinMaxTiles tiles launch_tile_layout
+// tile_base: u32[2][tiles] (bases, then the scatter's cursors), then u64[ceil(tiles / 64)] (bases of blocks of 64 tiles).  Beyond kBinMaxTiles tiles launch_tile_layout
 // publishes the header and the coarse bins' bases only; ranges, lists and tile bases follow in launch_tile_scatter.
 int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint32_t* matrix, uint32_t* group_visible,
                       hipStream_t s);
@@ -144,7 +144,9 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
                         gs355_header* header, const uint32_t* matrix, const uint32_t* group_visible, uint32_t n_cap,
                         uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, uint64_t* buckets, uint64_t* coarse,
                         bool two_level, hipStream_t s);
-int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, const uint32_t* lists,
+// lists: u32[kListHeader + 4 * tiles]: the four class counts, the class lists' work counters, the four lists
+constexpr int kListHeader = 8;
+int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, uint32_t* lists,
                      uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, hipStream_t s);
 
 // generic exclusive scan of u32 (n <= 2^32-1); tmp needs scan_tmp_words(n) words

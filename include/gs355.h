@@ -155,13 +155,16 @@ enum {
      *                 slices count per bin of 16 consecutive tiles, and ranges follow with TILE_SCATTER.
      *   TILE_SCATTER  (depth bits << 32 | index) pairs into their tile's bucket: straight for frames of fewer
      *                 than 6 * 2^20 pairs, through bins of 16 consecutive tiles beyond (decided on the device;
-     *                 always beyond 36000 tiles, or with GS355_STAGE_TILE_SCATTER_TWO_LEVEL set as well)
+     *                 always beyond 36000 tiles).  The decision costs the launch of the variant that then does
+     *                 nothing; a caller that knows the size of its frames (say from the previous frame's header)
+     *                 names the variant with one of the modifiers below.  Either variant is correct for any frame.
      *   TILESORT      every bucket sorted by (depth bits, index) in LDS
      * Needs tiles <= 576000 (every 8K image and beyond) and P <= 2^28; otherwise use the classic stages. */
     GS355_STAGE_TILE_COUNT = 128,
     GS355_STAGE_TILESORT = 256,
     GS355_STAGE_TILE_SCATTER = 512,
-    GS355_STAGE_TILE_SCATTER_TWO_LEVEL = 1024, /* modifier of TILE_SCATTER: the two-level scatter whatever the key count */
+    GS355_STAGE_TILE_SCATTER_TWO_LEVEL = 1024, /* modifier of TILE_SCATTER: through the bins whatever the key count */
+    GS355_STAGE_TILE_SCATTER_ONE_LEVEL = 2048, /* modifier of TILE_SCATTER: straight into the buckets (ignored beyond 36000 tiles) */
     GS355_PIPELINE_FAST = 1 | 128 | 512 | 256 | 32
 };
 

@@ -15,7 +15,9 @@ STAGE_PREPROCESS, STAGE_SCAN, STAGE_DUPLICATE, STAGE_SORT, STAGE_RANGES, STAGE_B
 STAGE_ALL = 63
 STAGE_BLEND_PLAIN = 64
 STAGE_TILE_COUNT, STAGE_TILESORT, STAGE_TILE_SCATTER = 128, 256, 512
-STAGE_TILE_SCATTER_TWO_LEVEL = 1024  # modifier: the two-level scatter whatever the key count
+STAGE_TILE_SCATTER_TWO_LEVEL = 1024  # modifiers of STAGE_TILE_SCATTER: name the variant instead of letting the device
+STAGE_TILE_SCATTER_ONE_LEVEL = 2048  # choose by the key count (which launches both)
+TWO_LEVEL_MIN_KEYS = 6 << 20         # the device's own threshold
 PIPELINE_FAST = STAGE_PREPROCESS | STAGE_TILE_COUNT | STAGE_TILE_SCATTER | STAGE_TILESORT | STAGE_BLEND
 MAX_FAST_TILES = 36000 * 16  # limits of the tile-bucketed stages (the classic stages have neither)
 MAX_FAST_GAUSSIANS = 1 << 28

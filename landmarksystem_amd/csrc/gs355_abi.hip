@@ -27,7 +27,8 @@ namespace {
 
 constexpr size_t kAlign = 256;
 constexpr uint32_t kKnownStages = GS355_STAGE_ALL | GS355_STAGE_BLEND_PLAIN | GS355_STAGE_TILE_COUNT | GS355_STAGE_TILESORT | GS355_STAGE_TILE_SCATTER |
-                                  GS355_STAGE_TILE_SCATTER_TWO_LEVEL;
+                                  GS355_STAGE_TILE_SCATTER_TWO_LEVEL | GS355_STAGE_TILE_SCATTER_ONE_LEVEL;
+constexpr uint32_t kStageModifiers = GS355_STAGE_TILE_SCATTER_TWO_LEVEL | GS355_STAGE_TILE_SCATTER_ONE_LEVEL;
 constexpr int64_t kMaxKeys = (1ll << 32) - 1 - kSortTile;  // key slots are indexed with u32
 
 size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
@@ -188,7 +189,8 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
               int64_t n_cap, const gs355_outputs* out, uint32_t stage_mask, void* stream)
 {
     int rc;
-    if ((stage_mask & ~kKnownStages) != 0 || (stage_mask & ~GS355_STAGE_TILE_SCATTER_TWO_LEVEL) == 0)
+    if ((stage_mask & ~kKnownStages) != 0 || (stage_mask & ~kStageModifiers) == 0 ||
+        (stage_mask & kStageModifiers) == kStageModifiers)
         return set_error(GS355_EINVAL, "stage_mask 0x%x selects no known stage", stage_mask);
     if ((rc = check_frame(frame, true))) return rc;
     if ((rc = check_geometry_inputs(g))) return rc;
@@ -259,7 +261,10 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
         // (the buffer the sorted keys will go to is free until the sort: it holds the coarse level of the scatter)
         if ((rc = launch_tile_scatter(fa, g->P, rects, depth_bits, header, bin_matrix, bin_visible, cap, tile_base, ranges,
                                       tile_lists, buckets, keys[L.sorted_buffer],
-                                      (stage_mask & GS355_STAGE_TILE_SCATTER_TWO_LEVEL) != 0, s)))
+                                      (stage_mask & GS355_STAGE_TILE_SCATTER_TWO_LEVEL)   ? 2
+                                      : (stage_mask & GS355_STAGE_TILE_SCATTER_ONE_LEVEL) ? 1
+                                                                                          : 0,
+                                      s)))
             return rc;
     if (stage_mask & GS355_STAGE_TILESORT)
         if ((rc = launch_tile_sort(header, tiles, ranges, tile_lists, buckets, keys[L.sorted_buffer],

@@ -1256,7 +1256,7 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
                         gs355_header* header, const uint32_t* matrix, const uint32_t* group_visible, uint32_t n_cap,
                         uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, uint64_t* buckets, uint64_t* coarse,
-                        bool two_level, hipStream_t s)
+                        int levels, hipStream_t s)
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
@@ -1266,16 +1266,20 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
     int rc = allow_large_lds();
     if (rc) return rc;
     uint32_t min_keys = 0;  // pairs from which the two levels run
+    bool fine = true;
     if (T <= kBinMaxTiles) {
-        if (!two_level) {
-            min_keys = kTwoLevelMinKeys;
+        if (levels != 2) {
+            min_keys = levels == 1 ? UINT32_MAX : kTwoLevelMinKeys;
             hipLaunchKernelGGL((scatter_kernel<0, false>), dim3(groups), dim3(kBinThreads), (size_t)T * sizeof(uint32_t), s,
                                f, P, per_group, rects, depth_bits, header, 0u, min_keys, matrix, tile_base, buckets);
             GS355_CHECK_LAUNCH("bin: scatter");
         }
-        hipLaunchKernelGGL((scatter_kernel<kCoarseShift, false>), dim3(groups), dim3(kBinThreads), coarse_lds, s, f, P,
-                           per_group, rects, depth_bits, header, min_keys, UINT32_MAX, matrix, tile_base, coarse);
-        GS355_CHECK_LAUNCH("bin: coarse scatter");
+        fine = levels != 1;
+        if (fine) {
+            hipLaunchKernelGGL((scatter_kernel<kCoarseShift, false>), dim3(groups), dim3(kBinThreads), coarse_lds, s, f, P,
+                               per_group, rects, depth_bits, header, min_keys, UINT32_MAX, matrix, tile_base, coarse);
+            GS355_CHECK_LAUNCH("bin: coarse scatter");
+        }
     } else {
         const uint32_t* bin_base = tile_cursor;  // (replaced by the tiles' cursors once the coarse level is done)
         hipLaunchKernelGGL((scatter_kernel<kCoarseShift, true>), dim3(groups), dim3(kBinThreads), coarse_lds, s, f, P,
@@ -1290,9 +1294,11 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
         if ((rc = launch_layout<true>(tile_base, T, blocks, group_visible, groups, n_cap, header, true, ranges, lists, s)))
             return rc;
     }
-    hipLaunchKernelGGL(fine_scatter_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, min_keys,
-                       tile_base, tile_cursor, T, coarse, buckets);
-    GS355_CHECK_LAUNCH("bin: fine scatter");
+    if (fine) {
+        hipLaunchKernelGGL(fine_scatter_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, min_keys,
+                           tile_base, tile_cursor, T, coarse, buckets);
+        GS355_CHECK_LAUNCH("bin: fine scatter");
+    }
     return GS355_OK;
 }
 

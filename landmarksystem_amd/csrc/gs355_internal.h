@@ -138,12 +138,13 @@ int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint
                       hipStream_t s);
 int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visible, int tiles, uint32_t n_cap,
                        gs355_header* header, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s);
-// `coarse`: a second buffer of the buckets' size (first level of the two-level scatter).  `two_level`: take the
-// two levels whatever the frame holds (otherwise chosen on the device by the key count)
+// `coarse`: a second buffer of the buckets' size (first level of the two-level scatter).  `levels`: 1 or 2 = that
+// scatter whatever the frame holds, 0 = chosen on the device by the key count (both variants are launched); images
+// beyond kBinMaxTiles tiles always take two levels
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
                         gs355_header* header, const uint32_t* matrix, const uint32_t* group_visible, uint32_t n_cap,
                         uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, uint64_t* buckets, uint64_t* coarse,
-                        bool two_level, hipStream_t s);
+                        int levels, hipStream_t s);
 // lists: u32[kListHeader + 4 * tiles]: the four class counts, the class lists' work counters, the four lists
 constexpr int kListHeader = 8;
 int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, uint32_t* lists,

@@ -54,6 +54,7 @@ class Workspace:
         self.header_event = torch.cuda.Event()
         self.frames = 0
         self.overflows = 0
+        self.last_num_keys = 0  # of the latest frame rendered over this workspace
 
     def ensure(self, P: int, n_cap: int, width: int, height: int) -> "_lib.Layout":
         layout = _lib.workspace_layout(P, n_cap, width, height)
@@ -279,6 +280,9 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
     if not classic and inputs.tiles <= _lib.MAX_FAST_TILES and inputs.P <= _lib.MAX_FAST_GAUSSIANS:
         front = _lib.STAGE_PREPROCESS | _lib.STAGE_TILE_COUNT
         back = _lib.STAGE_TILE_SCATTER | _lib.STAGE_TILESORT | _lib.STAGE_BLEND
+        # the scatter variant that suited the previous frame of this workspace (either is correct for any frame)
+        back |= (_lib.STAGE_TILE_SCATTER_TWO_LEVEL if ws.last_num_keys >= _lib.TWO_LEVEL_MIN_KEYS
+                 else _lib.STAGE_TILE_SCATTER_ONE_LEVEL)
     else:  # beyond the bucketed stages' limits (images past 8K): classic duplicate / radix sort / ranges
         front = _lib.STAGE_PREPROCESS | _lib.STAGE_SCAN
         back = _lib.STAGE_DUPLICATE | _lib.STAGE_SORT | _lib.STAGE_RANGES | _lib.STAGE_BLEND
@@ -292,7 +296,7 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
         total = int(ws.header_host[0])
         word1 = int(ws.header_host[1])
         overflow = (word1 >> 32) & 0xFFFFFFFF
-        out.num_keys = total
+        out.num_keys = ws.last_num_keys = total
         out.num_visible = int(ws.header_host[2]) & 0xFFFFFFFF
         ws.frames += 1
         if not overflow:

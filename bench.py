@@ -47,6 +47,13 @@ COUNTER_TRAFFIC = {
     "blend_issued_flops_source": "profiles/bench_c3_6M_1080p_valu_counters.txt",
 }
 
+# Same for `--config 5`: HBM bytes per launch of the two decode kernels (count + emit)
+COUNTER_TRAFFIC_C5 = {
+    "source": "profiles/bench_c5_scaffold_500k_hbm_traffic.txt",
+    "workload": "configs[4]",
+    "bytes": {"decode": 250.6e6},
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -201,15 +208,20 @@ def raster_report(stage_ms, stats, P, tiles, npix, colour_bytes, pairs, counters
                        "sorted_keys_per_s": round(N / sort_ms * 1e3) if N else 0,
                        "blend_frames_per_s": round(1e3 / stage_ms["blend"], 1)}
 
-    shipped = {"preprocess": stage_ms["preprocess"], "keys_sort_ranges": sort_ms, "blend": stage_ms["blend"]}
+    # the dominant KERNEL: preprocess and blend are one kernel each; count / scatter / sort are groups of several
+    # kernels, none of which comes near either (their sum is reported as stages.keys_sort_ranges)
+    shipped = {"preprocess": stage_ms["preprocess"], "blend": stage_ms["blend"]}
     dominant = max(shipped, key=lambda n: shipped[n])
-    traffic = {"bytes": cbytes[dominant], "source": counters["source"],
-               "note": "from earlier profiler runs of this workload, not measured by this run"} \
-        if counters and dominant in cbytes else None
+    # HBM bytes per launch of that kernel, from the committed counter runs (a number quoted from the named file,
+    # not an observation of this run)
+    traffic = cbytes[dominant] if counters and dominant in cbytes else None
+    traffic_source = (counters["source"] + " (rocprofv3 FETCH_SIZE + WRITE_SIZE of an earlier run of this workload)"
+                      if traffic else None)
     if dominant == "blend":
         kind = "algorithmic" if pairs else "upper"
         roofline = {"bound": "valu", "kernel": "blend_kernel", "achieved": blend["TFLOPs_" + kind],
                     "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": blend["frac_fp32_" + kind], "traffic": traffic,
+                    "traffic_source": traffic_source,
                     "note": "FP32 vector-ALU kernel (no matrix cores); peak is the MI355X fp32 vector figure (packed FMA; "
                             "this build issues unpacked fp32, half of it).  flops = 25 x the (pixel, Gaussian) pairs the "
                             "per-pixel loop evaluates" + (
@@ -217,8 +229,9 @@ def raster_report(stage_ms, stats, P, tiles, npix, colour_bytes, pairs, counters
                                 "< 1/255, so it issues fewer flops than that" if pairs else
                                 ", bounded above by 256 x the sum of the tile range lengths")}
     else:
-        roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": traffic}
+        roofline = {"bound": "hbm", "kernel": dominant + "_kernel", "achieved": stages[dominant]["GBps"],
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": traffic,
+                    "traffic_source": traffic_source}
     return stages, roofline
 
 
@@ -583,10 +596,15 @@ def bench_scaffold(args, torch, dev):
                         "frac_hbm": round(dec_bytes / dec_ms / 1e6 / HBM_PEAK_GBS, 4),
                         "note": "bound by HBM and instruction issue, not by the matrix cores (17 flop/B); bytes = inputs "
                                 "of the visible anchors once + the visibility mask + 56 B per emitted Gaussian"}
-    if dec_ms > max(stage_ms["preprocess"], stage_ms["blend"],
-                    stage_ms["tile_count"] + stage_ms["tile_scatter"] + stage_ms["tile_sort"]):
+    quoted = COUNTER_TRAFFIC_C5["bytes"]["decode"] if not args.gaussians else None  # (counted on the named workload)
+    if quoted:
+        stages["decode"].update({"counter_bytes": quoted, "counter_GBps": round(quoted / dec_ms / 1e6, 1),
+                                 "frac_hbm_counter": round(quoted / dec_ms / 1e6 / HBM_PEAK_GBS, 4)})
+    if dec_ms > max(stage_ms["preprocess"], stage_ms["blend"]):  # the dominant kernel(s): count + emit of the decode
         roofline = {"bound": "hbm", "kernel": "decode_kernel", "achieved": stages["decode"]["GBps"], "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": stages["decode"]["frac_hbm"], "traffic": None,
+                    "unit": "GB/s", "frac": stages["decode"]["frac_hbm"], "traffic": quoted,
+                    "traffic_source": (COUNTER_TRAFFIC_C5["source"] + " (rocprofv3 FETCH_SIZE + WRITE_SIZE of an earlier "
+                                       "run of this workload)") if quoted else None,
                     "mfma_frac": stages["decode"]["frac_mfma_f16"]}
     result = base_line("1080p frames/sec, Scaffold-GS with 500k anchors (1 GPU)", fps, ms_per_step, args, args.warmup,
                        "f32 (decode: f16 matrix inputs as hi+lo pairs, f32 accumulate)", {

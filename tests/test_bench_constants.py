@@ -48,6 +48,16 @@ def test_quoted_traffic_matches_the_profile_it_names():
         assert abs(table["bytes"][name] / 1e6 - mb) <= 0.002 * mb + 0.2, (name, table["bytes"][name] / 1e6, mb)
 
 
+def test_quoted_decode_traffic_matches_the_profile_it_names():
+    bench = load_bench()
+    table = bench.COUNTER_TRAFFIC_C5
+    path = os.path.join(ROOT, table["source"])
+    if not os.path.exists(path):
+        pytest.skip("profiles/ is not part of this checkout")
+    mb = sum(v for k, v in traffic_table(path).items() if k.startswith("decode_kernel"))
+    assert mb > 0 and abs(table["bytes"]["decode"] / 1e6 - mb) <= 0.002 * mb + 0.2, (table["bytes"]["decode"] / 1e6, mb)
+
+
 def test_quoted_issued_flops_match_the_profile_they_name():
     bench = load_bench()
     table = bench.COUNTER_TRAFFIC

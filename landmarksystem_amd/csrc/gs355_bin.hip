@@ -6,14 +6,16 @@
 // a pair is generated, so the most significant digit is resolved by counting:
 // pairs are counted per tile, an exclusive scan of the counts gives every tile
 // its slot range (these ARE the per-tile ranges), and pairs are scattered into
-// their tile's bucket.  What remains is an independent sort of each bucket by
-// its low word, done by one workgroup per tile as an LSD radix sort staged
-// entirely in LDS (up to 9216 pairs in the 160 KB of a CU; larger buckets run
-// the same passes through global memory).  Bucket order after the scatter is
-// arbitrary, so pairs are ordered by (depth bits, Gaussian index): exactly the
-// order a stable sort of the emission-ordered keys produces.
+// their tile's bucket (in one level, or through coarse bins of 16 tiles when
+// the frame holds many pairs).  What remains is an independent sort of each
+// bucket by its low word, done by one workgroup per tile entirely in LDS (up
+// to 10240 pairs in the 160 KB of a CU; larger buckets run radix passes
+// through global memory).  Bucket order after the scatter is arbitrary, so
+// pairs are ordered by (depth bits, Gaussian index): exactly the order a
+// stable sort of the emission-ordered keys produces.
 //
-// No workgroup waits on another; persistent loops run over fixed lists.
+// No workgroup waits on another; persistent loops run over fixed lists, or
+// take entries from a counter until it passes the list's length.
 #include <atomic>
 
 #include "gs355_internal.h"
@@ -1069,7 +1071,7 @@ __global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* 
     sorter.run(blockIdx.x, ranges, buckets, out_keys, out_vals);
 }
 
-// Larger size classes: persistent workgroups over the class list made by tile_layout_kernel.  A workgroup starts
+// Larger size classes: persistent workgroups over the class list made by tile_publish_kernel.  A workgroup starts
 // with the list entry of its own number and then takes the next one nobody has taken (`work`, a counter cleared by
 // tile_sort_each_kernel): buckets of one class differ in size by a factor of two and more, and a fixed assignment
 // leaves most of the chip waiting for the workgroups that drew the large ones.  The request for the next entry is

@@ -9,7 +9,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-SHIPPED_SORT_KERNELS = ("tile_count_kernel", "slice_prefix_kernel", "tile_layout_kernel", "scatter_kernel",
+SHIPPED_SORT_KERNELS = ("tile_count_kernel", "slice_prefix_kernel", "block_scan_kernel", "tile_publish_kernel", "scatter_kernel",
                         "fine_scatter_kernel", "tile_sort_each_kernel", "tile_sort_list_kernel",
                         "tile_sort_list_1024x5_kernel", "tile_sort_huge_kernel")
 

@@ -126,7 +126,8 @@ typedef struct gs355_layout {
     size_t ranges;        /* u32[tiles][2] */
     size_t bin_matrix;    /* u32[slices][tiles] pairs per (slice of Gaussians, tile), then their prefix over slices */
     size_t tile_base;     /* u32[2][tiles]   first slot of each tile's bucket; its next free slot during the scatter;
-                           * then u64[ceil(tiles/64)], the first slot of each block of 64 tiles */
+                           * then u64[ceil(tiles/64)], the first slot of each block of 64 tiles, and
+                           * u32[ceil(tiles/16)+1], the work list of the scatter's second level */
     size_t bin_visible;   /* u32[slices]     visible Gaussians per slice */
     size_t tile_lists;    /* u32[8+4*tiles]  counts, work counters and lists of the buckets of each larger sorter size class */
     size_t total_bytes;

@@ -88,7 +88,7 @@ int make_layout(int32_t P, int64_t n_cap, int32_t W, int32_t H, gs355_layout* L)
     L->sort_hist = take(hist_words * sizeof(uint32_t));
     L->ranges = take(tiles * 2 * sizeof(uint32_t));
     L->bin_matrix = take((tiles <= (size_t)kBinMaxTilesWide ? bin_matrix_words(tiles) : 0) * sizeof(uint32_t));
-    L->tile_base = take((2 * tiles + 2 * ((tiles + 63) / 64)) * sizeof(uint32_t));
+    L->tile_base = take((2 * tiles + 2 * ((tiles + 63) / 64) + (tiles + kCoarseTiles - 1) / kCoarseTiles + 1) * sizeof(uint32_t));
     L->bin_visible = take((size_t)kBinMaxGroups * sizeof(uint32_t));
     L->tile_lists = take((kListHeader + 4 * tiles) * sizeof(uint32_t));
     L->total_bytes = off;

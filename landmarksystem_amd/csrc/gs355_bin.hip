@@ -224,21 +224,63 @@ __global__ __launch_bounds__(kBinThreads) void scatter_kernel(FrameArgs f, int32
     }
 }
 
-// Second level: the pairs of a coarse bin (contiguous) go to the buckets of the bin's tiles.  kFineSplit workgroups
-// share a bin, each taking every kFineSplit-th chunk of it (bins differ in size by a factor of several, and one
-// workgroup per bin would leave the largest for last).  A chunk is split by tile inside LDS first (wave-level ranking
-// by the four tile bits, a scan over the 8 x 16 per-wave counts), the workgroup reserves a run of slots per bucket
-// with one global atomic each, and consecutive lanes then store consecutive pairs of one bucket: full-line writes
-// instead of one memory transaction per pair.  Order inside a bucket is arbitrary, as the sort expects.
+// Second level: the pairs of a coarse bin (contiguous) go to the buckets of the bin's tiles, a chunk of kFineChunk pairs
+// at a time.  Chunks never cross a bin; chunk_base[b] = chunks of the bins before b, chunk_base[bins] = all of them
+// (block_scan_kernel).  The kFineGrid workgroups take equal, contiguous runs of chunks, so every workgroup has work
+// however the pairs are spread over the bins, and a bin of many pairs is shared by many workgroups.  A chunk is split
+// by tile inside LDS first (wave-level ranking by the four tile bits, a scan over the 8 x 16 per-wave counts), the
+// workgroup reserves a run of slots per bucket with one global atomic each, and consecutive lanes then store
+// consecutive pairs of one bucket: full-line writes instead of one memory transaction per pair.  Order inside a
+// bucket is arbitrary, as the sort expects.
 constexpr int kFineThreads = 512;
 constexpr int kFineWaves = kFineThreads / 64;
 constexpr int kFineItems = 8;                             // pairs per thread and chunk
 constexpr int kFineChunk = kFineThreads * kFineItems;  // 4096 pairs = 32 KB of LDS
-constexpr int kFineSplit = 8;   // workgroups per bin
+constexpr int kFineGrid = 1024;                          // four workgroups of 512 threads per CU
+
+// A workgroup's run of chunks.  next() gives the following chunk's bin, first pair and pair count.
+struct ChunkRun {
+    const uint32_t* chunk_base;
+    uint32_t c, c_end;  // next chunk, end of the run
+    int b, bins;        // bin of chunk c (once begun)
+
+    __device__ ChunkRun(const uint32_t* __restrict__ base, int n_bins) : chunk_base(base), b(0), bins(n_bins)
+    {
+        const uint32_t total = base[n_bins], per = (total + gridDim.x - 1) / gridDim.x;
+        c = min(total, blockIdx.x * per);
+        c_end = min(total, c + per);
+        if (c < c_end) {  // the bin that holds chunk c: the last one whose base is <= c
+            int lo = 0, hi = n_bins;  // base[lo] <= c < base[hi]
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (base[mid] <= c) lo = mid;
+                else hi = mid;
+            }
+            b = lo;
+        }
+    }
+    // `first_pair(bin)`: where the bin's pairs start in the coarse buffer
+    template <typename First>
+    __device__ bool next(First first_pair, uint32_t num_keys, int& bin, uint32_t& j0, uint32_t& n, uint32_t& bin_begin,
+                         uint32_t& bin_end)
+    {
+        if (c >= c_end) return false;
+        while (chunk_base[b + 1] <= c) ++b;  // (bins without pairs have no chunks)
+        bin = b;
+        bin_begin = first_pair(b);
+        bin_end = b + 1 < bins ? first_pair(b + 1) : num_keys;
+        j0 = bin_begin + (c - chunk_base[b]) * (uint32_t)kFineChunk;
+        n = min((uint32_t)kFineChunk, bin_end - j0);
+        ++c;
+        return true;
+    }
+};
+
 __global__ __launch_bounds__(kFineThreads) void fine_scatter_kernel(const gs355_header* __restrict__ header,
                                                                     uint32_t min_keys,
                                                                     const uint32_t* __restrict__ tile_base,
                                                                     uint32_t* __restrict__ cursor, int T,
+                                                                    const uint32_t* __restrict__ chunk_base,
                                                                     const uint64_t* __restrict__ coarse,
                                                                     uint64_t* __restrict__ buckets)
 {
@@ -247,16 +289,16 @@ __global__ __launch_bounds__(kFineThreads) void fine_scatter_kernel(const gs355_
     __shared__ uint32_t s_start[kCoarseTiles + 1];          // first staged position of each tile's pairs
     __shared__ uint32_t s_slot[kCoarseTiles];               // first reserved slot of each bucket for this chunk
     if (header->overflow || header->num_keys < min_keys) return;
-    const int t0 = ((int)blockIdx.x / kFineSplit) << kCoarseShift;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const uint32_t begin = tile_base[t0];
-    const uint32_t end = t0 + kCoarseTiles < T ? tile_base[t0 + kCoarseTiles] : header->num_keys;
     const uint64_t lanes_below = (1ull << lane) - 1ull;
-    for (uint32_t j0 = begin + (blockIdx.x % kFineSplit) * (uint32_t)kFineChunk; j0 < end;
-         j0 += (uint32_t)(kFineSplit * kFineChunk)) {
+    const uint32_t num_keys = header->num_keys;
+    ChunkRun run(chunk_base, (T + kCoarseTiles - 1) >> kCoarseShift);
+    int bin;
+    uint32_t j0, n, begin, end;
+    while (run.next([&](int b) { return tile_base[b << kCoarseShift]; }, num_keys, bin, j0, n, begin, end)) {
+        const int t0 = bin << kCoarseShift;
         for (int k = tid; k < kFineWaves * kCoarseTiles; k += kFineThreads) (&s_count[0][0])[k] = 0;
         __syncthreads();
-        const uint32_t n = min((uint32_t)kFineChunk, end - j0);
         // a wavefront owns kFineItems x 64 consecutive pairs of the chunk
         uint64_t v[kFineItems];
         uint32_t rank[kFineItems];
@@ -331,27 +373,28 @@ __global__ __launch_bounds__(kFineThreads) void fine_scatter_kernel(const gs355_
     }
 }
 
-// Pairs per tile, counted from the coarse bins (images of more tiles than a slice can count in LDS): same chunks
-// as the fine scatter, a wavefront-level count by the four tile bits, one global atomic per tile and chunk.
+// Pairs per tile, counted from the coarse bins (images of more tiles than a slice can count in LDS): the chunks of
+// the fine scatter, a wavefront-level count by the four tile bits, one global atomic per tile and chunk.
 // `bin_base` [bins]: first pair of each bin; `totals` [T] and `block_sums` [T / 64] (pairs per 64 tiles) cleared
 // beforehand.
 __global__ __launch_bounds__(kFineThreads) void fine_count_kernel(const gs355_header* __restrict__ header,
                                                                   const uint32_t* __restrict__ bin_base, int bins,
-                                                                  int T, const uint64_t* __restrict__ coarse,
+                                                                  int T, const uint32_t* __restrict__ chunk_base,
+                                                                  const uint64_t* __restrict__ coarse,
                                                                   uint32_t* __restrict__ totals,
                                                                   uint64_t* __restrict__ block_sums)
 {
     __shared__ uint32_t s_count[kCoarseTiles];
     if (header->overflow) return;
-    const int b = (int)blockIdx.x / kFineSplit, t0 = b << kCoarseShift;
     const int tid = threadIdx.x, lane = tid & 63;
-    const uint32_t begin = bin_base[b];
-    const uint32_t end = b + 1 < bins ? bin_base[b + 1] : header->num_keys;
-    if (tid < kCoarseTiles) s_count[tid] = 0;
-    __syncthreads();
-    for (uint32_t j0 = begin + (blockIdx.x % kFineSplit) * (uint32_t)kFineChunk; j0 < end;
-         j0 += (uint32_t)(kFineSplit * kFineChunk)) {
-        const uint32_t n = min((uint32_t)kFineChunk, end - j0);
+    const uint32_t num_keys = header->num_keys;
+    ChunkRun run(chunk_base, bins);
+    int bin;
+    uint32_t j0, n, begin, end;
+    while (run.next([&](int b) { return bin_base[b]; }, num_keys, bin, j0, n, begin, end)) {
+        const int t0 = bin << kCoarseShift;
+        if (tid < kCoarseTiles) s_count[tid] = 0;
+        __syncthreads();
         uint64_t v[kFineItems];
 #pragma unroll
         for (int u = 0; u < kFineItems; ++u) {
@@ -371,11 +414,12 @@ __global__ __launch_bounds__(kFineThreads) void fine_count_kernel(const gs355_he
             }
             if (valid && lane == __ffsll((unsigned long long)peers) - 1) atomicAdd(&s_count[d], (uint32_t)__popcll(peers));
         }
-    }
-    __syncthreads();
-    if (tid < kCoarseTiles && t0 + tid < T && s_count[tid]) {
-        atomicAdd(&totals[t0 + tid], s_count[tid]);
-        atomicAdd(reinterpret_cast<unsigned long long*>(&block_sums[(t0 + tid) >> 6]), (unsigned long long)s_count[tid]);
+        __syncthreads();
+        if (tid < kCoarseTiles && t0 + tid < T && s_count[tid]) {
+            atomicAdd(&totals[t0 + tid], s_count[tid]);
+            atomicAdd(reinterpret_cast<unsigned long long*>(&block_sums[(t0 + tid) >> 6]), (unsigned long long)s_count[tid]);
+        }
+        __syncthreads();
     }
 }
 
@@ -386,7 +430,8 @@ __global__ __launch_bounds__(kFineThreads) void fine_count_kernel(const gs355_he
 // prefixes shifted by the quarters before them.
 __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict__ matrix, int groups, int tiles,
                                                            uint32_t* __restrict__ totals,
-                                                           uint64_t* __restrict__ block_sums)
+                                                           uint64_t* __restrict__ block_sums,
+                                                           uint32_t* __restrict__ bin_sums)
 {
     __shared__ uint32_t s_part[4][64];
     const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
@@ -431,6 +476,12 @@ __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict_
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) sum64 += __shfl_down(sum64, d, 64);
         if (lane == 0) block_sums[blockIdx.x] = sum64;
+        if (bin_sums) {  // columns are tiles: the pairs of each coarse bin (kCoarseTiles consecutive tiles)
+            uint32_t bin = live ? total : 0u;
+#pragma unroll
+            for (int d = 1; d < kCoarseTiles; d <<= 1) bin += __shfl_xor(bin, d, 64);
+            if ((lane & (kCoarseTiles - 1)) == 0 && live) bin_sums[t >> kCoarseShift] = bin;
+        }
     }
 }
 
@@ -441,10 +492,11 @@ __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict_
 __global__ __launch_bounds__(1024) void block_scan_kernel(uint64_t* __restrict__ blocks, uint32_t n_blocks,
                                                           const uint32_t* __restrict__ group_visible, int groups,
                                                           uint32_t n_cap, gs355_header* __restrict__ header,
-                                                          bool header_known, uint32_t* __restrict__ lists)
+                                                          bool header_known, uint32_t* __restrict__ lists,
+                                                          const uint32_t* bin_pairs, int bins, uint32_t* chunk_base)
 {
     __shared__ uint64_t s_wave[16];
-    __shared__ uint32_t s_vis;
+    __shared__ uint32_t s_vis, s_chunks[16];
     if (header_known && header->overflow) return;
     if (threadIdx.x == 0) s_vis = 0;
     __syncthreads();
@@ -491,6 +543,30 @@ __global__ __launch_bounds__(1024) void block_scan_kernel(uint64_t* __restrict__
     for (uint32_t k = 0; k < kRun; ++k) {
         if (b0 + k < b1) blocks[b0 + k] = first;
         first += v[k];
+    }
+    // The second scatter level works through every coarse bin in chunks of kFineChunk pairs: chunk_base[b] = chunks
+    // of the bins before b, chunk_base[bins] = all.  `bin_pairs` (pairs per bin) may be the same array.
+    if (bins > 0 && !overflow) {
+        const int per_thread = (bins + 1023) / 1024;
+        const int q0 = min((int)threadIdx.x * per_thread, bins), q1 = min(q0 + per_thread, bins);
+        uint32_t chunks = 0;
+        for (int q = q0; q < q1; ++q) chunks += (bin_pairs[q] + (uint32_t)kFineChunk - 1u) / (uint32_t)kFineChunk;
+        uint32_t cinc = chunks;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(cinc, d, 64);
+            if (lane >= d) cinc += up;
+        }
+        if (lane == 63) s_chunks[wave] = cinc;
+        __syncthreads();
+        uint32_t run = cinc - chunks;
+        for (int w = 0; w < wave; ++w) run += s_chunks[w];
+        for (int q = q0; q < q1; ++q) {  // (each element is read before it is overwritten, by its own thread)
+            const uint32_t n = (bin_pairs[q] + (uint32_t)kFineChunk - 1u) / (uint32_t)kFineChunk;
+            chunk_base[q] = run;
+            run += n;
+        }
+        if (threadIdx.x == 1023) chunk_base[bins] = run;
     }
 }
 
@@ -1196,6 +1272,11 @@ static int allow_large_lds()
 }
 
 static inline int coarse_bins(int tiles) { return (tiles + kCoarseTiles - 1) >> kCoarseShift; }
+// the tile_base array: u32[2][tiles], u64[blocks of 64 tiles], u32[coarse bins + 1] chunk bases
+static inline uint32_t* chunk_bases(uint32_t* tile_base, int tiles)
+{
+    return tile_base + 2 * (size_t)tiles + 2 * (size_t)((tiles + 63) / 64);
+}
 
 int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint32_t* matrix, uint32_t* group_visible,
                       hipStream_t s)
@@ -1219,11 +1300,11 @@ int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint
 template <bool kTiles>
 static int launch_layout(uint32_t* totals_and_bases, int columns, uint64_t* blocks, const uint32_t* group_visible,
                          int groups, uint32_t n_cap, gs355_header* header, bool header_known, uint32_t* ranges,
-                         uint32_t* lists, hipStream_t s)
+                         uint32_t* lists, const uint32_t* bin_pairs, int bins, uint32_t* chunk_base, hipStream_t s)
 {
     const int n_blocks = (columns + 63) / 64;
     hipLaunchKernelGGL(block_scan_kernel, dim3(1), dim3(1024), 0, s, blocks, (uint32_t)n_blocks, group_visible, groups,
-                       n_cap, header, header_known, lists);
+                       n_cap, header, header_known, lists, bin_pairs, bins, chunk_base);
     GS355_CHECK_LAUNCH("bin: block scan");
     hipLaunchKernelGGL(tile_publish_kernel<kTiles>, dim3((n_blocks + 3) / 4), dim3(256), 0, s, totals_and_bases,
                        (uint32_t)columns, blocks, header, totals_and_bases, ranges, lists);
@@ -1240,19 +1321,22 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
     int per_group;
     const int groups = bin_groups(P, &per_group);
     uint64_t* blocks = reinterpret_cast<uint64_t*>(tile_base + 2 * (size_t)tiles);
+    const int bins = coarse_bins(tiles);
+    uint32_t* chunk_base = chunk_bases(tile_base, tiles);
     if (tiles <= kBinMaxTiles) {
+        // (the pairs of each coarse bin go to chunk_base, which the block scan turns into chunk bases in place)
         hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(256), 0, s, matrix, groups, tiles,
-                           tile_base, blocks);
+                           tile_base, blocks, chunk_base);
         GS355_CHECK_LAUNCH("bin: slice prefix");
         return launch_layout<true>(tile_base, tiles, blocks, group_visible, groups, n_cap, header, false, ranges, lists,
-                                   s);
+                                   chunk_base, bins, chunk_base, s);
     }
-    const int bins = coarse_bins(tiles);
     uint32_t* bin_base = tile_base + tiles;
     hipLaunchKernelGGL(slice_prefix_kernel, dim3((bins + 63) / 64), dim3(256), 0, s, matrix, groups, bins, bin_base,
-                       blocks);
+                       blocks, (uint32_t*)nullptr);
     GS355_CHECK_LAUNCH("bin: slice prefix");
-    return launch_layout<false>(bin_base, bins, blocks, group_visible, groups, n_cap, header, false, ranges, lists, s);
+    return launch_layout<false>(bin_base, bins, blocks, group_visible, groups, n_cap, header, false, ranges, lists,
+                                bin_base, bins, chunk_base, s);
 }
 
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
@@ -1290,15 +1374,16 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
         uint64_t* blocks = reinterpret_cast<uint64_t*>(tile_base + 2 * (size_t)T);
         if ((rc = launch_fill_u32(tile_base, (size_t)T, 0u, s))) return rc;
         if ((rc = launch_fill_u32(reinterpret_cast<uint32_t*>(blocks), 2 * (size_t)((T + 63) / 64), 0u, s))) return rc;
-        hipLaunchKernelGGL(fine_count_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, bin_base, bins,
-                           T, coarse, tile_base, blocks);
+        hipLaunchKernelGGL(fine_count_kernel, dim3(kFineGrid), dim3(kFineThreads), 0, s, header, bin_base, bins, T,
+                           chunk_bases(tile_base, T), coarse, tile_base, blocks);
         GS355_CHECK_LAUNCH("bin: fine count");
-        if ((rc = launch_layout<true>(tile_base, T, blocks, group_visible, groups, n_cap, header, true, ranges, lists, s)))
+        if ((rc = launch_layout<true>(tile_base, T, blocks, group_visible, groups, n_cap, header, true, ranges, lists,
+                                      (const uint32_t*)nullptr, 0, (uint32_t*)nullptr, s)))
             return rc;
     }
     if (fine) {
-        hipLaunchKernelGGL(fine_scatter_kernel, dim3(bins * kFineSplit), dim3(kFineThreads), 0, s, header, min_keys,
-                           tile_base, tile_cursor, T, coarse, buckets);
+        hipLaunchKernelGGL(fine_scatter_kernel, dim3(kFineGrid), dim3(kFineThreads), 0, s, header, min_keys, tile_base,
+                           tile_cursor, T, chunk_bases(tile_base, T), coarse, buckets);
         GS355_CHECK_LAUNCH("bin: fine scatter");
     }
     return GS355_OK;

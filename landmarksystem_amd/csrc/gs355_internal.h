@@ -132,7 +132,8 @@ inline size_t bin_matrix_words(size_t tiles)
     const size_t columns = tiles <= (size_t)kBinMaxTiles ? tiles : (tiles + kCoarseTiles - 1) >> kCoarseShift;
     return (size_t)kBinMaxGroups * columns;
 }
-// tile_base: u32[2][tiles] (bases, then the scatter's cursors), then u64[ceil(tiles / 64)] (bases of blocks of 64 tiles).  Beyond kBinMaxTiles tiles launch_tile_layout
+// tile_base: u32[2][tiles] (bases, then the scatter's cursors), then u64[ceil(tiles / 64)] (bases of blocks of 64 tiles),
+// then u32[coarse bins + 1] (chunks of the second scatter level before each bin).  Beyond kBinMaxTiles tiles launch_tile_layout
 // publishes the header and the coarse bins' bases only; ranges, lists and tile bases follow in launch_tile_scatter.
 int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint32_t* matrix, uint32_t* group_visible,
                       hipStream_t s);

@@ -226,7 +226,7 @@ __global__ __launch_bounds__(kBinThreads) void scatter_kernel(FrameArgs f, int32
 
 // Second level: the pairs of a coarse bin (contiguous) go to the buckets of the bin's tiles, a chunk of kFineChunk pairs
 // at a time.  Chunks never cross a bin; chunk_base[b] = chunks of the bins before b, chunk_base[bins] = all of them
-// (block_scan_kernel).  The kFineGrid workgroups take equal, contiguous runs of chunks, so every workgroup has work
+// (tile_publish_kernel).  The kFineGrid workgroups take equal, contiguous runs of chunks, so every workgroup has work
 // however the pairs are spread over the bins, and a bin of many pairs is shared by many workgroups.  A chunk is split
 // by tile inside LDS first (wave-level ranking by the four tile bits, a scan over the 8 x 16 per-wave counts), the
 // workgroup reserves a run of slots per bucket with one global atomic each, and consecutive lanes then store
@@ -382,9 +382,11 @@ __global__ __launch_bounds__(kFineThreads) void fine_count_kernel(const gs355_he
                                                                   int T, const uint32_t* __restrict__ chunk_base,
                                                                   const uint64_t* __restrict__ coarse,
                                                                   uint32_t* __restrict__ totals,
-                                                                  uint64_t* __restrict__ block_sums)
+                                                                  uint64_t* __restrict__ block_sums,
+                                                                  uint32_t* __restrict__ list_counts)
 {
     __shared__ uint32_t s_count[kCoarseTiles];
+    if (blockIdx.x == 0 && threadIdx.x < 4) list_counts[threadIdx.x] = 0u;  // filled by tile_publish_kernel
     if (header->overflow) return;
     const int tid = threadIdx.x, lane = tid & 63;
     const uint32_t num_keys = header->num_keys;
@@ -431,9 +433,11 @@ __global__ __launch_bounds__(kFineThreads) void fine_count_kernel(const gs355_he
 __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict__ matrix, int groups, int tiles,
                                                            uint32_t* __restrict__ totals,
                                                            uint64_t* __restrict__ block_sums,
-                                                           uint32_t* __restrict__ bin_sums)
+                                                           uint32_t* __restrict__ bin_sums,
+                                                           uint32_t* __restrict__ list_counts)
 {
     __shared__ uint32_t s_part[4][64];
+    if (blockIdx.x == 0 && threadIdx.x < 4) list_counts[threadIdx.x] = 0u;  // filled by tile_publish_kernel
     const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
     const int t = blockIdx.x * 64 + lane;
     const int per = (groups + 3) / 4;
@@ -485,69 +489,65 @@ __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict_
     }
 }
 
-// Layout of the buckets from the tiles' totals, in two steps.  First one workgroup turns the totals of the blocks of
-// 64 tiles into block bases (exclusive scan, in place) and writes the frame header; the grand total decides overflow
-// before anything else is published.  `header_known`: second layout of a frame (by tile, after the one by coarse
-// bin): the header stands, and nothing is done on overflow.
-__global__ __launch_bounds__(1024) void block_scan_kernel(uint64_t* __restrict__ blocks, uint32_t n_blocks,
-                                                          const uint32_t* __restrict__ group_visible, int groups,
-                                                          uint32_t n_cap, gs355_header* __restrict__ header,
-                                                          bool header_known, uint32_t* __restrict__ lists,
-                                                          const uint32_t* bin_pairs, int bins, uint32_t* chunk_base)
+// Layout of the buckets from the tiles' totals: one wavefront per block of 64 tiles, four per workgroup.  Every
+// workgroup adds up the block totals itself (a few hundred words, at most 9000): those before its own blocks give its
+// first slot, all of them the frame's key count, which decides overflow before anything is published — so no
+// workgroup waits for another and no separate scan pass is launched.  Workgroup 0 also writes the frame header and
+// the work list of the scatter's second level: chunk_base[b] = chunks of kFineChunk pairs in the coarse bins before
+// b, chunk_base[bins] = all (`bin_pairs`, the pairs per bin, may be the same array).  With kTiles the wavefronts
+// publish tile bases, the scatter's cursors, the ranges and the lists of buckets too large for the small sorter
+// (`lists[0..3]` cleared by an earlier kernel); without, the columns are coarse bins and only their bases are
+// written.  `totals` and `tile_base` may be the same array.  `header_known`: second layout of a frame (by tile,
+// after the one by coarse bin): the header stands, and nothing is done on overflow.
+template <bool kTiles>
+__global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* totals, uint32_t tiles,
+                                                           const uint64_t* __restrict__ block_sums, uint32_t n_blocks,
+                                                           const uint32_t* __restrict__ group_visible, int groups,
+                                                           uint32_t n_cap, gs355_header* __restrict__ header,
+                                                           bool header_known, uint32_t* tile_base,
+                                                           uint32_t* __restrict__ ranges, uint32_t* __restrict__ lists,
+                                                           const uint32_t* bin_pairs, int bins, uint32_t* chunk_base)
 {
-    __shared__ uint64_t s_wave[16];
-    __shared__ uint32_t s_vis, s_chunks[16];
+    __shared__ uint64_t s_before[4], s_total[4];
+    __shared__ uint32_t s_vis[4], s_chunks[4];
     if (header_known && header->overflow) return;
-    if (threadIdx.x == 0) s_vis = 0;
-    __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    // every thread owns a run of consecutive blocks (9 at most for the largest image), so one scan over the 1024 run
-    // sums places them all
-    constexpr uint32_t kRun = (kBinMaxTilesWide / 64 + 1023) / 1024;
-    const uint32_t per = (n_blocks + 1023u) / 1024u;
-    const uint32_t b0 = min(threadIdx.x * per, n_blocks), b1 = min(b0 + per, n_blocks);
-    uint64_t v[kRun], mine = 0;
+    const uint32_t first_block = blockIdx.x * 4u, block = first_block + (uint32_t)wave;
+    {
+        uint64_t before = 0, total = 0;
+        for (uint32_t b = threadIdx.x; b < n_blocks; b += 256u) {
+            const uint64_t v = block_sums[b];
+            total += v;
+            before += b < first_block ? v : 0ull;
+        }
+        uint32_t vis = 0;
+        if (blockIdx.x == 0 && !header_known)
+            for (int c = threadIdx.x; c < groups; c += 256) vis += group_visible[c];
 #pragma unroll
-    for (uint32_t k = 0; k < kRun; ++k) {
-        v[k] = b0 + k < b1 ? blocks[b0 + k] : 0ull;
-        mine += v[k];
+        for (int d = 32; d > 0; d >>= 1) {
+            before += __shfl_down(before, d, 64);
+            total += __shfl_down(total, d, 64);
+            vis += __shfl_down(vis, d, 64);
+        }
+        if (lane == 0) {
+            s_before[wave] = before;
+            s_total[wave] = total;
+            s_vis[wave] = vis;
+        }
     }
-    uint32_t vis = 0;
-    for (int c = threadIdx.x; c < groups; c += 1024) vis += group_visible[c];
-    uint64_t inc = mine;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint64_t up = __shfl_up(inc, d, 64);
-        if (lane >= d) inc += up;
-    }
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) vis += __shfl_down(vis, d, 64);
-    if (lane == 63) s_wave[wave] = inc;
-    if (lane == 0 && vis) atomicAdd(&s_vis, vis);
     __syncthreads();
-    uint64_t total = 0, before = 0;
-    for (int w = 0; w < 16; ++w) {
-        if (w < wave) before += s_wave[w];
-        total += s_wave[w];
-    }
+    const uint64_t total = (s_total[0] + s_total[1]) + (s_total[2] + s_total[3]);
     const bool overflow = total > (uint64_t)n_cap;
-    if (threadIdx.x == 0 && !header_known) {
+    if (blockIdx.x == 0 && threadIdx.x == 0 && !header_known) {
         header->num_keys_total = total;
         header->num_keys = overflow ? n_cap : (uint32_t)total;
         header->overflow = overflow ? 1u : 0u;
-        header->num_visible = s_vis;
+        header->num_visible = (s_vis[0] + s_vis[1]) + (s_vis[2] + s_vis[3]);
     }
-    if (threadIdx.x < 4) lists[threadIdx.x] = 0u;  // the size-class lists are filled by tile_publish_kernel
-    uint64_t first = before + inc - mine;
-#pragma unroll
-    for (uint32_t k = 0; k < kRun; ++k) {
-        if (b0 + k < b1) blocks[b0 + k] = first;
-        first += v[k];
-    }
-    // The second scatter level works through every coarse bin in chunks of kFineChunk pairs: chunk_base[b] = chunks
-    // of the bins before b, chunk_base[bins] = all.  `bin_pairs` (pairs per bin) may be the same array.
-    if (bins > 0 && !overflow) {
-        const int per_thread = (bins + 1023) / 1024;
+    if (overflow) return;  // later stages do nothing either
+
+    if (blockIdx.x == 0 && bins > 0) {
+        const int per_thread = (bins + 255) / 256;
         const int q0 = min((int)threadIdx.x * per_thread, bins), q1 = min(q0 + per_thread, bins);
         uint32_t chunks = 0;
         for (int q = q0; q < q1; ++q) chunks += (bin_pairs[q] + (uint32_t)kFineChunk - 1u) / (uint32_t)kFineChunk;
@@ -566,23 +566,11 @@ __global__ __launch_bounds__(1024) void block_scan_kernel(uint64_t* __restrict__
             chunk_base[q] = run;
             run += n;
         }
-        if (threadIdx.x == 1023) chunk_base[bins] = run;
+        if (threadIdx.x == 255) chunk_base[bins] = run;
     }
-}
 
-// Second step, one wavefront per block of 64 tiles: tile bases (and, with kTiles, the scatter's cursors, the ranges
-// and the lists of buckets too large for the small sorter).  `totals` and `tile_base` may be the same array.  With
-// kTiles false the columns are coarse bins and only their bases are written.
-template <bool kTiles>
-__global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* totals, uint32_t tiles,
-                                                           const uint64_t* __restrict__ block_base,
-                                                           const gs355_header* __restrict__ header,
-                                                           uint32_t* tile_base, uint32_t* __restrict__ ranges,
-                                                           uint32_t* __restrict__ lists)
-{
-    if (header->overflow) return;  // later stages do nothing either
-    const int lane = threadIdx.x & 63;
-    const uint32_t block = blockIdx.x * 4u + (threadIdx.x >> 6);
+    uint64_t base = (s_before[0] + s_before[1]) + (s_before[2] + s_before[3]);  // first slot of the workgroup's blocks
+    for (int w = 0; w < wave; ++w) base += first_block + (uint32_t)w < n_blocks ? block_sums[first_block + w] : 0ull;
     const uint32_t t = block * 64u + (uint32_t)lane;
     const bool live = t < tiles;
     const uint32_t v = live ? totals[t] : 0u;
@@ -593,7 +581,7 @@ __global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* total
         if (lane >= d) inc += up;
     }
     if (block * 64u >= tiles) return;  // (uniform per wavefront)
-    const uint32_t first = (uint32_t)block_base[block] + inc - v;
+    const uint32_t first = (uint32_t)base + inc - v;
     if (live) tile_base[t] = first;
     if (!kTiles) return;
     if (live) {
@@ -1297,17 +1285,18 @@ int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint
 }
 
 // Bases of `columns` buckets from their totals (block sums already in `blocks`), and the per-tile outputs with kTiles.
+// `bases` may be `totals`, unless `bin_pairs` is `totals` too (workgroup 0 reads every bin's pairs while the others
+// already write bases).
 template <bool kTiles>
-static int launch_layout(uint32_t* totals_and_bases, int columns, uint64_t* blocks, const uint32_t* group_visible,
-                         int groups, uint32_t n_cap, gs355_header* header, bool header_known, uint32_t* ranges,
-                         uint32_t* lists, const uint32_t* bin_pairs, int bins, uint32_t* chunk_base, hipStream_t s)
+static int launch_layout(const uint32_t* totals, uint32_t* bases, int columns, const uint64_t* blocks,
+                         const uint32_t* group_visible, int groups, uint32_t n_cap, gs355_header* header,
+                         bool header_known, uint32_t* ranges, uint32_t* lists, const uint32_t* bin_pairs, int bins,
+                         uint32_t* chunk_base, hipStream_t s)
 {
     const int n_blocks = (columns + 63) / 64;
-    hipLaunchKernelGGL(block_scan_kernel, dim3(1), dim3(1024), 0, s, blocks, (uint32_t)n_blocks, group_visible, groups,
-                       n_cap, header, header_known, lists, bin_pairs, bins, chunk_base);
-    GS355_CHECK_LAUNCH("bin: block scan");
-    hipLaunchKernelGGL(tile_publish_kernel<kTiles>, dim3((n_blocks + 3) / 4), dim3(256), 0, s, totals_and_bases,
-                       (uint32_t)columns, blocks, header, totals_and_bases, ranges, lists);
+    hipLaunchKernelGGL(tile_publish_kernel<kTiles>, dim3((n_blocks + 3) / 4), dim3(256), 0, s, totals, (uint32_t)columns,
+                       blocks, (uint32_t)n_blocks, group_visible, groups, n_cap, header, header_known, bases, ranges, lists,
+                       bin_pairs, bins, chunk_base);
     GS355_CHECK_LAUNCH("bin: layout");
     return GS355_OK;
 }
@@ -1326,17 +1315,19 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
     if (tiles <= kBinMaxTiles) {
         // (the pairs of each coarse bin go to chunk_base, which the block scan turns into chunk bases in place)
         hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(256), 0, s, matrix, groups, tiles,
-                           tile_base, blocks, chunk_base);
+                           tile_base, blocks, chunk_base, lists);
         GS355_CHECK_LAUNCH("bin: slice prefix");
-        return launch_layout<true>(tile_base, tiles, blocks, group_visible, groups, n_cap, header, false, ranges, lists,
-                                   chunk_base, bins, chunk_base, s);
+        return launch_layout<true>(tile_base, tile_base, tiles, blocks, group_visible, groups, n_cap, header, false, ranges,
+                                   lists, chunk_base, bins, chunk_base, s);
     }
+    // (both in the cursor half of tile_base, which the tile-level layout of launch_tile_scatter overwrites later)
     uint32_t* bin_base = tile_base + tiles;
-    hipLaunchKernelGGL(slice_prefix_kernel, dim3((bins + 63) / 64), dim3(256), 0, s, matrix, groups, bins, bin_base,
-                       blocks, (uint32_t*)nullptr);
+    uint32_t* bin_pairs = bin_base + bins;
+    hipLaunchKernelGGL(slice_prefix_kernel, dim3((bins + 63) / 64), dim3(256), 0, s, matrix, groups, bins, bin_pairs,
+                       blocks, (uint32_t*)nullptr, lists);
     GS355_CHECK_LAUNCH("bin: slice prefix");
-    return launch_layout<false>(bin_base, bins, blocks, group_visible, groups, n_cap, header, false, ranges, lists,
-                                bin_base, bins, chunk_base, s);
+    return launch_layout<false>(bin_pairs, bin_base, bins, blocks, group_visible, groups, n_cap, header, false, ranges,
+                                lists, bin_pairs, bins, chunk_base, s);
 }
 
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
@@ -1375,10 +1366,10 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
         if ((rc = launch_fill_u32(tile_base, (size_t)T, 0u, s))) return rc;
         if ((rc = launch_fill_u32(reinterpret_cast<uint32_t*>(blocks), 2 * (size_t)((T + 63) / 64), 0u, s))) return rc;
         hipLaunchKernelGGL(fine_count_kernel, dim3(kFineGrid), dim3(kFineThreads), 0, s, header, bin_base, bins, T,
-                           chunk_bases(tile_base, T), coarse, tile_base, blocks);
+                           chunk_bases(tile_base, T), coarse, tile_base, blocks, lists);
         GS355_CHECK_LAUNCH("bin: fine count");
-        if ((rc = launch_layout<true>(tile_base, T, blocks, group_visible, groups, n_cap, header, true, ranges, lists,
-                                      (const uint32_t*)nullptr, 0, (uint32_t*)nullptr, s)))
+        if ((rc = launch_layout<true>(tile_base, tile_base, T, blocks, group_visible, groups, n_cap, header, true, ranges,
+                                      lists, (const uint32_t*)nullptr, 0, (uint32_t*)nullptr, s)))
             return rc;
     }
     if (fine) {

@@ -592,7 +592,7 @@ __global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* total
     // buckets beyond the smallest sorter's capacity go on the list of their size class (order within a list is free):
     // one request per wavefront and class
     int cls = -1;
-    if (v > (uint32_t)kTileSortCap[3]) cls = 3;
+    if (v > (uint32_t)kTileSortCap[3]) cls = -1;  // beyond the LDS sorters: sorted by its own workgroup of the class-0 kernel
     else if (v > (uint32_t)kTileSortCap[2]) cls = 2;
     else if (v > (uint32_t)kTileSortCap[1]) cls = 1;
     else if (v > (uint32_t)kTileSortCap[0]) cls = 0;
@@ -1119,11 +1119,13 @@ struct LdsSorter {
     }
 };
 
-// Smallest size class: one workgroup per tile (tiles with larger buckets leave at once).
+// Smallest size class: one workgroup per tile; tiles with larger buckets leave at once, except those beyond the
+// capacity of the largest LDS sorter, which are sorted here by radix passes through global memory, ping-ponging
+// between the bucket and the tile's slice of the output keys (their scratch lies over the LDS sorter's area).
 template <int kT, int kR>
 __global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* __restrict__ header,
                                                             const uint32_t* __restrict__ ranges,
-                                                            const uint64_t* __restrict__ buckets,
+                                                            uint64_t* __restrict__ buckets,
                                                             uint64_t* __restrict__ out_keys,
                                                             uint32_t* __restrict__ out_vals,
                                                             uint32_t* __restrict__ list_work)
@@ -1131,8 +1133,20 @@ __global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* 
     extern __shared__ uint32_t s_dyn[];
     if (blockIdx.x == 0 && threadIdx.x < 4) list_work[threadIdx.x] = 0u;  // for the list kernels launched after this one
     if (header->overflow) return;
+    static_assert(kT == kThreads, "the global-memory passes are written for kThreads threads");
+    static_assert((256 + kWaves * 256 + 8) * sizeof(uint32_t) <= LdsSorter<kT, kR>::kBytes, "scratch of the global passes");
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
+    if (n > (uint32_t)kTileSortCap[3]) {  // (uniform over the workgroup)
+        const SortScratch sc = {s_dyn, reinterpret_cast<uint32_t(*)[256]>(s_dyn + 256), s_dyn + 256 + kWaves * 256};
+        const GlobalPairs A = {buckets + lo}, B = {out_keys + lo};
+        const bool in_b = sort_pairs(A, B, n, sc);
+        // when the result sits in the output slice itself, each element is rewritten in place by the thread that read it
+        write_sorted(in_b ? B : A, n, tile, out_keys + lo, out_vals + lo);
+        return;
+    }
     const LdsSorter<kT, kR> sorter(s_dyn);
-    sorter.run(blockIdx.x, ranges, buckets, out_keys, out_vals);
+    sorter.run(tile, ranges, buckets, out_keys, out_vals);
 }
 
 // Larger size classes: persistent workgroups over the class list made by tile_publish_kernel.  A workgroup starts
@@ -1186,33 +1200,6 @@ __global__ __launch_bounds__(kT) void tile_sort_list_kernel(const gs355_header* 
 {
     extern __shared__ uint32_t s_dyn[];
     tile_sort_list_body<kT, kR>(header, ranges, list, list_count, work, buckets, out_keys, out_vals, s_dyn);
-}
-
-// Buckets beyond the LDS capacity: the same passes through global memory,
-// ping-ponging between the bucket and the tile's slice of the output keys.
-__global__ __launch_bounds__(kThreads) void tile_sort_huge_kernel(const gs355_header* __restrict__ header,
-                                                                  const uint32_t* __restrict__ ranges,
-                                                                  const uint32_t* __restrict__ lists, uint32_t tiles,
-                                                                  uint64_t* __restrict__ buckets,
-                                                                  uint64_t* __restrict__ out_keys,
-                                                                  uint32_t* __restrict__ out_vals)
-{
-    __shared__ uint32_t s_hist[256];
-    __shared__ uint32_t s_cnt[kWaves][256];
-    __shared__ uint32_t s_flags[8];
-    if (header->overflow) return;
-    const SortScratch sc = {s_hist, s_cnt, s_flags};
-    const uint32_t count = lists[3];
-    for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) {
-        const uint32_t tile = lists[kListHeader + 3 * (size_t)tiles + k];
-        const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
-        const GlobalPairs A = {buckets + lo}, B = {out_keys + lo};
-        const bool in_b = sort_pairs(A, B, n, sc);
-        // when the result sits in the output slice itself, each element is
-        // rewritten in place by the thread that read it
-        write_sorted(in_b ? B : A, n, tile, out_keys + lo, out_vals + lo);
-        __syncthreads();
-    }
 }
 
 }  // namespace
@@ -1406,9 +1393,6 @@ int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* rang
     hipLaunchKernelGGL((tile_sort_list_kernel<1024, 10>), grid(256), dim3(1024), S3::kBytes, s, header, ranges,
                        list0 + 2 * (size_t)tiles, lists + 2, work + 2, buckets, out_keys, out_vals);
     GS355_CHECK_LAUNCH("tile sort: class 3");
-    hipLaunchKernelGGL(tile_sort_huge_kernel, grid(256), dim3(kThreads), 0, s, header, ranges, lists, (uint32_t)tiles,
-                       buckets, out_keys, out_vals);
-    GS355_CHECK_LAUNCH("tile sort: beyond LDS");
     return GS355_OK;
 }
 

@@ -10,9 +10,9 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 # the kernels of the steady-state frame (the one-level scatter_kernel<0> only runs for a workspace's first frame there)
-SHIPPED_SORT_KERNELS = ("tile_count_kernel", "slice_prefix_kernel", "block_scan_kernel", "tile_publish_kernel", "scatter_kernel<4",
+SHIPPED_SORT_KERNELS = ("tile_count_kernel", "slice_prefix_kernel", "tile_publish_kernel", "scatter_kernel<4",
                         "fine_scatter_kernel", "tile_sort_each_kernel", "tile_sort_list_kernel",
-                        "tile_sort_list_1024x5_kernel", "tile_sort_huge_kernel")
+                        "tile_sort_list_1024x5_kernel")
 
 
 def load_bench():

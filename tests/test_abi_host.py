@@ -281,6 +281,58 @@ def test_decode_validates_before_any_hip_call():
     assert lib.gs355_decode_scratch_bytes(1000, C.byref(need)) == 0 and need.value >= 256
 
 
+def test_one_call_decode_validates_before_any_hip_call():
+    """gs355_decode / gs355_decode_workspace_bytes: phases, capacity, outputs, workspace, feature bank and level
+    input are all checked before anything could be launched."""
+    lib = _lib.load()
+    out = _lib.Decoded()
+
+    def dec(d, a, cap, o, ws, nbytes, phases):
+        return lib.gs355_decode(C.byref(d), C.byref(a), cap, C.byref(o) if o is not None else None, ws, nbytes, phases, None)
+
+    ok = (_decoder(), _anchors(), 100, out, 0x1000, 1 << 30)
+    assert "phases" in _err(_lib.GS355_EINVAL, dec, *ok, 0)
+    assert "phases" in _err(_lib.GS355_EINVAL, dec, *ok, 4)
+    assert "feat_dim" in _err(_lib.GS355_EINVAL, dec, _decoder(feat=64), *ok[1:], _lib.DECODE_ALL)
+    assert "capacity" in _err(_lib.GS355_EINVAL, dec, _decoder(), _anchors(), -1, out, 0x1000, 1 << 30, _lib.DECODE_ALL)
+    assert "capacity" in _err(_lib.GS355_EINVAL, dec, _decoder(), _anchors(), 1 << 32, out, 0x1000, 1 << 30, _lib.DECODE_ALL)
+    assert "outputs is NULL" in _err(_lib.GS355_EINVAL, dec, _decoder(), _anchors(), 100, None, 0x1000, 1 << 30,
+                                     _lib.DECODE_ALL)
+    assert "non-NULL" in _err(_lib.GS355_EINVAL, dec, *ok, _lib.DECODE_EMIT)  # the five output arrays are missing
+    assert "workspace is NULL" in _err(_lib.GS355_EINVAL, dec, _decoder(), _anchors(), 100, out, None, 1 << 30,
+                                       _lib.DECODE_COUNT)
+    assert "aligned" in _err(_lib.GS355_EINVAL, dec, _decoder(), _anchors(), 100, out, 0x1010, 1 << 30, _lib.DECODE_COUNT)
+    assert "needed" in _err(_lib.GS355_ENOSPC, dec, _decoder(), _anchors(A=100_000), 100, out, 0x1000, 64,
+                            _lib.DECODE_COUNT)
+    # level input: every head reads [feat | view | level] (36 columns) and the level array must be there
+    lvl = _decoder(in_dim=(36, 36, 36))
+    lvl.add_level = 1
+    assert "level" in _err(_lib.GS355_EINVAL, dec, lvl, _anchors(), 100, out, 0x1000, 1 << 30, _lib.DECODE_COUNT)
+    narrow = _decoder(in_dim=(35, 35, 35))
+    narrow.add_level = 1
+    an = _anchors()
+    an.level = 0x1000
+    assert _err(_lib.GS355_EINVAL, dec, narrow, an, 100, out, 0x1000, 1 << 30, _lib.DECODE_COUNT)
+    # feature bank: its input is [view] or [view | level], and all four weight arrays must be given
+    bank = _decoder()
+    bank.bank_in_dim = 5
+    assert "bank" in _err(_lib.GS355_EINVAL, dec, bank, _anchors(), 100, out, 0x1000, 1 << 30, _lib.DECODE_COUNT)
+    bank.bank_in_dim = 3
+    assert "bank" in _err(_lib.GS355_EINVAL, dec, bank, _anchors(), 100, out, 0x1000, 1 << 30, _lib.DECODE_COUNT)
+    # the two-call entry points have no workspace for the mixed features
+    bank.bank_w0 = bank.bank_b0 = bank.bank_w1 = bank.bank_b1 = 0x1000
+    assert "bank" in _err(_lib.GS355_EINVAL, lib.gs355_decode_count, C.byref(bank), C.byref(_anchors()), 0x1000, 0x1000,
+                          0x1000, 1 << 20, None)
+
+    need, with_bank = C.c_size_t(), C.c_size_t()
+    assert lib.gs355_decode_workspace_bytes(500_000, 10, 0, C.byref(need)) == 0
+    assert lib.gs355_decode_workspace_bytes(500_000, 10, 1, C.byref(with_bank)) == 0
+    assert need.value % 256 == 0 and with_bank.value >= need.value + 500_000 * 32 * 4
+    assert "offsets per anchor" in _err(_lib.GS355_EINVAL, lib.gs355_decode_workspace_bytes, 10, 11, 0, C.byref(need))
+    assert "A must be" in _err(_lib.GS355_EINVAL, lib.gs355_decode_workspace_bytes, -1, 10, 0, C.byref(need))
+    assert _err(_lib.GS355_EINVAL, lib.gs355_decode_workspace_bytes, 10, 10, 0, None)
+
+
 def test_header_is_plain_c(tmp_path):
     """include/gs355.h must compile as C99 (the boundary carries no C++ or torch types), and a C caller's view of the
     struct sizes must match what the Python binding assumes."""

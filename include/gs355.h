@@ -124,7 +124,8 @@ typedef struct gs355_layout {
     size_t values[2];     /* u32[n_cap] x 2 */
     size_t sort_hist;     /* u32[...] per-block digit histograms of the radix sort */
     size_t ranges;        /* u32[tiles][2] */
-    size_t bin_matrix;    /* u32[slices][tiles] pairs per (slice of Gaussians, tile), then their prefix over slices */
+    size_t bin_matrix;    /* u32[slices][tiles] pairs per (slice of Gaussians, tile), then their prefix over slices;
+                           * beyond 36000 tiles u32[slices][ceil(tiles/16)], per bin of 16 consecutive tiles */
     size_t tile_base;     /* u32[2][tiles]   first slot of each tile's bucket; its next free slot during the scatter;
                            * then u64[ceil(tiles/64)], the first slot of each block of 64 tiles, and
                            * u32[ceil(tiles/16)+1], the work list of the scatter's second level */

@@ -236,7 +236,7 @@ constexpr int kFineThreads = 512;
 constexpr int kFineWaves = kFineThreads / 64;
 constexpr int kFineItems = 8;                             // pairs per thread and chunk
 constexpr int kFineChunk = kFineThreads * kFineItems;  // 4096 pairs = 32 KB of LDS
-constexpr int kFineGrid = 1024;                          // four workgroups of 512 threads per CU
+constexpr int kFineGrid = 4096;                          // about one workgroup per chunk at 6M Gaussians, a few chunks each at 4K
 
 // A workgroup's run of chunks.  next() gives the following chunk's bin, first pair and pair count.
 struct ChunkRun {

@@ -228,15 +228,15 @@ __global__ __launch_bounds__(kBinThreads) void scatter_kernel(FrameArgs f, int32
 // at a time.  Chunks never cross a bin; chunk_base[b] = chunks of the bins before b, chunk_base[bins] = all of them
 // (tile_publish_kernel).  The kFineGrid workgroups take equal, contiguous runs of chunks, so every workgroup has work
 // however the pairs are spread over the bins, and a bin of many pairs is shared by many workgroups.  A chunk is split
-// by tile inside LDS first (wave-level ranking by the four tile bits, a scan over the 8 x 16 per-wave counts), the
+// by tile inside LDS first (wave-level ranking by the four tile bits, a scan over the per-wave counts), the
 // workgroup reserves a run of slots per bucket with one global atomic each, and consecutive lanes then store
 // consecutive pairs of one bucket: full-line writes instead of one memory transaction per pair.  Order inside a
 // bucket is arbitrary, as the sort expects.
-constexpr int kFineThreads = 512;
+constexpr int kFineThreads = 256;
 constexpr int kFineWaves = kFineThreads / 64;
 constexpr int kFineItems = 8;                             // pairs per thread and chunk
-constexpr int kFineChunk = kFineThreads * kFineItems;  // 4096 pairs = 32 KB of LDS
-constexpr int kFineGrid = 4096;                          // about one workgroup per chunk at 6M Gaussians, a few chunks each at 4K
+constexpr int kFineChunk = kFineThreads * kFineItems;  // 2048 pairs = 16 KB of LDS
+constexpr int kFineGrid = 8192;                          // a chunk per workgroup at 6M Gaussians / 1080p, a few each at 4K
 
 // A workgroup's run of chunks.  next() gives the following chunk's bin, first pair and pair count.
 struct ChunkRun {

@@ -173,7 +173,16 @@ __global__ __launch_bounds__(kBinThreads) void scatter_kernel(FrameArgs f, int32
         while (ta < tb) {
             const int stop = min(tb, ((ta >> kShift) + 1) << kShift);
             uint32_t slot = atomicAdd(&s_bin[ta >> kShift], (uint32_t)(stop - ta));
-            for (; ta < stop; ++ta) dst[slot++] = payload | (uint64_t)(ta & (kSpan - 1));
+            // the segment's slots are consecutive: two pairs per 16-byte store where the slot is even (every store
+            // is a 64-byte request on the way to the L2, however few bytes it carries)
+            if ((slot & 1u) && ta < stop) dst[slot++] = payload | (uint64_t)(ta++ & (kSpan - 1));
+            for (; ta + 1 < stop; ta += 2, slot += 2) {
+                ulonglong2 two;
+                two.x = payload | (uint64_t)(ta & (kSpan - 1));
+                two.y = payload | (uint64_t)((ta + 1) & (kSpan - 1));
+                *reinterpret_cast<ulonglong2*>(dst + slot) = two;
+            }
+            if (ta < stop) dst[slot] = payload | (uint64_t)(ta++ & (kSpan - 1));
         }
     };
 

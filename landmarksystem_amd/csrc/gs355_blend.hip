@@ -76,14 +76,28 @@ __device__ __forceinline__ float splat_exponent(float dx, float dy, float hx, fl
     return (t1 + t2) + t3;
 }
 
+// The hardware exp2 is monotone, so exp2(t) < 1/255 exactly when t < kAlphaCut, the smallest float whose exp2 reaches
+// 1/255 (found by running v_exp_f32 over every float between -8.2 and -7.8).  The shipped blend decides on t and
+// leaves the exp2 (a quarter-rate instruction) to the pairs that pass; the verification variant decides on the
+// exponential itself, and the tests hold the two to identical images on scenes full of opacities around 1/255.
+constexpr float kAlphaCut = -7.99435329f;  // bits 0xc0ffd1be
+
 // a = px, py, hx, ny;  b = hz, log2(opacity), r, g;  c = b, depth, reach_x, reach_y
+template <bool kCutOnExponent>
 __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, const float4 a, const float4 b,
                                           const float4 c)
 {
     const float dx = a.x - pxf, dy = a.y - pyf;
     const float power = splat_exponent(dx, dy, a.z, a.w, b.x);
-    const float alpha = fminf(0.99f, __builtin_amdgcn_exp2f(__builtin_fmaf(power, 1.4426950408889634f, b.y)));
-    if (power > 0.0f || alpha < 1.0f / 255.0f) return;
+    const float t = __builtin_fmaf(power, 1.4426950408889634f, b.y);
+    float alpha;
+    if (kCutOnExponent) {
+        if (power > 0.0f || t < kAlphaCut) return;
+        alpha = fminf(0.99f, __builtin_amdgcn_exp2f(t));
+    } else {
+        alpha = fminf(0.99f, __builtin_amdgcn_exp2f(t));
+        if (power > 0.0f || alpha < 1.0f / 255.0f) return;
+    }
     const float test_T = p.T * (1.0f - alpha);
     if (test_T >= 0.0001f) {
         const float w = alpha * p.T;
@@ -150,7 +164,7 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
     const char* const rec_b = reinterpret_cast<const char*>(s_b);
     const char* const rec_c = reinterpret_cast<const char*>(s_c);
     auto blend_entry = [&](uint32_t entry) {
-        blend_one(p, pxf, pyf, *reinterpret_cast<const float4*>(rec_a + entry),
+        blend_one<kCull>(p, pxf, pyf, *reinterpret_cast<const float4*>(rec_a + entry),
                   *reinterpret_cast<const float4*>(rec_b + entry), *reinterpret_cast<const float4*>(rec_c + entry));
     };
 

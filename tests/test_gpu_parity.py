@@ -202,11 +202,16 @@ def test_rerun_is_bit_identical(gpu_device):
 
 @pytest.mark.parametrize("make", [lambda: scenes.config3(P=400_000), lambda: scenes.config2(P=80_000),
                                   lambda: scenes.tiny_scene(P=3000, width=333, height=211, sh_degree=1, seed=2,
-                                                            log_scale_mean=-1.0)])
+                                                            log_scale_mean=-1.0),
+                                  lambda: crowded_scene(5000, width=96, height=80, seed=3),
+                                  lambda: crowded_scene(2000, width=160, height=96, seed=4),
+                                  lambda: scenes.config3()])
 def test_block_culling_is_result_neutral(gpu_device, make):
     """The blend stage skips (4x4 pixel block, Gaussian) pairs whose bounding box
-    shows alpha < 1/255 on all 16 pixels; the verification variant evaluates
-    every pair.  Both must give identical bits."""
+    shows alpha < 1/255 on all 16 pixels, and it takes the alpha < 1/255 decision on the exponent (against the
+    smallest argument whose hardware exp2 reaches 1/255); the verification variant evaluates every pair and compares
+    the exponential itself.  Both must give identical bits -- the crowded scenes consist of opacities 0.004 .. 0.024
+    around 1/255 = 0.0039, millions of decisions next to the threshold."""
     scene = make()
     s = settings_for(scene, gpu_device)
     inp = pipeline.FrameInputs(s, scene.means3D.to(gpu_device), opacities=scene.opacities.to(gpu_device),

@@ -44,7 +44,7 @@
 extern "C" {
 #endif
 
-#define GS355_VERSION 1
+#define GS355_VERSION 2
 #define GS355_API __attribute__((visibility("default")))
 #define GS355_TILE 16 /* tile edge in pixels */
 
@@ -98,6 +98,10 @@ typedef struct gs355_outputs {
     float *depth;   /* [H,W]  sum of depth * alpha * T, or NULL */
     float *alpha;   /* [H,W]  1 - T_final, or NULL */
     int32_t *radii; /* [P] */
+    /* Optional (NULL = unused): where the stage that writes the workspace header (scan or tile count) stores a
+     * second copy of its 64 bytes.  Pinned host memory is fine (the GPU addresses it like its own): the caller
+     * then learns the key count and the overflow flag by waiting for that stage, without enqueuing a copy. */
+    void *header_copy;
 } gs355_outputs;
 
 /* Words of the workspace header (u32 unless noted), written by the scan stage (classic pipeline) or the

@@ -60,7 +60,8 @@ class Gaussians(C.Structure):
 
 
 class Outputs(C.Structure):
-    _fields_ = [("image", C.c_void_p), ("depth", C.c_void_p), ("alpha", C.c_void_p), ("radii", C.c_void_p)]
+    _fields_ = [("image", C.c_void_p), ("depth", C.c_void_p), ("alpha", C.c_void_p), ("radii", C.c_void_p),
+                ("header_copy", C.c_void_p)]
 
 
 class Header(C.Structure):

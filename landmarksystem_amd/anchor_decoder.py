@@ -248,11 +248,16 @@ class FusedAnchorDecoder(nn.Module):
         if self.dist2level == "progressive" and prog_ratio is not None and transition_mask is not None:
             raise NotImplementedError("progressive level-of-detail opacity scaling is not part of this decoder")
         dev, A, dec, an, tensors = self._marshal(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, level)
-        counts = torch.empty(2, dtype=torch.int32, device=dev)
+        # the two counters go straight into pinned host memory (which the GPU addresses like its own): no copy is
+        # enqueued, the host waits for the count phase and reads them
+        if self._host_count is None:
+            self._host_count = torch.zeros(2, dtype=torch.int32, pin_memory=True)
+        counts = self._host_count
         o = _lib.Decoded()
         o.count, o.num_visible = counts.data_ptr(), counts.data_ptr() + 4
         self._run(dec, an, 0, o, _lib.DECODE_COUNT, dev)
-        G, a_vis = self.read_counts(counts)
+        torch.cuda.current_stream(dev).synchronize()
+        G, a_vis = int(counts[0]), int(counts[1])
         f = lambda *shape: torch.empty(shape, dtype=torch.float32, device=dev)  # noqa: E731
         out = (f(G, 3), f(G, 3), f(G, 1), f(G, 3), f(G, 4))
         extra = (None, None)

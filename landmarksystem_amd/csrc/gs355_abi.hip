@@ -240,7 +240,9 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     if (stage_mask & GS355_STAGE_PREPROCESS)
         if ((rc = launch_preprocess(fa, *g, false, records, touched, rects, depth_bits, out->radii, s))) return rc;
     if (stage_mask & GS355_STAGE_SCAN)
-        if ((rc = launch_scan_offsets(touched, out->radii, g->P, g->P_device, offsets, scan_tmp, header, cap, s))) return rc;
+        if ((rc = launch_scan_offsets(touched, out->radii, g->P, g->P_device, offsets, scan_tmp, header,
+                                      static_cast<gs355_header*>(out->header_copy), cap, s)))
+            return rc;
     if (stage_mask & GS355_STAGE_DUPLICATE)
         if ((rc = launch_duplicate(fa, g->P, records, out->radii, offsets, header, keys[0], vals[0], s))) return rc;
     if (stage_mask & GS355_STAGE_SORT)
@@ -253,7 +255,8 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
     uint64_t* buckets = keys[1 - L.sorted_buffer];
     if (stage_mask & GS355_STAGE_TILE_COUNT) {
         if ((rc = launch_tile_count(fa, g->P, rects, bin_matrix, bin_visible, s))) return rc;
-        if ((rc = launch_tile_layout(g->P, bin_matrix, bin_visible, tiles, cap, header, tile_base, ranges, tile_lists,
+        if ((rc = launch_tile_layout(g->P, bin_matrix, bin_visible, tiles, cap, header,
+                                     static_cast<gs355_header*>(out->header_copy), tile_base, ranges, tile_lists,
                                      s)))
             return rc;
     }

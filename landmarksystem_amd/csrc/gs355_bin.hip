@@ -513,7 +513,8 @@ __global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* total
                                                            const uint64_t* __restrict__ block_sums, uint32_t n_blocks,
                                                            const uint32_t* __restrict__ group_visible, int groups,
                                                            uint32_t n_cap, gs355_header* __restrict__ header,
-                                                           bool header_known, uint32_t* tile_base,
+                                                           gs355_header* __restrict__ header_copy, bool header_known,
+                                                           uint32_t* tile_base,
                                                            uint32_t* __restrict__ ranges, uint32_t* __restrict__ lists,
                                                            const uint32_t* bin_pairs, int bins, uint32_t* chunk_base)
 {
@@ -552,6 +553,12 @@ __global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* total
         header->num_keys = overflow ? n_cap : (uint32_t)total;
         header->overflow = overflow ? 1u : 0u;
         header->num_visible = (s_vis[0] + s_vis[1]) + (s_vis[2] + s_vis[3]);
+        if (header_copy) {  // (may be host memory: plain stores, complete when the kernel is)
+            header_copy->num_keys_total = total;
+            header_copy->num_keys = overflow ? n_cap : (uint32_t)total;
+            header_copy->overflow = overflow ? 1u : 0u;
+            header_copy->num_visible = (s_vis[0] + s_vis[1]) + (s_vis[2] + s_vis[3]);
+        }
     }
     if (overflow) return;  // later stages do nothing either
 
@@ -1286,12 +1293,12 @@ int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint
 template <bool kTiles>
 static int launch_layout(const uint32_t* totals, uint32_t* bases, int columns, const uint64_t* blocks,
                          const uint32_t* group_visible, int groups, uint32_t n_cap, gs355_header* header,
-                         bool header_known, uint32_t* ranges, uint32_t* lists, const uint32_t* bin_pairs, int bins,
+                         gs355_header* header_copy, bool header_known, uint32_t* ranges, uint32_t* lists, const uint32_t* bin_pairs, int bins,
                          uint32_t* chunk_base, hipStream_t s)
 {
     const int n_blocks = (columns + 63) / 64;
     hipLaunchKernelGGL(tile_publish_kernel<kTiles>, dim3((n_blocks + 3) / 4), dim3(256), 0, s, totals, (uint32_t)columns,
-                       blocks, (uint32_t)n_blocks, group_visible, groups, n_cap, header, header_known, bases, ranges, lists,
+                       blocks, (uint32_t)n_blocks, group_visible, groups, n_cap, header, header_copy, header_known, bases, ranges, lists,
                        bin_pairs, bins, chunk_base);
     GS355_CHECK_LAUNCH("bin: layout");
     return GS355_OK;
@@ -1301,7 +1308,7 @@ static int launch_layout(const uint32_t* totals, uint32_t* bases, int columns, c
 // header).  Beyond: the header and the coarse bins' bases (in tile_cursor[0, bins)); the per-tile layout follows
 // in launch_tile_scatter once the pairs of each bin can be counted by tile.
 int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visible, int tiles, uint32_t n_cap,
-                       gs355_header* header, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s)
+                       gs355_header* header, gs355_header* header_copy, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s)
 {
     int per_group;
     const int groups = bin_groups(P, &per_group);
@@ -1313,7 +1320,7 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
         hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(256), 0, s, matrix, groups, tiles,
                            tile_base, blocks, chunk_base, lists);
         GS355_CHECK_LAUNCH("bin: slice prefix");
-        return launch_layout<true>(tile_base, tile_base, tiles, blocks, group_visible, groups, n_cap, header, false, ranges,
+        return launch_layout<true>(tile_base, tile_base, tiles, blocks, group_visible, groups, n_cap, header, header_copy, false, ranges,
                                    lists, chunk_base, bins, chunk_base, s);
     }
     // (both in the cursor half of tile_base, which the tile-level layout of launch_tile_scatter overwrites later)
@@ -1322,7 +1329,7 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
     hipLaunchKernelGGL(slice_prefix_kernel, dim3((bins + 63) / 64), dim3(256), 0, s, matrix, groups, bins, bin_pairs,
                        blocks, (uint32_t*)nullptr, lists);
     GS355_CHECK_LAUNCH("bin: slice prefix");
-    return launch_layout<false>(bin_pairs, bin_base, bins, blocks, group_visible, groups, n_cap, header, false, ranges,
+    return launch_layout<false>(bin_pairs, bin_base, bins, blocks, group_visible, groups, n_cap, header, header_copy, false, ranges,
                                 lists, bin_pairs, bins, chunk_base, s);
 }
 
@@ -1364,7 +1371,7 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
         hipLaunchKernelGGL(fine_count_kernel, dim3(kFineGrid), dim3(kFineThreads), 0, s, header, bin_base, bins, T,
                            chunk_bases(tile_base, T), coarse, tile_base, blocks, lists);
         GS355_CHECK_LAUNCH("bin: fine count");
-        if ((rc = launch_layout<true>(tile_base, tile_base, T, blocks, group_visible, groups, n_cap, header, true, ranges,
+        if ((rc = launch_layout<true>(tile_base, tile_base, T, blocks, group_visible, groups, n_cap, header, nullptr, true, ranges,
                                       lists, (const uint32_t*)nullptr, 0, (uint32_t*)nullptr, s)))
             return rc;
     }

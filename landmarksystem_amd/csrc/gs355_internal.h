@@ -86,7 +86,7 @@ __device__ __forceinline__ Rect tile_rect(float px, float py, int radius, int gr
 int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_only, float* records,
                       uint32_t* tiles_touched, uint64_t* rects, uint32_t* depth_bits, int32_t* radii, hipStream_t s);
 int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int32_t P, const uint32_t* p_device,
-                        uint32_t* offsets, uint32_t* scan_tmp, gs355_header* header, uint32_t n_cap, hipStream_t s);
+                        uint32_t* offsets, uint32_t* scan_tmp, gs355_header* header, gs355_header* header_copy, uint32_t n_cap, hipStream_t s);
 int launch_anchor_filter(const FrameArgs& f, const gs355_gaussians& g, const FilterArgs& x, int32_t* radii, hipStream_t s);
 int launch_duplicate(const FrameArgs& f, int32_t P, const float* records, const int32_t* radii,
                      const uint32_t* offsets, const gs355_header* header, uint64_t* keys, uint32_t* values,
@@ -138,7 +138,7 @@ inline size_t bin_matrix_words(size_t tiles)
 int launch_tile_count(const FrameArgs& f, int32_t P, const uint64_t* rects, uint32_t* matrix, uint32_t* group_visible,
                       hipStream_t s);
 int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visible, int tiles, uint32_t n_cap,
-                       gs355_header* header, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s);
+                       gs355_header* header, gs355_header* header_copy, uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, hipStream_t s);
 // `coarse`: a second buffer of the buckets' size (first level of the two-level scatter).  `levels`: 1 or 2 = that
 // scatter whatever the frame holds, 0 = chosen on the device by the key count (both variants are launched); images
 // beyond kBinMaxTiles tiles always take two levels

@@ -93,7 +93,8 @@ __global__ __launch_bounds__(kScanThreads) void tile_sum_kernel(const uint32_t* 
 
 // ---- one workgroup: exclusive scan of the tile sums (in place), totals -----
 __global__ __launch_bounds__(256) void scan_sums_kernel(uint64_t* __restrict__ sums, const uint32_t* __restrict__ visible,
-                                                        uint32_t nb, gs355_header* __restrict__ header, uint32_t n_cap)
+                                                        uint32_t nb, gs355_header* __restrict__ header, uint32_t n_cap,
+                                                        gs355_header* __restrict__ header_copy)
 {
     __shared__ uint64_t s_wave[4];
     __shared__ uint64_t s_carry;
@@ -127,6 +128,12 @@ __global__ __launch_bounds__(256) void scan_sums_kernel(uint64_t* __restrict__ s
             header->num_keys = total > n_cap ? n_cap : (uint32_t)total;
             header->overflow = total > n_cap ? 1u : 0u;
             header->num_visible = s_vis[0] + s_vis[1] + s_vis[2] + s_vis[3];
+            if (header_copy) {  // (may be host memory: plain stores, complete when the kernel is)
+                header_copy->num_keys_total = total;
+                header_copy->num_keys = total > n_cap ? n_cap : (uint32_t)total;
+                header_copy->overflow = total > n_cap ? 1u : 0u;
+                header_copy->num_visible = s_vis[0] + s_vis[1] + s_vis[2] + s_vis[3];
+            }
         }
     }
 }
@@ -174,7 +181,8 @@ size_t scan_tmp_words(size_t n)
 }
 
 int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int32_t P, const uint32_t* p_device,
-                        uint32_t* offsets, uint32_t* scan_tmp, gs355_header* header, uint32_t n_cap, hipStream_t s)
+                        uint32_t* offsets, uint32_t* scan_tmp, gs355_header* header, gs355_header* header_copy,
+                        uint32_t n_cap, hipStream_t s)
 {
     const uint32_t nb = (uint32_t)(((size_t)P + kScanTile - 1) / kScanTile);
     uint64_t* sums = reinterpret_cast<uint64_t*>(scan_tmp);
@@ -184,7 +192,7 @@ int launch_scan_offsets(const uint32_t* tiles_touched, const int32_t* radii, int
                            p_device, sums, visible);
         GS355_CHECK_LAUNCH("scan: tile sums");
     }
-    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, s, sums, visible, nb, header, n_cap);
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, s, sums, visible, nb, header, n_cap, header_copy);
     GS355_CHECK_LAUNCH("scan: sums");
     if (nb) {
         hipLaunchKernelGGL(tile_scan_kernel<true>, dim3(nb), dim3(kScanThreads), 0, s, tiles_touched, (size_t)P,
@@ -203,7 +211,7 @@ int launch_exclusive_scan(const uint32_t* in, uint32_t* out, size_t n, uint32_t*
                        (const uint32_t*)nullptr, sums, (uint32_t*)nullptr);
     GS355_CHECK_LAUNCH("scan: tile sums");
     hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, s, sums, (const uint32_t*)nullptr, nb,
-                       (gs355_header*)nullptr, 0u);
+                       (gs355_header*)nullptr, 0u, (gs355_header*)nullptr);
     GS355_CHECK_LAUNCH("scan: sums");
     hipLaunchKernelGGL(tile_scan_kernel<false>, dim3(nb), dim3(kScanThreads), 0, s, in, n, (const uint32_t*)nullptr, sums,
                        out);

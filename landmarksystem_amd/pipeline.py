@@ -267,10 +267,10 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
     """All stages of one frame (`classic`: through scan / duplicate / radix sort / ranges even where the
     tile-bucketed stages apply; same results).
 
-    The key count is only known on the device after the scan.  The header is
-    copied to pinned host memory right after the scan and the remaining stages
-    are enqueued against the current capacity without waiting; the host then
-    waits for that small copy only (the GPU keeps working on sort and blend).
+    The key count is only known on the device after the scan.  The kernel that
+    computes it also stores the header in pinned host memory; the remaining stages
+    are enqueued against the current capacity without waiting, and the host then
+    waits for that kernel only (the GPU keeps working on sort and blend).
     If the frame needed more keys than the capacity, it is redone once with
     the exact requirement plus headroom; capacity never shrinks."""
     ws = ws or default_workspace(inputs.device)
@@ -288,8 +288,10 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
         back = _lib.STAGE_DUPLICATE | _lib.STAGE_SORT | _lib.STAGE_RANGES | _lib.STAGE_BLEND
     for attempt in range(3):
         n_cap = ws.key_capacity
-        layout = run_stages(inputs, out, ws, n_cap, front)
-        ws.header_host.copy_(ws.buffer[layout.header:layout.header + 64].view(torch.int64), non_blocking=True)
+        # the stage that produces the header also stores it in pinned host memory (no copy is enqueued)
+        out.c.header_copy = ws.header_host.data_ptr()
+        run_stages(inputs, out, ws, n_cap, front)
+        out.c.header_copy = None
         ws.header_event.record(torch.cuda.current_stream(inputs.device))
         run_stages(inputs, out, ws, n_cap, back)
         ws.header_event.synchronize()

@@ -23,7 +23,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert names == sorted(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.gs355_version() == 1
+    assert lib.gs355_version() == 2
 
 
 def test_struct_sizes_match_the_header():
@@ -31,7 +31,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(_lib.Header) == 64
     assert C.sizeof(_lib.Frame) == 7 * 4 + 4 + 4 * 8  # 7 scalars, padding to 8, 4 pointers
     assert C.sizeof(_lib.Gaussians) == 8 + 8 * 8  # P (padded to 8), 7 tensors, the optional device-side count
-    assert C.sizeof(_lib.Outputs) == 4 * 8
+    assert C.sizeof(_lib.Outputs) == 5 * 8  # image, depth, alpha, radii, the optional second copy of the header
     assert C.sizeof(_lib.Layout) == 18 * 8 + 4 * 4
     assert C.sizeof(_lib.AnchorLod) == 2 * 8 + 4 * 4 + 2 * 4
     assert C.sizeof(_lib.BackwardInputs) == 7 * 8 and C.sizeof(_lib.Gradients) == 8 * 8

@@ -79,6 +79,16 @@ __global__ __launch_bounds__(kBinThreads) void tile_count_kernel(FrameArgs f, in
                     ++visible;
                     if (area > kInlineTiles) {
                         s_queue[atomicAdd(&s_nqueue, 1u)] = (uint32_t)i;
+                    } else if (kWide) {  // a rectangle row: one request per coarse bin it crosses
+                        for (int ty = y0; ty < y1; ++ty) {
+                            int ta = ty * f.grid_x + x0;
+                            const int tb = ty * f.grid_x + x1;
+                            while (ta < tb) {
+                                const int stop = min(tb, ((ta >> kCoarseShift) + 1) << kCoarseShift);
+                                atomicAdd(&s_count[ta >> kCoarseShift], (uint32_t)(stop - ta));
+                                ta = stop;
+                            }
+                        }
                     } else {
                         for (int ty = y0; ty < y1; ++ty)
                             for (int tx = x0; tx < x1; ++tx) add(ty * f.grid_x + tx);

@@ -40,7 +40,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 COUNTER_TRAFFIC = {
     "source": "profiles/bench_c3_6M_1080p_hbm_traffic.txt",
     "workload": "configs[2]",
-    "bytes": {"blend": 1846.2e6, "preprocess": 1701.9e6, "keys_sort_ranges": 834.6e6},
+    "bytes": {"blend": 1846.2e6, "preprocess": 1701.9e6, "keys_sort_ranges": 834.7e6},
     # fp32 flops the blend kernel issues per launch (64 lanes x (2 FMA + MUL + ADD) wavefront instructions), from
     # profiles/bench_c3_6M_1080p_valu_counters.txt
     "blend_issued_flops": 10.86e9,

@@ -255,10 +255,10 @@ def backward_report(torch, pipeline, inp, n_cap, N, V, P, sh_coeffs, ms_per_step
         e1.record()
         torch.cuda.synchronize()
         t_bwd[label] = e0.elapsed_time(e1) / stage_steps
-    # algorithmic bytes: a 64-B gradient record per key written and 48 B of it read back; per key the sorted
+    # algorithmic bytes: a 48-B gradient record per key written and read back; per key the sorted
     # value, the 48-B record of its Gaussian, rectangle and first-record index; per visible Gaussian its inputs
     # and record; per Gaussian radius, key count, first-record index and every gradient written
-    bwd_bytes = N * (64 + 48 + 4 + 48 + 12) + V * (12 + 12 + 16 + 4 * 3 * sh_coeffs + 48) + \
+    bwd_bytes = N * (48 + 48 + 4 + 48 + 12) + V * (12 + 12 + 16 + 4 * 3 * sh_coeffs + 48) + \
         P * (12 + 12 + 12 + 4 + 12 + 16 + 4 * 3 * sh_coeffs)
     return {"ms": round(t_bwd["all_gradients"], 4), "ms_without_sh_gradient": round(t_bwd["without_sh_gradient"], 4),
             "bytes": bwd_bytes, "GBps": round(bwd_bytes / t_bwd["all_gradients"] / 1e6, 1),

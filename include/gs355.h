@@ -230,7 +230,7 @@ GS355_API int gs355_anchor_filter(const gs355_frame *frame, const gs355_gaussian
  * origin_gs/gs_model.py:129-139,225-236).  It runs over the workspace the forward pass of the same frame left
  * behind (records, sorted values, ranges: nothing else may have used that workspace in between) and the
  * forward outputs. */
-#define GS355_KEY_GRAD_FLOATS 16 /* scratch floats per (tile, Gaussian) key */
+#define GS355_KEY_GRAD_FLOATS 12 /* scratch floats per (tile, Gaussian) key */
 
 typedef struct gs355_backward_inputs {
     const float *image;     /* [3,H,W] forward output */
@@ -258,7 +258,7 @@ typedef struct gs355_gradients {
     float *cov3D_precomp;  /* [P,6] */
 } gs355_gradients;
 
-/* Bytes of scratch gs355_render_backward needs for P Gaussians and a key capacity of n_cap: one 64-byte
+/* Bytes of scratch gs355_render_backward needs for P Gaussians and a key capacity of n_cap: one 48-byte
  * gradient record per key, and the index of each Gaussian's first record. */
 GS355_API int gs355_backward_scratch_bytes(int32_t P, int64_t n_cap, size_t *bytes);
 

@@ -11,7 +11,7 @@
 //                    division by a transmittance and no second, reversed walk.  Per-pair contributions are summed
 //                    over the 16 pixels of a block by lane exchanges inside the 16-lane row, added to the staged
 //                    Gaussian's accumulators in LDS (one LDS atomic per step: LDS float atomics are slow), and
-//                    written once per batch of 256 as one 64-byte record per (tile, Gaussian) key.  No global
+//                    written once per batch of 256 as one 48-byte record per (tile, Gaussian) key.  No global
 //                    atomics (they cost more than the rest of the kernel): the records of a Gaussian are
 //                    consecutive, in the order its tile rectangle is walked, and the next kernel sums them in
 //                    that order, so gradients are identical from run to run.
@@ -26,7 +26,7 @@ namespace gs355 {
 namespace {
 
 constexpr int kGradFloats = 12;  // accumulators per staged Gaussian in LDS: 10 used
-constexpr int kKeyFloats = GS355_KEY_GRAD_FLOATS;  // per-key record: dpx, dpy, dconic xyz, dopacity, drgb, ddepth, 6 unused
+constexpr int kKeyFloats = GS355_KEY_GRAD_FLOATS;  // per-key record: dpx, dpy, dconic xyz, dopacity, drgb, ddepth, 2 unused
 
 // Record slot of the key (tile, Gaussian): the Gaussian's keys in the order its tile rectangle is walked
 // (row by row), after those of all Gaussians before it.
@@ -237,7 +237,6 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
             dst[0] = make_float4(-(a.z * m[0] + a.w * m[1]), -(cz * m[1] + a.w * m[0]), -0.5f * m[2], -m[3]);
             dst[1] = make_float4(-0.5f * m[4], m[5], m[6], m[7]);
             dst[2] = make_float4(m[8], m[9], 0.f, 0.f);
-            dst[3] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
     // keys the tile never reached (every pixel finished before them) contribute nothing: every record is written
@@ -245,7 +244,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
         const uint32_t g = values[j];
         float4* __restrict__ dst =
             reinterpret_cast<float4*>(key_grads + (size_t)key_slot(first_key[g], rects[g], tile_x, tile_y) * kKeyFloats);
-        dst[0] = dst[1] = dst[2] = dst[3] = make_float4(0.f, 0.f, 0.f, 0.f);
+        dst[0] = dst[1] = dst[2] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
 
@@ -340,7 +339,7 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(FrameArgs f, g
                 for (int u = 0; u < 4; ++u) {
                     const size_t k = min(k0 + (uint32_t)u, n - 1);
 #pragma unroll
-                    for (int q = 0; q < 3; ++q) r[u][q] = rec[4 * k + q];
+                    for (int q = 0; q < 3; ++q) r[u][q] = rec[3 * k + q];
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {

@@ -530,3 +530,36 @@ def test_non_finite_and_degenerate_inputs(gpu_device):
         ok = np.isfinite(r) & (ref["fragile"] == 0)
         assert (np.abs(g - r)[ok] <= 1e-4 * np.maximum(1.0, np.abs(r[ok]))).all(), name  # one colour is 1e29
         np.testing.assert_array_equal(fast[name], g)
+
+
+@pytest.mark.parametrize("modifier", [_lib.STAGE_TILE_SCATTER_ONE_LEVEL, _lib.STAGE_TILE_SCATTER_TWO_LEVEL, 0])
+def test_device_side_count_equals_a_shorter_input(gpu_device, modifier):
+    """gs355_gaussians.P_device: arrays sized for a capacity, the number of Gaussians in a device word.  Every stage
+    (both scatter variants) must give what the same call over the first `count` rows gives."""
+    scene = scenes.config2(P=120_000, width=800, height=450)
+    d = scene.to(gpu_device)
+    s = settings_for(scene, gpu_device)
+    count = 77_777
+    mask = _lib.PIPELINE_FAST | modifier
+
+    def run(n_rows, count_tensor):
+        inp = pipeline.FrameInputs(s, d.means3D[:n_rows], opacities=d.opacities[:n_rows], shs=d.shs[:n_rows],
+                                   scales=d.scales[:n_rows], rotations=d.rotations[:n_rows], count=count_tensor)
+        out = pipeline.FrameOutputs(inp)
+        out.radii.zero_()
+        ws = pipeline.Workspace(gpu_device)
+        lay = pipeline.run_stages(inp, out, ws, 4_000_000, mask)
+        torch.cuda.synchronize()
+        n = int(ws.view(lay, "header", inp.P, 0, inp.tiles)[0].item())
+        return dict(n=n, keys=u64(ws.view(lay, "sorted_keys", inp.P, n, inp.tiles)),
+                    values=u32(ws.view(lay, "sorted_values", inp.P, n, inp.tiles)),
+                    ranges=u32(ws.view(lay, "ranges", inp.P, n, inp.tiles)), image=out.image.cpu().numpy(),
+                    radii=out.radii.cpu().numpy())
+
+    short = run(count, None)
+    capped = run(scene.P, torch.tensor([count], dtype=torch.int32, device=gpu_device))
+    assert short["n"] == capped["n"] > 100_000
+    for name in ("keys", "values", "ranges", "image"):
+        np.testing.assert_array_equal(capped[name], short[name], err_msg=name)
+    np.testing.assert_array_equal(capped["radii"][:count], short["radii"])
+    assert not capped["radii"][count:].any()  # rows at and beyond the count are left alone

@@ -40,7 +40,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 COUNTER_TRAFFIC = {
     "source": "profiles/bench_c3_6M_1080p_hbm_traffic.txt",
     "workload": "configs[2]",
-    "bytes": {"blend": 1846.2e6, "preprocess": 1701.9e6, "keys_sort_ranges": 834.7e6},
+    "bytes": {"blend": 1846.0e6, "preprocess": 1701.9e6, "keys_sort_ranges": 834.2e6},
     # fp32 flops the blend kernel issues per launch (64 lanes x (2 FMA + MUL + ADD) wavefront instructions), from
     # profiles/bench_c3_6M_1080p_valu_counters.txt
     "blend_issued_flops": 10.86e9,
@@ -119,8 +119,16 @@ def stage_breakdown(torch, pipeline, _lib, inp, n_cap, steps):
     duplicate / LSD radix sort / ranges stages it replaces."""
     ws = pipeline.Workspace(inp.device)
     out = pipeline.FrameOutputs(inp)
+    # like render() on a steady stream of frames, the sort stage leaves out the launches of the sorter size classes
+    # that this frame leaves empty (a hint to the library, read from the header the tile-count stage writes)
+    lay = pipeline.run_stages(inp, out, ws, n_cap, _lib.STAGE_PREPROCESS | _lib.STAGE_TILE_COUNT)
+    torch.cuda.synchronize()
+    words = [int(w) for w in ws.view(lay, "header", inp.P, 0, inp.tiles)[:4].tolist()]
+    class_counts = ((words[2] >> 32) & 0xFFFFFFFF, words[3] & 0xFFFFFFFF, (words[3] >> 32) & 0xFFFFFFFF)
+    skip = sum(m for m, c in zip(_lib.STAGE_TILESORT_SKIP, class_counts) if c == 0)
     fast = [("preprocess", _lib.STAGE_PREPROCESS), ("tile_count", _lib.STAGE_TILE_COUNT),
-            ("tile_scatter", _lib.STAGE_TILE_SCATTER), ("tile_sort", _lib.STAGE_TILESORT), ("blend", _lib.STAGE_BLEND)]
+            ("tile_scatter", _lib.STAGE_TILE_SCATTER), ("tile_sort", _lib.STAGE_TILESORT | skip),
+            ("blend", _lib.STAGE_BLEND)]
     classic = [("scan", _lib.STAGE_SCAN), ("duplicate", _lib.STAGE_DUPLICATE), ("sort", _lib.STAGE_SORT),
                ("ranges", _lib.STAGE_RANGES)]
     ms = time_stages(torch, pipeline, inp, out, ws, n_cap, fast, steps)
@@ -129,7 +137,8 @@ def stage_breakdown(torch, pipeline, _lib, inp, n_cap, steps):
     hdr = ws.view(lay, "header", inp.P, 0, inp.tiles).cpu()
     ranges = ws.view(lay, "ranges", inp.P, 0, inp.tiles).cpu().numpy().view("uint32")
     stats = {"num_keys": int(hdr[0]), "num_visible": int(hdr[2]) & 0xFFFFFFFF,
-             "range_sum": int((ranges[:, 1].astype("int64") - ranges[:, 0]).sum()), "sort_passes": int(lay.sort_passes)}
+             "range_sum": int((ranges[:, 1].astype("int64") - ranges[:, 0]).sum()), "sort_passes": int(lay.sort_passes),
+             "sort_class_buckets": list(class_counts)}
     return ms, stats
 
 

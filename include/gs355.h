@@ -111,7 +111,11 @@ typedef struct gs355_header {
     uint32_t num_keys;       /* min(num_keys_total, key capacity): what later stages process */
     uint32_t overflow;       /* 1 if num_keys_total > key capacity (the frame must be redone with more) */
     uint32_t num_visible;    /* Gaussians with radius > 0 */
-    uint32_t reserved[11];
+    /* Tile-count stage, images of at most 36000 tiles: buckets in each of the three larger sorter size classes
+     * (1025..2048, 2049..5120, 5121..10240 pairs); 0xFFFFFFFF = not counted (scan stage, larger images).  What a
+     * caller needs to choose GS355_STAGE_TILESORT_SKIP_* for the next frame. */
+    uint32_t sort_class_count[3];
+    uint32_t reserved[8];
 } gs355_header;
 
 /* Byte offsets of every array inside the caller's workspace (each 256-byte
@@ -132,7 +136,8 @@ typedef struct gs355_layout {
                            * beyond 36000 tiles u32[slices][ceil(tiles/16)], per bin of 16 consecutive tiles */
     size_t tile_base;     /* u32[2][tiles]   first slot of each tile's bucket; its next free slot during the scatter;
                            * then u64[ceil(tiles/64)], the first slot of each block of 64 tiles, and
-                           * u32[ceil(tiles/16)+1], the work list of the scatter's second level */
+                           * u32[ceil(tiles/16)+1], the work list of the scatter's second level, and
+                           * u32[ceil(tiles/64)], buckets per larger sorter size class in each block of 64 tiles */
     size_t bin_visible;   /* u32[slices]     visible Gaussians per slice */
     size_t tile_lists;    /* u32[8+4*tiles]  counts, work counters and lists of the buckets of each larger sorter size class */
     size_t total_bytes;
@@ -171,6 +176,13 @@ enum {
     GS355_STAGE_TILE_SCATTER = 512,
     GS355_STAGE_TILE_SCATTER_TWO_LEVEL = 1024, /* modifier of TILE_SCATTER: through the bins whatever the key count */
     GS355_STAGE_TILE_SCATTER_ONE_LEVEL = 2048, /* modifier of TILE_SCATTER: straight into the buckets (ignored beyond 36000 tiles) */
+    /* Modifiers of TILESORT: do not launch the sorter of the 2nd / 3rd / 4th size class (1025..2048, 2049..5120,
+     * 5121..10240 pairs per bucket).  A launch over an empty class costs 4-6 us, and most frames leave one or more
+     * classes empty (header.sort_class_count of the previous frame is a good predictor).  A hint, not a promise:
+     * buckets of a skipped class are still sorted, one workgroup each through global memory -- same result, slower. */
+    GS355_STAGE_TILESORT_SKIP_1 = 4096,
+    GS355_STAGE_TILESORT_SKIP_2 = 8192,
+    GS355_STAGE_TILESORT_SKIP_3 = 16384,
     GS355_PIPELINE_FAST = 1 | 128 | 512 | 256 | 32
 };
 

@@ -18,6 +18,7 @@ STAGE_TILE_COUNT, STAGE_TILESORT, STAGE_TILE_SCATTER = 128, 256, 512
 STAGE_TILE_SCATTER_TWO_LEVEL = 1024  # modifiers of STAGE_TILE_SCATTER: name the variant instead of letting the device
 STAGE_TILE_SCATTER_ONE_LEVEL = 2048  # choose by the key count (which launches both)
 TWO_LEVEL_MIN_KEYS = 6 << 20         # the device's own threshold
+STAGE_TILESORT_SKIP = (4096, 8192, 16384)  # modifiers of STAGE_TILESORT: do not launch that size class's sorter
 PIPELINE_FAST = STAGE_PREPROCESS | STAGE_TILE_COUNT | STAGE_TILE_SCATTER | STAGE_TILESORT | STAGE_BLEND
 MAX_FAST_TILES = 36000 * 16  # limits of the tile-bucketed stages (the classic stages have neither)
 MAX_FAST_GAUSSIANS = 1 << 28
@@ -70,7 +71,8 @@ class Header(C.Structure):
         ("num_keys", C.c_uint32),
         ("overflow", C.c_uint32),
         ("num_visible", C.c_uint32),
-        ("reserved", C.c_uint32 * 11),
+        ("sort_class_count", C.c_uint32 * 3),
+        ("reserved", C.c_uint32 * 8),
     ]
 
 

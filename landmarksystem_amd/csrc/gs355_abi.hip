@@ -27,8 +27,11 @@ namespace {
 
 constexpr size_t kAlign = 256;
 constexpr uint32_t kKnownStages = GS355_STAGE_ALL | GS355_STAGE_BLEND_PLAIN | GS355_STAGE_TILE_COUNT | GS355_STAGE_TILESORT | GS355_STAGE_TILE_SCATTER |
-                                  GS355_STAGE_TILE_SCATTER_TWO_LEVEL | GS355_STAGE_TILE_SCATTER_ONE_LEVEL;
-constexpr uint32_t kStageModifiers = GS355_STAGE_TILE_SCATTER_TWO_LEVEL | GS355_STAGE_TILE_SCATTER_ONE_LEVEL;
+                                  GS355_STAGE_TILE_SCATTER_TWO_LEVEL | GS355_STAGE_TILE_SCATTER_ONE_LEVEL |
+                                  GS355_STAGE_TILESORT_SKIP_1 | GS355_STAGE_TILESORT_SKIP_2 | GS355_STAGE_TILESORT_SKIP_3;
+constexpr uint32_t kScatterModifiers = GS355_STAGE_TILE_SCATTER_TWO_LEVEL | GS355_STAGE_TILE_SCATTER_ONE_LEVEL;
+constexpr uint32_t kStageModifiers =
+    kScatterModifiers | GS355_STAGE_TILESORT_SKIP_1 | GS355_STAGE_TILESORT_SKIP_2 | GS355_STAGE_TILESORT_SKIP_3;
 constexpr int64_t kMaxKeys = (1ll << 32) - 1 - kSortTile;  // key slots are indexed with u32
 
 size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
@@ -88,7 +91,7 @@ int make_layout(int32_t P, int64_t n_cap, int32_t W, int32_t H, gs355_layout* L)
     L->sort_hist = take(hist_words * sizeof(uint32_t));
     L->ranges = take(tiles * 2 * sizeof(uint32_t));
     L->bin_matrix = take((tiles <= (size_t)kBinMaxTilesWide ? bin_matrix_words(tiles) : 0) * sizeof(uint32_t));
-    L->tile_base = take((2 * tiles + 2 * ((tiles + 63) / 64) + (tiles + kCoarseTiles - 1) / kCoarseTiles + 1) * sizeof(uint32_t));
+    L->tile_base = take((2 * tiles + 3 * ((tiles + 63) / 64) + (tiles + kCoarseTiles - 1) / kCoarseTiles + 1) * sizeof(uint32_t));
     L->bin_visible = take((size_t)kBinMaxGroups * sizeof(uint32_t));
     L->tile_lists = take((kListHeader + 4 * tiles) * sizeof(uint32_t));
     L->total_bytes = off;
@@ -190,7 +193,7 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
 {
     int rc;
     if ((stage_mask & ~kKnownStages) != 0 || (stage_mask & ~kStageModifiers) == 0 ||
-        (stage_mask & kStageModifiers) == kStageModifiers)
+        (stage_mask & kScatterModifiers) == kScatterModifiers)
         return set_error(GS355_EINVAL, "stage_mask 0x%x selects no known stage", stage_mask);
     if ((rc = check_frame(frame, true))) return rc;
     if ((rc = check_geometry_inputs(g))) return rc;
@@ -271,7 +274,11 @@ int gs355_run(const gs355_frame* frame, const gs355_gaussians* g, void* workspac
             return rc;
     if (stage_mask & GS355_STAGE_TILESORT)
         if ((rc = launch_tile_sort(header, tiles, ranges, tile_lists, buckets, keys[L.sorted_buffer],
-                                   vals[L.sorted_buffer], s)))
+                                   vals[L.sorted_buffer],
+                                   ((stage_mask & GS355_STAGE_TILESORT_SKIP_1) ? 1u : 0u) |
+                                       ((stage_mask & GS355_STAGE_TILESORT_SKIP_2) ? 2u : 0u) |
+                                       ((stage_mask & GS355_STAGE_TILESORT_SKIP_3) ? 4u : 0u),
+                                   s)))
             return rc;
     if (stage_mask & (GS355_STAGE_BLEND | GS355_STAGE_BLEND_PLAIN))
         if ((rc = launch_blend(fa, header, ranges, vals[L.sorted_buffer], records, out->image, out->depth, out->alpha,

@@ -453,6 +453,7 @@ __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict_
                                                            uint32_t* __restrict__ totals,
                                                            uint64_t* __restrict__ block_sums,
                                                            uint32_t* __restrict__ bin_sums,
+                                                           uint32_t* __restrict__ block_classes,
                                                            uint32_t* __restrict__ list_counts)
 {
     __shared__ uint32_t s_part[4][64];
@@ -499,6 +500,13 @@ __global__ __launch_bounds__(256) void slice_prefix_kernel(uint32_t* __restrict_
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) sum64 += __shfl_down(sum64, d, 64);
         if (lane == 0) block_sums[blockIdx.x] = sum64;
+        if (block_classes) {  // columns are tiles: how many of the 64 fall in each larger sorter size class, a byte each
+            const uint32_t v = live ? total : 0u;
+            const uint32_t n1 = (uint32_t)__popcll(__ballot(v > (uint32_t)kTileSortCap[0] && v <= (uint32_t)kTileSortCap[1]));
+            const uint32_t n2 = (uint32_t)__popcll(__ballot(v > (uint32_t)kTileSortCap[1] && v <= (uint32_t)kTileSortCap[2]));
+            const uint32_t n3 = (uint32_t)__popcll(__ballot(v > (uint32_t)kTileSortCap[2] && v <= (uint32_t)kTileSortCap[3]));
+            if (lane == 0) block_classes[blockIdx.x] = n1 | (n2 << 8) | (n3 << 16);
+        }
         if (bin_sums) {  // columns are tiles: the pairs of each coarse bin (kCoarseTiles consecutive tiles)
             uint32_t bin = live ? total : 0u;
 #pragma unroll
@@ -526,11 +534,14 @@ __global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* total
                                                            gs355_header* __restrict__ header_copy, bool header_known,
                                                            uint32_t* tile_base,
                                                            uint32_t* __restrict__ ranges, uint32_t* __restrict__ lists,
-                                                           const uint32_t* bin_pairs, int bins, uint32_t* chunk_base)
+                                                           const uint32_t* bin_pairs, int bins, uint32_t* chunk_base,
+                                                           const uint32_t* __restrict__ block_classes)
 {
     __shared__ uint64_t s_before[4], s_total[4];
-    __shared__ uint32_t s_vis[4], s_chunks[4];
+    __shared__ uint32_t s_vis[4], s_chunks[4], s_class[3];
     if (header_known && header->overflow) return;
+    if (threadIdx.x < 3) s_class[threadIdx.x] = 0u;
+    __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t first_block = blockIdx.x * 4u, block = first_block + (uint32_t)wave;
     {
@@ -541,8 +552,22 @@ __global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* total
             before += b < first_block ? v : 0ull;
         }
         uint32_t vis = 0;
-        if (blockIdx.x == 0 && !header_known)
+        if (blockIdx.x == 0 && !header_known) {
             for (int c = threadIdx.x; c < groups; c += 256) vis += group_visible[c];
+            // buckets per larger sorter size class, for the header (counted per block by the slice prefix)
+            if (block_classes) {
+                uint32_t n1 = 0, n2 = 0, n3 = 0;
+                for (uint32_t b = threadIdx.x; b < n_blocks; b += 256u) {
+                    const uint32_t w = block_classes[b];
+                    n1 += w & 0xFFu;
+                    n2 += (w >> 8) & 0xFFu;
+                    n3 += (w >> 16) & 0xFFu;
+                }
+                if (n1) atomicAdd(&s_class[0], n1);
+                if (n2) atomicAdd(&s_class[1], n2);
+                if (n3) atomicAdd(&s_class[2], n3);
+            }
+        }
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) {
             before += __shfl_down(before, d, 64);
@@ -563,11 +588,14 @@ __global__ __launch_bounds__(256) void tile_publish_kernel(const uint32_t* total
         header->num_keys = overflow ? n_cap : (uint32_t)total;
         header->overflow = overflow ? 1u : 0u;
         header->num_visible = (s_vis[0] + s_vis[1]) + (s_vis[2] + s_vis[3]);
+        const bool counted = block_classes != nullptr;
+        for (int c = 0; c < 3; ++c) header->sort_class_count[c] = counted ? s_class[c] : 0xFFFFFFFFu;
         if (header_copy) {  // (may be host memory: plain stores, complete when the kernel is)
             header_copy->num_keys_total = total;
             header_copy->num_keys = overflow ? n_cap : (uint32_t)total;
             header_copy->overflow = overflow ? 1u : 0u;
             header_copy->num_visible = (s_vis[0] + s_vis[1]) + (s_vis[2] + s_vis[3]);
+            for (int c = 0; c < 3; ++c) header_copy->sort_class_count[c] = counted ? s_class[c] : 0xFFFFFFFFu;
         }
     }
     if (overflow) return;  // later stages do nothing either
@@ -1148,13 +1176,16 @@ struct LdsSorter {
 // Smallest size class: one workgroup per tile; tiles with larger buckets leave at once, except those beyond the
 // capacity of the largest LDS sorter, which are sorted here by radix passes through global memory, ping-ponging
 // between the bucket and the tile's slice of the output keys (their scratch lies over the LDS sorter's area).
+// `skip_classes` (bit c: the sorter of larger class c is not launched for this frame, the caller expecting no bucket
+// of that size): such a bucket, should there be one after all, takes the global-memory route too, so every bucket is
+// sorted whatever the caller expected.
 template <int kT, int kR>
 __global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* __restrict__ header,
                                                             const uint32_t* __restrict__ ranges,
                                                             uint64_t* __restrict__ buckets,
                                                             uint64_t* __restrict__ out_keys,
                                                             uint32_t* __restrict__ out_vals,
-                                                            uint32_t* __restrict__ list_work)
+                                                            uint32_t* __restrict__ list_work, uint32_t skip_classes)
 {
     extern __shared__ uint32_t s_dyn[];
     if (blockIdx.x == 0 && threadIdx.x < 4) list_work[threadIdx.x] = 0u;  // for the list kernels launched after this one
@@ -1163,7 +1194,12 @@ __global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* 
     static_assert((256 + kWaves * 256 + 8) * sizeof(uint32_t) <= LdsSorter<kT, kR>::kBytes, "scratch of the global passes");
     const uint32_t tile = blockIdx.x;
     const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
-    if (n > (uint32_t)kTileSortCap[3]) {  // (uniform over the workgroup)
+    bool through_global = n > (uint32_t)kTileSortCap[3];
+    if (skip_classes != 0u && n > (uint32_t)kTileSortCap[0] && !through_global) {
+        const int cls = n <= (uint32_t)kTileSortCap[1] ? 0 : n <= (uint32_t)kTileSortCap[2] ? 1 : 2;
+        through_global = (skip_classes >> cls) & 1u;
+    }
+    if (through_global) {  // (uniform over the workgroup)
         const SortScratch sc = {s_dyn, reinterpret_cast<uint32_t(*)[256]>(s_dyn + 256), s_dyn + 256 + kWaves * 256};
         const GlobalPairs A = {buckets + lo}, B = {out_keys + lo};
         const bool in_b = sort_pairs(A, B, n, sc);
@@ -1304,12 +1340,12 @@ template <bool kTiles>
 static int launch_layout(const uint32_t* totals, uint32_t* bases, int columns, const uint64_t* blocks,
                          const uint32_t* group_visible, int groups, uint32_t n_cap, gs355_header* header,
                          gs355_header* header_copy, bool header_known, uint32_t* ranges, uint32_t* lists, const uint32_t* bin_pairs, int bins,
-                         uint32_t* chunk_base, hipStream_t s)
+                         uint32_t* chunk_base, const uint32_t* block_classes, hipStream_t s)
 {
     const int n_blocks = (columns + 63) / 64;
     hipLaunchKernelGGL(tile_publish_kernel<kTiles>, dim3((n_blocks + 3) / 4), dim3(256), 0, s, totals, (uint32_t)columns,
                        blocks, (uint32_t)n_blocks, group_visible, groups, n_cap, header, header_copy, header_known, bases, ranges, lists,
-                       bin_pairs, bins, chunk_base);
+                       bin_pairs, bins, chunk_base, block_classes);
     GS355_CHECK_LAUNCH("bin: layout");
     return GS355_OK;
 }
@@ -1325,22 +1361,23 @@ int launch_tile_layout(int32_t P, uint32_t* matrix, const uint32_t* group_visibl
     uint64_t* blocks = reinterpret_cast<uint64_t*>(tile_base + 2 * (size_t)tiles);
     const int bins = coarse_bins(tiles);
     uint32_t* chunk_base = chunk_bases(tile_base, tiles);
+    uint32_t* block_classes = chunk_base + bins + 1;  // [ceil(tiles / 64)]
     if (tiles <= kBinMaxTiles) {
         // (the pairs of each coarse bin go to chunk_base, which the block scan turns into chunk bases in place)
         hipLaunchKernelGGL(slice_prefix_kernel, dim3((tiles + 63) / 64), dim3(256), 0, s, matrix, groups, tiles,
-                           tile_base, blocks, chunk_base, lists);
+                           tile_base, blocks, chunk_base, block_classes, lists);
         GS355_CHECK_LAUNCH("bin: slice prefix");
         return launch_layout<true>(tile_base, tile_base, tiles, blocks, group_visible, groups, n_cap, header, header_copy, false, ranges,
-                                   lists, chunk_base, bins, chunk_base, s);
+                                   lists, chunk_base, bins, chunk_base, block_classes, s);
     }
     // (both in the cursor half of tile_base, which the tile-level layout of launch_tile_scatter overwrites later)
     uint32_t* bin_base = tile_base + tiles;
     uint32_t* bin_pairs = bin_base + bins;
     hipLaunchKernelGGL(slice_prefix_kernel, dim3((bins + 63) / 64), dim3(256), 0, s, matrix, groups, bins, bin_pairs,
-                       blocks, (uint32_t*)nullptr, lists);
+                       blocks, (uint32_t*)nullptr, (uint32_t*)nullptr, lists);
     GS355_CHECK_LAUNCH("bin: slice prefix");
     return launch_layout<false>(bin_pairs, bin_base, bins, blocks, group_visible, groups, n_cap, header, header_copy, false, ranges,
-                                lists, bin_pairs, bins, chunk_base, s);
+                                lists, bin_pairs, bins, chunk_base, nullptr, s);
 }
 
 int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, const uint32_t* depth_bits,
@@ -1382,7 +1419,7 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
                            chunk_bases(tile_base, T), coarse, tile_base, blocks, lists);
         GS355_CHECK_LAUNCH("bin: fine count");
         if ((rc = launch_layout<true>(tile_base, tile_base, T, blocks, group_visible, groups, n_cap, header, nullptr, true, ranges,
-                                      lists, (const uint32_t*)nullptr, 0, (uint32_t*)nullptr, s)))
+                                      lists, (const uint32_t*)nullptr, 0, (uint32_t*)nullptr, nullptr, s)))
             return rc;
     }
     if (fine) {
@@ -1394,7 +1431,7 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
 }
 
 int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, uint32_t* lists, uint64_t* buckets,
-                     uint64_t* out_keys, uint32_t* out_vals, hipStream_t s)
+                     uint64_t* out_keys, uint32_t* out_vals, uint32_t skip_classes, hipStream_t s)
 {
     using S0 = LdsSorter<256, 4>;    // <= 1024 pairs, one workgroup per tile
     using S1 = LdsSorter<512, 4>;    // <= 2048
@@ -1407,18 +1444,25 @@ int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* rang
     const uint32_t* list0 = lists + kListHeader;
     uint32_t* work = lists + 4;  // next untaken entry of each class list
     hipLaunchKernelGGL((tile_sort_each_kernel<256, 4>), dim3(tiles), dim3(256), S0::kBytes, s, header, ranges, buckets,
-                       out_keys, out_vals, work);
+                       out_keys, out_vals, work, skip_classes);
     GS355_CHECK_LAUNCH("tile sort: class 0");
     auto grid = [&](int want) { return dim3(tiles < want ? tiles : want); };
-    hipLaunchKernelGGL((tile_sort_list_kernel<512, 4>), grid(1024), dim3(512), S1::kBytes, s, header, ranges, list0,
-                       lists + 0, work + 0, buckets, out_keys, out_vals);
-    GS355_CHECK_LAUNCH("tile sort: class 1");
-    hipLaunchKernelGGL(tile_sort_list_1024x5_kernel, grid(512), dim3(1024), S2::kBytes, s, header, ranges,
-                       list0 + (size_t)tiles, lists + 1, work + 1, buckets, out_keys, out_vals);
-    GS355_CHECK_LAUNCH("tile sort: class 2");
-    hipLaunchKernelGGL((tile_sort_list_kernel<1024, 10>), grid(256), dim3(1024), S3::kBytes, s, header, ranges,
-                       list0 + 2 * (size_t)tiles, lists + 2, work + 2, buckets, out_keys, out_vals);
-    GS355_CHECK_LAUNCH("tile sort: class 3");
+    // (skip_classes: bit c set = the caller expects list c to be empty; the kernel above has sorted what is on it)
+    if (!(skip_classes & 1u)) {
+        hipLaunchKernelGGL((tile_sort_list_kernel<512, 4>), grid(1024), dim3(512), S1::kBytes, s, header, ranges, list0,
+                           lists + 0, work + 0, buckets, out_keys, out_vals);
+        GS355_CHECK_LAUNCH("tile sort: class 1");
+    }
+    if (!(skip_classes & 2u)) {
+        hipLaunchKernelGGL(tile_sort_list_1024x5_kernel, grid(512), dim3(1024), S2::kBytes, s, header, ranges,
+                           list0 + (size_t)tiles, lists + 1, work + 1, buckets, out_keys, out_vals);
+        GS355_CHECK_LAUNCH("tile sort: class 2");
+    }
+    if (!(skip_classes & 4u)) {
+        hipLaunchKernelGGL((tile_sort_list_kernel<1024, 10>), grid(256), dim3(1024), S3::kBytes, s, header, ranges,
+                           list0 + 2 * (size_t)tiles, lists + 2, work + 2, buckets, out_keys, out_vals);
+        GS355_CHECK_LAUNCH("tile sort: class 3");
+    }
     return GS355_OK;
 }
 

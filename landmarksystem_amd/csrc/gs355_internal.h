@@ -149,7 +149,7 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
 // lists: u32[kListHeader + 4 * tiles]: the four class counts, the class lists' work counters, the four lists
 constexpr int kListHeader = 8;
 int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, uint32_t* lists,
-                     uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, hipStream_t s);
+                     uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, uint32_t skip_classes, hipStream_t s);
 
 // generic exclusive scan of u32 (n <= 2^32-1); tmp needs scan_tmp_words(n) words
 size_t scan_tmp_words(size_t n);

@@ -128,11 +128,14 @@ __global__ __launch_bounds__(256) void scan_sums_kernel(uint64_t* __restrict__ s
             header->num_keys = total > n_cap ? n_cap : (uint32_t)total;
             header->overflow = total > n_cap ? 1u : 0u;
             header->num_visible = s_vis[0] + s_vis[1] + s_vis[2] + s_vis[3];
+            header->sort_class_count[0] = header->sort_class_count[1] = header->sort_class_count[2] = 0xFFFFFFFFu;
             if (header_copy) {  // (may be host memory: plain stores, complete when the kernel is)
                 header_copy->num_keys_total = total;
                 header_copy->num_keys = total > n_cap ? n_cap : (uint32_t)total;
                 header_copy->overflow = total > n_cap ? 1u : 0u;
                 header_copy->num_visible = s_vis[0] + s_vis[1] + s_vis[2] + s_vis[3];
+                header_copy->sort_class_count[0] = header_copy->sort_class_count[1] = header_copy->sort_class_count[2] =
+                    0xFFFFFFFFu;
             }
         }
     }

@@ -54,7 +54,10 @@ class Workspace:
         self.header_event = torch.cuda.Event()
         self.frames = 0
         self.overflows = 0
+        self.sort_mispredictions = 0  # frames with buckets in a sorter size class that was expected empty
         self.last_num_keys = 0  # of the latest frame rendered over this workspace
+        self.sort_class_idle = [0, 0, 0]  # consecutive frames that left each larger sorter size class empty
+        self.sort_class_wait = [4, 4, 4]  # ... and how many of them it takes before the class's launch is left out
 
     def ensure(self, P: int, n_cap: int, width: int, height: int) -> "_lib.Layout":
         layout = _lib.workspace_layout(P, n_cap, width, height)
@@ -283,9 +286,16 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
         # the scatter variant that suited the previous frame of this workspace (either is correct for any frame)
         back |= (_lib.STAGE_TILE_SCATTER_TWO_LEVEL if ws.last_num_keys >= _lib.TWO_LEVEL_MIN_KEYS
                  else _lib.STAGE_TILE_SCATTER_ONE_LEVEL)
+        # no launch for a sorter size class that the last few frames left empty (a hint: the library sorts the
+        # buckets of such a class all the same, but far slower than the launch costs, so a class that turns up
+        # unexpectedly has to stay away four times as long before it is left out again)
+        skipped = [c for c in range(3) if ws.sort_class_idle[c] >= ws.sort_class_wait[c]]
+        for c in skipped:
+            back |= _lib.STAGE_TILESORT_SKIP[c]
     else:  # beyond the bucketed stages' limits (images past 8K): classic duplicate / radix sort / ranges
         front = _lib.STAGE_PREPROCESS | _lib.STAGE_SCAN
         back = _lib.STAGE_DUPLICATE | _lib.STAGE_SORT | _lib.STAGE_RANGES | _lib.STAGE_BLEND
+        skipped = []
     for attempt in range(3):
         n_cap = ws.key_capacity
         # the stage that produces the header also stores it in pinned host memory (no copy is enqueued)
@@ -301,10 +311,22 @@ def render(inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True
         out.num_keys = ws.last_num_keys = total
         out.num_visible = int(ws.header_host[2]) & 0xFFFFFFFF
         ws.frames += 1
+        word3 = int(ws.header_host[3])
+        counts = ((int(ws.header_host[2]) >> 32) & 0xFFFFFFFF, word3 & 0xFFFFFFFF, (word3 >> 32) & 0xFFFFFFFF)
+        for c in range(3):  # (0xFFFFFFFF: this path does not count the classes)
+            ws.sort_class_idle[c] = ws.sort_class_idle[c] + 1 if counts[c] == 0 else 0
+        wrong = [c for c in skipped if counts[c] != 0]
+        if wrong and not overflow:
+            ws.sort_mispredictions += 1  # (the frame is right all the same: the library sorts such buckets the slow way)
+            for c in wrong:
+                ws.sort_class_wait[c] = min(4 * ws.sort_class_wait[c], 4096)
         if not overflow:
             out.key_capacity = n_cap
             return out
         ws.overflows += 1
+        for c in [c for c in skipped if counts[c] != 0]:
+            back &= ~_lib.STAGE_TILESORT_SKIP[c]
+            skipped.remove(c)
         ws.key_capacity = int(total * _KEY_HEADROOM) + 4096
     raise RuntimeError("key capacity still insufficient after regrowing (needed %d keys)" % out.num_keys)
 

@@ -119,7 +119,8 @@ def test_run_validates_before_any_hip_call():
     assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 1024)  # a modifier alone
     assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 2048)
     assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, _lib.PIPELINE_FAST | 1024 | 2048)
-    assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 4096)
+    assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, sum(_lib.STAGE_TILESORT_SKIP))
+    assert "stage_mask" in _err(_lib.GS355_EINVAL, run, f, g, 0x1000, 1 << 30, 100, out, 32768)  # no such stage
     assert "SHs or precomputed colors" in _err(_lib.GS355_EINVAL, run, f, _gauss(shs=True, colors=True), 0x1000,
                                                 1 << 30, 100, out, _lib.STAGE_ALL)
     assert "SHs or precomputed colors" in _err(_lib.GS355_EINVAL, run, f, _gauss(shs=False, colors=False), 0x1000,

@@ -192,6 +192,40 @@ def test_key_capacity_overflow_is_reported_and_recovered(gpu_device):
                  ref, "overflow redo")
 
 
+def test_sorter_launches_left_out_and_made_up_for(gpu_device):
+    """render() leaves out the launch of a sorter size class that the workspace's last few frames left empty; a frame
+    that then has buckets of that class has them sorted by the fallback inside the first sorter kernel, and gives the
+    same bits as on a fresh workspace."""
+    def inputs_of(scene):
+        s = settings_for(scene, gpu_device)
+        return pipeline.FrameInputs(s, scene.means3D.to(gpu_device), opacities=scene.opacities.to(gpu_device),
+                                    shs=scene.shs.to(gpu_device), scales=scene.scales.to(gpu_device),
+                                    rotations=scene.rotations.to(gpu_device))
+    sparse = inputs_of(scenes.tiny_scene(P=300, width=64, height=64, sh_degree=0, seed=3))
+    ws = pipeline.Workspace(gpu_device)
+    first = pipeline.render(sparse, ws=ws)
+    for _ in range(3):
+        pipeline.render(sparse, ws=ws)
+    assert ws.sort_class_idle == [4, 4, 4] == ws.sort_class_wait and ws.sort_mispredictions == 0
+    fifth = pipeline.render(sparse, ws=ws)  # all three larger sorters left out
+    assert ws.sort_mispredictions == 0
+    for a, b in ((first.image, fifth.image), (first.depth, fifth.depth), (first.alpha, fifth.alpha)):
+        assert torch.equal(a, b)
+    for n_redo, (P, side, used) in enumerate([(1500, 64, 0), (5000, 64, 1), (8000, 32, 2)], 1):
+        # (the fullest tiles of these crowded scenes fall in the 2nd, 3rd and 4th size class)
+        crowded = inputs_of(crowded_scene(P, width=side, height=side, duplicates=100))
+        ws.sort_class_idle = [5000, 5000, 5000]
+        got = pipeline.render(crowded, ws=ws)
+        want = pipeline.render(crowded, ws=pipeline.Workspace(gpu_device))
+        assert ws.sort_mispredictions == n_redo, (P, ws.sort_mispredictions)
+        assert ws.sort_class_idle[used] == 0 and ws.sort_class_wait[used] == 16, (ws.sort_class_idle, ws.sort_class_wait)
+        assert got.num_keys == want.num_keys
+        for a, b in ((got.image, want.image), (got.depth, want.depth), (got.alpha, want.alpha)):
+            assert torch.equal(a, b), P
+        again = pipeline.render(crowded, ws=ws)  # the class now counts as used: its sorter is launched
+        assert ws.sort_mispredictions == n_redo and torch.equal(again.image, want.image)
+
+
 def test_rerun_is_bit_identical(gpu_device):
     scene = scenes.config2(P=50_000)
     a = run_all_stages(scene, gpu_device)
@@ -228,7 +262,7 @@ def test_block_culling_is_result_neutral(gpu_device, make):
     assert float(out.alpha.max()) > 0.5
 
 
-def run_fast_path(scene, device, two_level=False):
+def run_fast_path(scene, device, two_level=False, modifiers=0):
     """PREPROCESS | TILE_COUNT | TILE_SCATTER | TILESORT | BLEND over an exactly sized workspace (`two_level`: the
     scatter through coarse bins, which frames of few pairs otherwise skip)."""
     s = settings_for(scene, device)
@@ -241,9 +275,12 @@ def run_fast_path(scene, device, two_level=False):
     lay = pipeline.run_stages(inp, out, ws, 0, _lib.STAGE_PREPROCESS | _lib.STAGE_TILE_COUNT)
     torch.cuda.synchronize()
     n = int(ws.view(lay, "header", P, 0, tiles)[0].item())
-    lay = pipeline.run_stages(inp, out, ws, n, _lib.PIPELINE_FAST | (_lib.STAGE_TILE_SCATTER_TWO_LEVEL if two_level else 0))
+    lay = pipeline.run_stages(inp, out, ws, n, _lib.PIPELINE_FAST | modifiers |
+                              (_lib.STAGE_TILE_SCATTER_TWO_LEVEL if two_level else 0))
     torch.cuda.synchronize()
-    return dict(sorted_keys=u64(ws.view(lay, "sorted_keys", P, n, tiles)),
+    words = [int(w) for w in ws.view(lay, "header", P, n, tiles)[:4].tolist()]
+    return dict(class_counts=[(words[2] >> 32) & 0xFFFFFFFF, words[3] & 0xFFFFFFFF, (words[3] >> 32) & 0xFFFFFFFF],
+                sorted_keys=u64(ws.view(lay, "sorted_keys", P, n, tiles)),
                 sorted_values=u32(ws.view(lay, "sorted_values", P, n, tiles)),
                 ranges=u32(ws.view(lay, "ranges", P, n, tiles)), image=out.image.cpu().numpy(),
                 depth=out.depth.cpu().numpy()[0], alpha=out.alpha.cpu().numpy()[0], num_keys=n,
@@ -286,8 +323,17 @@ def test_tile_bucketed_path_equals_oracle(gpu_device, make, label):
     two = run_fast_path(scene, gpu_device, two_level=True)
     for name in ("ranges", "sorted_keys", "sorted_values", "image", "depth", "alpha"):
         np.testing.assert_array_equal(two[name], got[name], err_msg=label + " two-level " + name)
+    # without the launches of the larger sorters (a caller's hint that their classes are empty), whatever the
+    # buckets' sizes really are: the same arrays again
+    hinted = run_fast_path(scene, gpu_device, modifiers=sum(_lib.STAGE_TILESORT_SKIP))
+    for name in ("ranges", "sorted_keys", "sorted_values", "image", "depth", "alpha"):
+        np.testing.assert_array_equal(hinted[name], got[name], err_msg=label + " larger sorters skipped: " + name)
     # the crowded scenes are made of faint Gaussians (opacity 0.004 .. 0.024 around the 1/255 threshold)
     check_images(got, ref, label, max_fragile_frac=0.5 if "ties" in label else 0.02)
+    # the header's count of buckets per larger sorter size class (what lets a caller leave a sorter's launch out)
+    lens = (ref["ranges"][:, 1].astype(np.int64) - ref["ranges"][:, 0])
+    assert got["class_counts"] == [int(((lens > lo) & (lens <= hi)).sum())
+                                   for lo, hi in ((1024, 2048), (2048, 5120), (5120, 10240))], label
     if "ties" in label:
         k = got["sorted_keys"]
         assert (k[1:] == k[:-1]).any()

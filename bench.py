@@ -45,6 +45,7 @@ COUNTER_TRAFFIC = {
     # profiles/bench_c3_6M_1080p_valu_counters.txt
     "blend_issued_flops": 10.86e9,
     "blend_issued_flops_source": "profiles/bench_c3_6M_1080p_valu_counters.txt",
+    "blend_valu_busy": 1.05,
 }
 
 # Same for `--config 5`: HBM bytes per launch of the two decode kernels (count + emit)
@@ -75,6 +76,9 @@ def parse_args():
     ap.add_argument("--spatial-order", action="store_true",
                     help="store the scene along a Morton curve first (the checkpoint loaders' spatial_order option); "
                          "same Gaussians, coherent memory traffic; not the headline workload")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="default workload only: leave out the compact lines of configs[1], [3] and [4] "
+                         "(`other_configs`), e.g. for a profiler run")
     ap.add_argument("--two-in-flight", action="store_true",
                     help="also time the frames with two in flight on alternating streams (reported beside `value`)")
     return ap.parse_args()
@@ -228,15 +232,28 @@ def raster_report(stage_ms, stats, P, tiles, npix, colour_bytes, pairs, counters
                       if traffic else None)
     if dominant == "blend":
         kind = "algorithmic" if pairs else "upper"
-        roofline = {"bound": "valu", "kernel": "blend_kernel", "achieved": blend["TFLOPs_" + kind],
-                    "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": blend["frac_fp32_" + kind], "traffic": traffic,
-                    "traffic_source": traffic_source,
-                    "note": "FP32 vector-ALU kernel (no matrix cores); peak is the MI355X fp32 vector figure (packed FMA; "
-                            "this build issues unpacked fp32, half of it).  flops = 25 x the (pixel, Gaussian) pairs the "
-                            "per-pixel loop evaluates" + (
-                                ", counted by the C checker in this run; the kernel skips pairs whose alpha is provably "
-                                "< 1/255, so it issues fewer flops than that" if pairs else
-                                ", bounded above by 256 x the sum of the tile range lengths")}
+        work_rate = {"TFLOPs": blend["TFLOPs_" + kind], "of_peak": blend["frac_fp32_" + kind],
+                     "definition": "25 flop x the (pixel, Gaussian) pairs of the reference's per-pixel loop" + (
+                         " (counted by the C checker in this run)" if pairs else
+                         " (upper bound: 256 x the sum of the tile range lengths)") +
+                     " / kernel time: a rate of useful work, NOT a utilisation -- the kernel skips pairs whose alpha is "
+                     "provably < 1/255 without evaluating them, so this exceeds 1 on sparse frames"}
+        if counters:
+            roofline = {"bound": "valu", "kernel": "blend_kernel", "achieved": blend["TFLOPs_issued"],
+                        "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": blend["frac_fp32_issued"],
+                        "frac_of_unpacked_fp32_peak": round(blend["TFLOPs_issued"] / (FP32_PEAK_TFLOPS / 2), 4),
+                        "valu_busy": counters.get("blend_valu_busy"), "traffic": traffic, "traffic_source": traffic_source,
+                        "issued_flops_source": counters["blend_issued_flops_source"], "work_rate": work_rate,
+                        "note": "achieved = fp32 flops the kernel ISSUED per launch (wavefront FMA / MUL / ADD instructions x "
+                                "64 lanes, FMA = 2; hardware counters of an earlier run of this workload, named above) / the "
+                                "launch time measured in this run.  peak = MI355X fp32 vector peak with packed FMA (157.3); "
+                                "this build issues unpacked fp32 only (packed fp32 is disabled on this pool), whose peak is "
+                                "78.6.  valu_busy = share of cycles the vector ALUs were issuing (same counter run): the "
+                                "kernel is bound by instruction issue, most of it compares, selects and address arithmetic"}
+        else:
+            roofline = {"bound": "valu", "kernel": "blend_kernel", "achieved": None, "peak": FP32_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": None, "traffic": None, "work_rate": work_rate,
+                        "note": "issued flops need hardware counters, which exist for the default workload only"}
     else:
         roofline = {"bound": "hbm", "kernel": dominant + "_kernel", "achieved": stages[dominant]["GBps"],
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": stages[dominant]["frac_hbm"], "traffic": traffic,
@@ -277,9 +294,10 @@ def backward_report(torch, pipeline, inp, n_cap, N, V, P, sh_coeffs, ms_per_step
 # ----------------------------------------------------------------------------------------------------------------
 # CPU side (rank 0, N = 1): the checkers timed on the host cores.  Only this leg touches oracle/.
 
-def cpu_pair_stats(scene, cam=None, colors_precomp=None, sh_degree=None):
+def cpu_pair_stats(scene, cam=None, colors_precomp=None, sh_degree=None, keep_frame=False):
     """The C checker over the whole frame: the (pixel, Gaussian) pair counts that define the blend's algorithmic
-    flops, and the checker's own frame time on the host cores."""
+    flops, and the checker's own frame time on the host cores.  `keep_frame`: also return everything the checker
+    produced (radii, sorted keys and values, ranges, image, depth, alpha) under "frame", for the parity leg."""
     import numpy as np
 
     from oracle import c_oracle as co
@@ -296,10 +314,33 @@ def cpu_pair_stats(scene, cam=None, colors_precomp=None, sh_degree=None):
     g = co.Gaussians(scene.means3D.numpy(), scene.opacities.numpy(), **kw)
     threads = co.set_threads(min(os.cpu_count() or 1, 16))
     t0 = time.perf_counter()
-    out = co.render(fr, g, keep_intermediates=False)
+    out = co.render(fr, g, keep_intermediates=keep_frame)
     seconds = time.perf_counter() - t0
     return {"evaluated": out["pairs_evaluated"], "accepted": out["pairs_accepted"], "tile_work": out["tile_work"],
-            "num_keys": out["num_keys"], "seconds": seconds, "threads": threads}
+            "num_keys": out["num_keys"], "seconds": seconds, "threads": threads, "frame": out if keep_frame else None}
+
+
+def parity_leg(torch, pipeline, inp, ref):
+    """The `parity` object: one frame through the product path (pipeline.render over a workspace of its own) against
+    the frame the C checker rendered from the same inputs: radii, key count, every sorted key and value and the
+    tile ranges bit for bit; image, depth and alpha as measured errors."""
+    import numpy as np
+
+    from oracle import compare
+    ws = pipeline.Workspace(inp.device)
+    out = pipeline.render(inp, ws=ws)
+    torch.cuda.synchronize()
+    lay = ws.ensure(inp.P, out.key_capacity, inp.width, inp.height)
+    n = out.num_keys
+    take = lambda name, kind: ws.view(lay, name, inp.P, n, inp.tiles).cpu().numpy().view(kind)  # noqa: E731
+    exact = {"radii": bool(np.array_equal(out.radii.cpu().numpy(), ref["radii"])),
+             "num_keys": bool(n == ref["num_keys"])}
+    if n == ref["num_keys"]:
+        exact["sorted_keys"] = bool(np.array_equal(take("sorted_keys", np.uint64), ref["sorted_keys"]))
+        exact["sorted_values"] = bool(np.array_equal(take("sorted_values", np.uint32), ref["sorted_values"]))
+        exact["tile_ranges"] = bool(np.array_equal(take("ranges", np.uint32), ref["ranges"]))
+    got = dict(image=out.image.cpu().numpy(), depth=out.depth.cpu().numpy(), alpha=out.alpha.cpu().numpy())
+    return compare.parity_object(got, ref, exact)
 
 
 def cpu_baseline(scene, pairs, colors_precomp=None, extra_seconds=0.0, extra_note=""):
@@ -367,7 +408,7 @@ def base_line(metric, fps, ms_per_step, args, warmup, dtype, config):
 
 
 def bench_vanilla(args, torch, dev):
-    """configs[0..2]: one camera, the vanilla rasterizer call of the reference's model."""
+    """configs[0..2]: one camera, the vanilla rasterizer call of the reference's model.  Returns the bench line."""
     from landmarksystem_amd import GaussianRasterizer, _lib, pipeline, scenes
 
     t0 = time.time()
@@ -385,7 +426,7 @@ def bench_vanilla(args, torch, dev):
     kwargs = dict(means3D=d.means3D, means2D=None, shs=d.shs, colors_precomp=None, opacities=d.opacities,
                   scales=d.scales, rotations=d.rotations, cov3D_precomp=None)
     fps, ms_per_step = frame_loop(torch, rast, kwargs, args.warmup, args.steps)
-    latency = synchronised_latency(torch, lambda: rast(**kwargs), min(args.steps, 60))
+    latency = None if args.compact else synchronised_latency(torch, lambda: rast(**kwargs), min(args.steps, 60))
 
     # the same frames with two in flight (alternating HIP streams, one workspace each): the next frame's
     # HBM-bound preprocess overlaps the current frame's VALU-bound blend.  Reported beside `value`, never as it.
@@ -441,10 +482,13 @@ def bench_vanilla(args, torch, dev):
     n_cap = pipeline.default_workspace(dev).key_capacity
     stage_ms, stats = stage_breakdown(torch, pipeline, _lib, inp, n_cap, args.stage_steps)
     P, V, N = scene.P, stats["num_visible"], stats["num_keys"]
-    pairs, pairs_error = (None, None) if args.no_cpu_baseline else guarded(cpu_pair_stats, scene)
+    pairs, pairs_error = (None, None) if args.no_cpu_baseline else guarded(cpu_pair_stats, scene, keep_frame=True)
     counters = COUNTER_TRAFFIC if (args.config == 3 and not args.gaussians and not args.spatial_order) else None
     stages, roofline = raster_report(stage_ms, stats, P, inp.tiles, inp.width * inp.height, 12 * scene.shs.shape[1],
                                      pairs, counters)
+    parity, parity_error = guarded(parity_leg, torch, pipeline, inp, pairs["frame"]) if pairs else (None, None)
+    if pairs:
+        pairs["frame"] = None  # (a few hundred MB of host memory)
     if pairs and pairs["num_keys"] != N:
         stages["blend"]["pairs_note"] = "the checker counted %d keys, the GPU %d" % (pairs["num_keys"], N)
     if not args.no_backward:
@@ -458,13 +502,20 @@ def bench_vanilla(args, torch, dev):
                     (args.config - 1, scene.name, P, scene.sh_degree, inp.width, inp.height),
         "visible": V, "keys": N, "tiles": inp.tiles, "scene_gen_s": round(gen_s, 1)})
     result.update({"roofline": roofline, "stages": stages, "model_forward_frames_per_s": model_fps,
-                   "two_frames_in_flight_frames_per_s": fps_two_in_flight, "synchronised_per_frame": latency})
+                   "two_frames_in_flight_frames_per_s": fps_two_in_flight, "synchronised_per_frame": latency,
+                   "steady_state_note": "the timed loop re-renders one camera, so the two per-frame hints the driver takes "
+                                        "from the previous frame of its workspace (scatter variant, empty sorter classes) "
+                                        "are always right; the 30-pose trajectory of configs[3] is the case where they "
+                                        "change from frame to frame"})
     if not args.no_cpu_baseline:
+        result["parity"] = parity if parity else {"error": parity_error or pairs_error}
+        if args.compact:
+            return result
         base, err = guarded(cpu_baseline, scene, pairs)
         result["cpu_baseline"] = base if base else {"error": err}
         if pairs_error:
             result["cpu_baseline"]["c_checker_error"] = pairs_error
-    print(json.dumps(result))
+    return result
 
 
 def bench_trajectory(args, torch, dev):
@@ -514,7 +565,7 @@ def bench_trajectory(args, torch, dev):
         result["cpu_baseline"] = base if base else {"error": err}
         if pairs_error:
             result["cpu_baseline"]["c_checker_error"] = pairs_error
-    print(json.dumps(result))
+    return result
 
 
 def bench_scaffold(args, torch, dev):
@@ -535,7 +586,7 @@ def bench_scaffold(args, torch, dev):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     fps, ms_per_step = args.steps / elapsed, elapsed * 1e3 / args.steps
-    latency = synchronised_latency(torch, lambda: model(cam), min(args.steps, 60))
+    latency = None if args.compact else synchronised_latency(torch, lambda: model(cam), min(args.steps, 60))
 
     # the same frames with the one-kernel anchor prefilter, and an Octree-GS model over the same anchors (random
     # levels 0..4) with the reference's level-of-detail sequence and with the fused prefilter
@@ -634,11 +685,55 @@ def bench_scaffold(args, torch, dev):
         result["cpu_baseline"] = base if base else {"error": err}
         if pairs_error:
             result["cpu_baseline"]["c_checker_error"] = pairs_error
-    print(json.dumps(result))
+    return result
+
+
+def compact_entry(line):
+    """What `other_configs` keeps of another workload's bench line: frame rate, the stage times, the dominant
+    kernel with its roofline figure, and the parity object where the line has one."""
+    stages = line.get("stages", {})
+    keep = {"metric": line["metric"], "frames_per_s": line["value"], "ms_per_frame": line["ms_per_step"],
+            "steps": line["steps"], "workload": line["config"].get("workload"),
+            "stage_ms": {k: v["ms"] for k, v in stages.items() if isinstance(v, dict) and "ms" in v},
+            "dominant_kernel": line["roofline"].get("kernel"), "roofline": {
+                k: line["roofline"].get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "work_rate", "mfma_frac")
+                if line["roofline"].get(k) is not None}}
+    for name in ("preprocess", "keys_sort_ranges", "decode"):
+        if name in stages and "frac_hbm" in stages[name]:
+            keep.setdefault("frac_hbm_algorithmic", {})[name] = stages[name]["frac_hbm"]
+    for extra in ("parity", "model_variants_frames_per_s"):
+        if line.get(extra):
+            keep[extra] = line[extra]
+    for extra in ("keys_min_mean_max", "visible_fraction_min_max", "visible_anchors", "decoded_gaussians", "keys"):
+        if extra in line["config"]:
+            keep[extra] = line["config"][extra]
+    return keep
+
+
+def other_configs(args, torch, dev):
+    """Compact lines of the other single-GPU workloads BASELINE.json names, measured in the same run: configs[1]
+    (1M Gaussians, with its parity object), configs[3] (20M Gaussians at 4K over the 30-pose trajectory) and
+    configs[4] (Scaffold-GS, 500k anchors)."""
+    import copy
+    import gc
+    out = {}
+    for index, fn, steps in ((2, bench_vanilla, 200), (4, bench_trajectory, 60), (5, bench_scaffold, 200)):
+        sub = copy.copy(args)
+        sub.config, sub.gaussians, sub.spatial_order, sub.two_in_flight, sub.calibration_copy = index, None, False, False, False
+        sub.steps, sub.warmup, sub.stage_steps, sub.compact = steps, 10, 10, True
+        sub.no_model_level, sub.no_backward = index != 5, True
+        sub.no_cpu_baseline = index != 2  # the C checker renders the 1M-Gaussian frame in well under a second
+        line, err = guarded(fn, sub, torch, dev)
+        out["configs[%d]" % (index - 1)] = compact_entry(line) if line else {"error": err}
+        del line
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
 
 
 def main():
     args = parse_args()
+    args.compact = False
     if args.gpus != 1:
         print("bench.py: this build renders on one GPU; --gpus %d is not supported (run with --gpus 1)" % args.gpus,
               file=sys.stderr)
@@ -652,10 +747,17 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     if args.config == 4:
-        return bench_trajectory(args, torch, dev)
-    if args.config == 5:
-        return bench_scaffold(args, torch, dev)
-    return bench_vanilla(args, torch, dev)
+        result = bench_trajectory(args, torch, dev)
+    elif args.config == 5:
+        result = bench_scaffold(args, torch, dev)
+    else:
+        result = bench_vanilla(args, torch, dev)
+        if args.config == 3 and not args.gaussians and not args.spatial_order and not args.no_other_configs:
+            import gc
+            gc.collect()
+            torch.cuda.empty_cache()
+            result["other_configs"] = other_configs(args, torch, dev)
+    print(json.dumps(result))
 
 
 if __name__ == "__main__":

@@ -17,6 +17,8 @@
  *                   432-434, octree_gs/gs_model.py:491-493
  *   ScaffoldGS / OctreeGS.prefilter_voxel   -> gs355_anchor_filter (one pass for the models' own sequence)
  *       call sites: scaffold_gs/gs_model.py:385-436, octree_gs/gs_model.py:445-497
+ *   GaussianModel.forward's gather of the visible rows -> gs355_gather_rows
+ *       call site:  origin_gs/gs_model.py:199-208 (five boolean-index operations)
  *   autograd backward of forward(...)       -> gs355_render_backward
  *       call site:  benchmarks/nerf/origin_gs/gs_trainer.py:117-124 (loss.backward())
  *   GaussianRasterizationSettings(...)      -> gs355_frame
@@ -234,6 +236,25 @@ typedef struct gs355_anchor_lod {
 GS355_API int gs355_anchor_filter(const gs355_frame *frame, const gs355_gaussians *anchors, int32_t scale_stride,
                                   const gs355_anchor_lod *lod, uint8_t *lod_mask, uint8_t *visible, int32_t *radii,
                                   void *stream);
+
+/* The eval-mode gather of the reference's vanilla model (benchmarks/nerf/origin_gs/gs_model.py:199-208: means3D,
+ * shs, opacity, scales, rotations -- or override colours / covariances -- indexed by the prefilter's visible mask,
+ * five boolean-index operations there) as one pass: the rows of up to GS355_GATHER_MAX_ARRAYS row-major arrays
+ * whose mask byte is non-zero are copied, in order, to the front of the destination arrays (each sized for all P
+ * rows, or for the number of selected rows if the caller knows it), and the number of selected rows is stored in
+ * *count (device word, optional).  row_bytes: a multiple of 4, at most GS355_GATHER_MAX_ROW_BYTES; sources and
+ * destinations 4-byte aligned (16-byte aligned arrays of 16-byte-multiple rows are copied 16 bytes at a time).
+ * scratch: gs355_gather_scratch_bytes(P), caller-owned device memory. */
+#define GS355_GATHER_MAX_ARRAYS 8
+#define GS355_GATHER_MAX_ROW_BYTES 4096
+typedef struct gs355_gather_array {
+    const void *src; /* [P][row_bytes] */
+    void *dst;       /* [>= selected rows][row_bytes] */
+    uint32_t row_bytes;
+} gs355_gather_array;
+GS355_API int gs355_gather_scratch_bytes(int32_t P, size_t *bytes);
+GS355_API int gs355_gather_rows(int32_t P, const uint8_t *mask, int32_t n_arrays, const gs355_gather_array *arrays,
+                      uint32_t *count, void *scratch, size_t scratch_bytes, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Backward pass of GaussianRasterizer.forward: what autograd calls when the reference trains through the

@@ -9,6 +9,8 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgs355.so")
 
+ABI_VERSION = 2  # GS355_VERSION of include/gs355.h that the structures in this file mirror
+
 GS355_OK, GS355_EINVAL, GS355_ENOSPC, GS355_EOVERFLOW, GS355_EHIP = 0, -1, -2, -3, -4
 
 STAGE_PREPROCESS, STAGE_SCAN, STAGE_DUPLICATE, STAGE_SORT, STAGE_RANGES, STAGE_BLEND = 1, 2, 4, 8, 16, 32
@@ -27,7 +29,8 @@ DECODE_COUNT, DECODE_EMIT, DECODE_ALL = 1, 2, 3
 EXPORTS = ("gs355_version", "gs355_last_error", "gs355_workspace_layout", "gs355_run", "gs355_render",
            "gs355_visible_filter", "gs355_anchor_filter", "gs355_decode_scratch_bytes", "gs355_decode_count",
            "gs355_decode_count_static", "gs355_decode_emit", "gs355_decode_workspace_bytes", "gs355_decode",
-           "gs355_backward_scratch_bytes", "gs355_render_backward")
+           "gs355_backward_scratch_bytes", "gs355_render_backward", "gs355_gather_scratch_bytes", "gs355_gather_rows")
+GATHER_MAX_ARRAYS, GATHER_MAX_ROW_BYTES = 8, 4096
 
 
 class Frame(C.Structure):
@@ -44,6 +47,10 @@ class Frame(C.Structure):
         ("campos", C.c_void_p),
         ("bg", C.c_void_p),
     ]
+
+
+class GatherArray(C.Structure):
+    _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("row_bytes", C.c_uint32)]
 
 
 class Gaussians(C.Structure):
@@ -175,6 +182,9 @@ def load() -> C.CDLL:
         )
     lib = C.CDLL(LIB_PATH)
     lib.gs355_version.restype = C.c_int
+    if lib.gs355_version() != ABI_VERSION:  # (the structures below would not match the library's)
+        raise ImportError("%s has ABI version %d, this package binds version %d: rebuild it with "
+                          "`python -m landmarksystem_amd.csrc.build`" % (LIB_PATH, lib.gs355_version(), ABI_VERSION))
     lib.gs355_last_error.restype = C.c_char_p
     lib.gs355_workspace_layout.argtypes = [C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.POINTER(Layout)]
     lib.gs355_workspace_layout.restype = C.c_int
@@ -210,6 +220,11 @@ def load() -> C.CDLL:
                                           C.POINTER(BackwardInputs), C.c_void_p, C.c_size_t, C.POINTER(Gradients),
                                           C.c_void_p]
     lib.gs355_render_backward.restype = C.c_int
+    lib.gs355_gather_scratch_bytes.argtypes = [C.c_int32, C.POINTER(C.c_size_t)]
+    lib.gs355_gather_scratch_bytes.restype = C.c_int
+    lib.gs355_gather_rows.argtypes = [C.c_int32, C.c_void_p, C.c_int32, C.POINTER(GatherArray), C.c_void_p, C.c_void_p,
+                                      C.c_size_t, C.c_void_p]
+    lib.gs355_gather_rows.restype = C.c_int
     _lib = lib
     return lib
 

@@ -33,6 +33,7 @@ SOURCES = [
     ("gs355_scan.hip", []),
     ("gs355_sort.hip", []),
     ("gs355_bin.hip", []),
+    ("gs355_gather.hip", []),
     ("gs355_decode.hip", []),
     ("gs355_blend.hip", []),
     ("gs355_backward.hip", []),

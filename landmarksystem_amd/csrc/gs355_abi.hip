@@ -407,4 +407,39 @@ int gs355_anchor_filter(const gs355_frame* frame, const gs355_gaussians* anchors
     return launch_anchor_filter(fa, *anchors, x, radii, static_cast<hipStream_t>(stream));
 }
 
+int gs355_gather_scratch_bytes(int32_t P, size_t* bytes)
+{
+    if (P < 0) return set_error(GS355_EINVAL, "P must be >= 0 (got %d)", P);
+    if (!bytes) return set_error(GS355_EINVAL, "bytes is NULL");
+    *bytes = gather_scratch_words(P) * sizeof(uint32_t);
+    return GS355_OK;
+}
+
+int gs355_gather_rows(int32_t P, const uint8_t* mask, int32_t n_arrays, const gs355_gather_array* arrays,
+                      uint32_t* count, void* scratch, size_t scratch_bytes, void* stream)
+{
+    if (P < 0) return set_error(GS355_EINVAL, "P must be >= 0 (got %d)", P);
+    if (n_arrays < 0 || n_arrays > GS355_GATHER_MAX_ARRAYS)
+        return set_error(GS355_EINVAL, "n_arrays must be in [0, %d] (got %d)", GS355_GATHER_MAX_ARRAYS, n_arrays);
+    if (n_arrays > 0 && !arrays) return set_error(GS355_EINVAL, "arrays is NULL");
+    for (int k = 0; k < n_arrays; ++k) {
+        const gs355_gather_array& a = arrays[k];
+        if (a.row_bytes == 0 || (a.row_bytes & 3u) || a.row_bytes > GS355_GATHER_MAX_ROW_BYTES)
+            return set_error(GS355_EINVAL, "arrays[%d]: row_bytes must be a multiple of 4 in [4, %d] (got %u)", k,
+                             GS355_GATHER_MAX_ROW_BYTES, a.row_bytes);
+        if (P > 0 && (!a.src || !a.dst)) return set_error(GS355_EINVAL, "arrays[%d]: src / dst is NULL", k);
+        if (((uintptr_t)a.src | (uintptr_t)a.dst) & 3u)
+            return set_error(GS355_EINVAL, "arrays[%d]: src / dst must be 4-byte aligned", k);
+    }
+    if (P > 0 && !mask) return set_error(GS355_EINVAL, "mask is NULL");
+    if (P > 0 && !scratch) return set_error(GS355_EINVAL, "scratch is NULL");
+    if (((uintptr_t)scratch & 7u) || ((uintptr_t)count & 3u))
+        return set_error(GS355_EINVAL, "scratch must be 8-byte aligned, count 4-byte aligned");
+    const size_t need = gather_scratch_words(P) * sizeof(uint32_t);
+    if (P > 0 && scratch_bytes < need)
+        return set_error(GS355_ENOSPC, "gather scratch too small: %zu bytes given, %zu needed", scratch_bytes, need);
+    return launch_gather_rows(P, mask, n_arrays, arrays, count, static_cast<uint32_t*>(scratch),
+                              static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

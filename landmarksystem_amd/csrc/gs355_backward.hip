@@ -36,15 +36,6 @@ __device__ __forceinline__ uint32_t key_slot(uint32_t first, uint64_t rect, int 
     return first + (uint32_t)((tile_y - y0) * (x1 - x0) + (tile_x - x0));
 }
 
-__device__ __forceinline__ float splat_exponent(float dx, float dy, float qx, float qy, float qz)
-{
-#pragma clang fp contract(off)
-    const float t1 = (qx * dx) * dx;
-    const float t2 = (qz * dy) * dy;
-    const float t3 = (qy * dx) * dy;
-    return -0.5f * (t1 + t2) - t3;
-}
-
 template <int kCtrl>
 __device__ __forceinline__ float dpp(float v)
 {
@@ -76,11 +67,11 @@ __device__ __forceinline__ bool backward_one(float& T, float& prefix, const Pixe
                                              bool enabled, int sub, float& sum)
 {
     const float dx = a.x - pxf, dy = a.y - pyf;
-    const float power = splat_exponent(dx, dy, a.z, a.w, b.x);
+    const float power = pair_exponent(dx, dy, a.z, a.w, b.x);  // a.z, a.w, b.x = -conic_x / 2, -conic_y, -conic_z / 2
     const float raw = __builtin_amdgcn_exp2f(__builtin_fmaf(power, 1.4426950408889634f, b.y));  // opacity * exp(power)
     const float alpha = fminf(0.99f, raw);
     const bool accept = enabled && !(power > 0.0f || alpha < 1.0f / 255.0f);
-    const float test_T = T * (1.0f - alpha);
+    const float test_T = __builtin_fmaf(-alpha, T, T);  // T - alpha T, as the forward blend forms it
     const bool hit = accept && test_T >= 0.0001f;
     if (accept && !hit && T > 0.0f) T = -T;
     if (__ballot(hit) == 0ull) return false;
@@ -124,8 +115,8 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
     const float* __restrict__ g_depth, const float* __restrict__ g_alpha, const uint64_t* __restrict__ rects,
     const uint32_t* __restrict__ first_key, float* __restrict__ key_grads)
 {
-    __shared__ float4 s_a[256];  // px, py, conic_x, conic_y
-    __shared__ float4 s_b[256];  // conic_z, log2(opacity), r, g
+    __shared__ float4 s_a[256];  // px, py, -conic_x / 2, -conic_y   (rescaled as the forward blend stages them)
+    __shared__ float4 s_b[256];  // -conic_z / 2, log2(opacity), r, g
     __shared__ float4 s_c[256];  // b, depth, reach_x, reach_y
     __shared__ float s_inv_opacity[256];
     __shared__ float s_grad[256 * kGradFloats];
@@ -172,10 +163,10 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
         if (j < hi) {
             const uint32_t g = values[j];
             const float4* __restrict__ rec = reinterpret_cast<const float4*>(records + (size_t)g * kRecordFloats);
-            const float4 r1 = rec[1];
+            const float4 r0 = rec[0], r1 = rec[1];
             const float opacity = r1.y < 0.0f ? 0.0f : r1.y;  // as the forward blend: a negative opacity never blends
-            s_a[tid] = rec[0];
-            s_b[tid] = make_float4(r1.x, __builtin_amdgcn_logf(opacity), r1.z, r1.w);
+            s_a[tid] = make_float4(r0.x, r0.y, -0.5f * r0.z, -r0.w);
+            s_b[tid] = make_float4(-0.5f * r1.x, __builtin_amdgcn_logf(opacity), r1.z, r1.w);
             s_c[tid] = rec[2];
             s_inv_opacity[tid] = __builtin_amdgcn_rcpf(opacity);
             slot = key_slot(first_key[g], rects[g], tile_x, tile_y);
@@ -232,9 +223,10 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
         if (j < hi) {
             const float* __restrict__ m = s_grad + tid * kGradFloats;
             const float4 a = s_a[tid];
-            const float cz = s_b[tid].x;
+            const float hz = s_b[tid].x;
             float4* __restrict__ dst = reinterpret_cast<float4*>(key_grads + (size_t)slot * kKeyFloats);
-            dst[0] = make_float4(-(a.z * m[0] + a.w * m[1]), -(cz * m[1] + a.w * m[0]), -0.5f * m[2], -m[3]);
+            // d power / d centre = -(conic_x dx + conic_y dy, conic_z dy + conic_y dx), with conic_x = -2 a.z etc.
+            dst[0] = make_float4(2.0f * a.z * m[0] + a.w * m[1], 2.0f * hz * m[1] + a.w * m[0], -0.5f * m[2], -m[3]);
             dst[1] = make_float4(-0.5f * m[4], m[5], m[6], m[7]);
             dst[2] = make_float4(m[8], m[9], 0.f, 0.f);
         }

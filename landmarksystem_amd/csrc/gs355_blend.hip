@@ -48,16 +48,17 @@ __global__ __launch_bounds__(256) void ranges_kernel(const gs355_header* __restr
 }
 
 // One (pixel, Gaussian) pair: exponent, alpha, the three discrete tests and the
-// accumulation.  The exponent is evaluated with unfused multiplies and adds in
-// a fixed order (contraction is switched off for it), so the sign test and the
-// alpha threshold see the same value as a scalar evaluation of the formula
-//     power = -0.5 * ((qx * dx) * dx + (qz * dy) * dy) - (qy * dx) * dy .
-// The staged record carries hx = -0.5 qx, hz = -0.5 qz and ny = -qy: scaling by a
-// power of two and negation commute with rounding, so
-//     ((hx * dx) * dx + (hz * dy) * dy) + (ny * dx) * dy
-// has the same bits with two instructions fewer.  The opacity enters through its
-// base-2 logarithm: alpha = min(0.99, exp2(power * log2(e) + log2(opacity))), one
-// multiply-add and the hardware exp2.
+// accumulation.  The staged record carries hx = -conic_x / 2, ny = -conic_y and
+// hz = -conic_z / 2, so the exponent
+//     power = hx dx^2 + ny dx dy + hz dy^2
+// is two nested multiply-adds (pair_exponent: five instructions), and the
+// opacity enters through its base-2 logarithm:
+//     alpha = min(0.99, exp2(power * log2(e) + log2(opacity))),
+// one more multiply-add and the hardware exp2.  Fused multiply-adds round
+// once where the scalar formula rounds twice, so `power` agrees with a scalar
+// evaluation to the rounding of its terms, not bit for bit: a pair whose alpha
+// lies within that distance of 1/255 may be decided either way (the checker
+// counts those pairs per pixel).
 //
 // A pixel's transmittance T stays >= 1e-4 while it is live, so the sign of T
 // carries the "finished" state: T > 0 live, T <= 0 finished with |T| the final
@@ -67,28 +68,19 @@ struct PixelState {
     float T, c0, c1, c2, depth;
 };
 
-__device__ __forceinline__ float splat_exponent(float dx, float dy, float hx, float ny, float hz)
-{
-#pragma clang fp contract(off)
-    const float t1 = (hx * dx) * dx;
-    const float t2 = (hz * dy) * dy;
-    const float t3 = (ny * dx) * dy;
-    return (t1 + t2) + t3;
-}
-
 // The hardware exp2 is monotone, so exp2(t) < 1/255 exactly when t < kAlphaCut, the smallest float whose exp2 reaches
 // 1/255 (found by running v_exp_f32 over every float between -8.2 and -7.8).  The shipped blend decides on t and
 // leaves the exp2 (a quarter-rate instruction) to the pairs that pass; the verification variant decides on the
 // exponential itself, and the tests hold the two to identical images on scenes full of opacities around 1/255.
 constexpr float kAlphaCut = -7.99435329f;  // bits 0xc0ffd1be
 
-// a = px, py, hx, ny;  b = hz, log2(opacity), r, g;  c = b, depth, reach_x, reach_y
+// a = px, py, hx, ny;  b = hz, log2(opacity), r, g;  rec_c + entry = b, depth (read only by pixels that accept)
 template <bool kCutOnExponent>
 __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, const float4 a, const float4 b,
-                                          const float4 c)
+                                          const char* rec_c, uint32_t entry)
 {
     const float dx = a.x - pxf, dy = a.y - pyf;
-    const float power = splat_exponent(dx, dy, a.z, a.w, b.x);
+    const float power = pair_exponent(dx, dy, a.z, a.w, b.x);
     const float t = __builtin_fmaf(power, 1.4426950408889634f, b.y);
     float alpha;
     if (kCutOnExponent) {
@@ -98,21 +90,24 @@ __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, c
         alpha = fminf(0.99f, __builtin_amdgcn_exp2f(t));
         if (power > 0.0f || alpha < 1.0f / 255.0f) return;
     }
-    const float test_T = p.T * (1.0f - alpha);
-    if (test_T >= 0.0001f) {
-        const float w = alpha * p.T;
-        p.c0 += b.z * w;
-        p.c1 += b.w * w;
-        p.c2 += c.x * w;
-        p.depth += c.y * w;
-        p.T = test_T;
-    } else if (p.T > 0.0f) {
-        p.T = -p.T;  // this Gaussian is not applied; the pixel is finished
+    // w = alpha T is the pair's weight and T - alpha T, rounded once, the transmittance behind it
+    const float w = alpha * p.T;
+    const float test_T = __builtin_fmaf(-alpha, p.T, p.T);
+    const bool apply = test_T >= 0.0001f;
+    if (apply) {
+        const float2 cd = *reinterpret_cast<const float2*>(rec_c + entry);
+        p.c0 = __builtin_fmaf(b.z, w, p.c0);
+        p.c1 = __builtin_fmaf(b.w, w, p.c1);
+        p.c2 = __builtin_fmaf(cd.x, w, p.c2);
+        p.depth = __builtin_fmaf(cd.y, w, p.depth);
     }
+    p.T = apply ? test_T : -fabsf(p.T);  // not applied: the pixel is finished (and stays so)
 }
 
+using ListEntry = uint16_t;
 constexpr int kBatch = 256;            // records staged per round
 constexpr uint32_t kNullEntry = kBatch * 16;  // list entry of the null record (opacity 0: rejected by every pixel)
+constexpr int kListWords = kBatch + 8;  // entries per list: a batch, padded to a multiple of four, one round read ahead
 
 // kCull: each wavefront first tests the staged Gaussians (one per lane) against
 // the four 4x4 blocks of its quadrant, using the bounding box of the
@@ -121,10 +116,12 @@ constexpr uint32_t kNullEntry = kBatch * 16;  // list entry of the null record (
 // that is left out is one whose 16 pixels would all have taken the
 // `alpha < 1/255` branch, and every pixel still sees its Gaussians front to
 // back with the same arithmetic, so both variants produce identical images.
-// List entries are the byte offsets of the staged records (16 x record number);
-// the lists are padded with the null record to a common length that is a
-// multiple of four, so the walk needs no per-entry length test, reads four
-// entries at a time and checks for finished wavefronts once per four entries.
+// List entries are the byte offsets of the staged records (16 x record number)
+// in 16 bits (32-bit entries would serve as LDS addresses as they are, but the
+// larger lists cost two workgroups per CU and 20 % of the kernel's speed); the
+// lists are padded with the null record to a common length that is a multiple
+// of four, so the walk needs no per-entry length test, reads four entries at
+// a time and checks for finished wavefronts once per four entries.
 template <bool kCull>
 __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_header* __restrict__ header,
                                                     const uint32_t* __restrict__ ranges,
@@ -137,7 +134,7 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
     __shared__ float4 s_c[kBatch + 1];  // b, depth, reach_x, reach_y
     __shared__ uint32_t s_wave_done[4];
     // per wavefront and 4x4 block: byte offsets of the staged records of the Gaussians that can reach the block
-    __shared__ __align__(8) uint16_t s_list[kCull ? 4 : 1][4][kBatch + 8];
+    __shared__ __align__(8) ListEntry s_list[kCull ? 4 : 1][4][kListWords];
 
     if (header->overflow) return;
     const int tile = blockIdx.x;
@@ -165,11 +162,12 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
     const char* const rec_c = reinterpret_cast<const char*>(s_c);
     auto blend_entry = [&](uint32_t entry) {
         blend_one<kCull>(p, pxf, pyf, *reinterpret_cast<const float4*>(rec_a + entry),
-                  *reinterpret_cast<const float4*>(rec_b + entry), *reinterpret_cast<const float4*>(rec_c + entry));
+                         *reinterpret_cast<const float4*>(rec_b + entry), rec_c, entry);
     };
 
     for (uint32_t base = lo; base < hi; base += kBatch) {
-        const bool wave_done = __ballot(p.T > 0.0f) == 0ull;
+        const uint64_t live = __ballot(p.T > 0.0f);  // lanes whose pixel is still accumulating
+        const bool wave_done = live == 0ull;
         if (lane == 0) s_wave_done[wave] = wave_done ? 1u : 0u;
         const uint32_t j = base + tid;
         if (j < hi) {
@@ -203,9 +201,12 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
                     }
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
+                        // a block whose 16 pixels have all finished gets no entries (its lane group idles through
+                        // the null record while the other blocks of the wavefront are served)
+                        if (((live >> (16 * b)) & 0xFFFFull) == 0ull) continue;
                         const bool hit = ((b & 1) ? in_x1 : in_x0) && ((b >> 1) ? in_y1 : in_y0);
                         const uint64_t m = __ballot(hit);
-                        if (hit) s_list[wave][b][len[b] + (uint32_t)__popcll(m & lanes_below)] = (uint16_t)(k * 16);
+                        if (hit) s_list[wave][b][len[b] + (uint32_t)__popcll(m & lanes_below)] = (ListEntry)(k * 16);
                         len[b] += (uint32_t)__popcll(m);
                     }
                 }
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
 #pragma unroll
                 for (int b = 0; b < 4; ++b)
                     for (uint32_t at = len[b] + (uint32_t)lane; at < quads * 4u; at += 64u)
-                        s_list[wave][b][at] = (uint16_t)kNullEntry;
+                        s_list[wave][b][at] = (ListEntry)kNullEntry;
                 // a wavefront's LDS operations execute in order: its list writes precede the reads below
                 wave_lds_sync();
                 // ---- the four lane groups walk their lists side by side, four entries per round ----

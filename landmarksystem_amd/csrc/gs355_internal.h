@@ -82,6 +82,19 @@ __device__ __forceinline__ Rect tile_rect(float px, float py, int radius, int gr
     return q;
 }
 
+// Exponent of one (pixel, Gaussian) pair,  hx dx^2 + ny dx dy + hz dy^2  with hx = -conic_x / 2, ny = -conic_y,
+// hz = -conic_z / 2 and (dx, dy) = centre - pixel, as two nested multiply-adds: five instructions.  The forward
+// blend and the backward blend both call this, so the two passes see the same value and decide alike.
+__device__ __forceinline__ float pair_exponent(float dx, float dy, float hx, float ny, float hz)
+{
+#pragma clang fp contract(off)
+    const float u = hx * dx;
+    const float v = __builtin_fmaf(ny, dy, u);
+    const float w = hz * dy;
+    const float z = w * dy;
+    return __builtin_fmaf(dx, v, z);
+}
+
 // stage launchers (each returns a gs355_status)
 int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_only, float* records,
                       uint32_t* tiles_touched, uint64_t* rects, uint32_t* depth_bits, int32_t* radii, hipStream_t s);
@@ -150,6 +163,11 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
 constexpr int kListHeader = 8;
 int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, uint32_t* lists,
                      uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, uint32_t skip_classes, hipStream_t s);
+
+// row compaction by a byte mask (gs355_gather_rows); scratch: gather_scratch_words(P) words
+size_t gather_scratch_words(int32_t P);
+int launch_gather_rows(int32_t P, const uint8_t* mask, int32_t n_arrays, const gs355_gather_array* arrays,
+                       uint32_t* count_out, uint32_t* scratch, hipStream_t s);
 
 // generic exclusive scan of u32 (n <= 2^32-1); tmp needs scan_tmp_words(n) words
 size_t scan_tmp_words(size_t n);

@@ -26,6 +26,7 @@ from typing import Optional
 import torch
 from torch import nn
 
+from . import pipeline
 from .anchor_decoder import FusedAnchorDecoder
 from .rasterizer import GaussianRasterizationSettings, GaussianRasterizer
 
@@ -97,7 +98,7 @@ class GaussianModel(nn.Module):
 
     def __init__(self, xyz=None, features_dc=None, features_rest=None, scaling=None, rotation=None, opacity=None,
                  sh_degree: int = 3, white_bkgd: bool = False, act_cache: bool = False,
-                 compute_cov3D_python: bool = False, convert_SHs_python: bool = False, fuse_prefilter: bool = False,
+                 compute_cov3D_python: bool = False, convert_SHs_python: bool = False, fuse_prefilter: bool = True,
                  config=None, scene_manager=None):
         super().__init__()
         if xyz is not None and not torch.is_tensor(xyz):  # the reference's signature: (config, scene_manager)
@@ -113,8 +114,8 @@ class GaussianModel(nn.Module):
             xyz, features_dc, features_rest = e(0, 3), e(0, 1, 3), e(0, (sh_degree + 1) ** 2 - 1, 3)
             scaling, rotation, opacity = e(0, 3), e(0, 4), e(0, 1)
         self.config, self.scene_manager = config, scene_manager
-        # fuse_prefilter: render all Gaussians in one pass instead of "visibility prefilter, gather the survivors,
-        # render them".  The prefilter applies the same cull / radius / tile-rectangle tests as the rasterizer's own
+        # fuse_prefilter (default): render all Gaussians in one pass instead of "visibility prefilter, gather the
+        # survivors, render them" (False = the reference's sequence, call by call).  The prefilter applies the same cull / radius / tile-rectangle tests as the rasterizer's own
         # preprocess with the same camera, and a boolean-mask gather keeps relative order, so image, visibility_filter
         # and radii come out identical; the second per-Gaussian pass and the 236 B/Gaussian gathers disappear.
         self.fuse_prefilter = fuse_prefilter
@@ -302,10 +303,9 @@ class GaussianModel(nn.Module):
             self._radii = radii if self.training else None
             return rendered_image
         if not self.training:  # the reference renders only what its prefilter kept (origin_gs/gs_model.py:199-208)
-            mask = voxel_visible_mask.nonzero().squeeze(-1)
-            pick = lambda t: None if t is None else t[mask]  # noqa: E731
-            means3D, shs, colors_precomp, opacity = pick(means3D), pick(shs), pick(colors_precomp), pick(opacity)
-            scales, rotations, cov3D_precomp = pick(scales), pick(rotations), pick(cov3D_precomp)
+            # (five boolean-index operations there; one pass over the tensors and one wait for the row count here)
+            means3D, shs, colors_precomp, opacity, scales, rotations, cov3D_precomp = pipeline.gather_rows(
+                voxel_visible_mask, [means3D, shs, colors_precomp, opacity, scales, rotations, cov3D_precomp])
         rendered_image, radii, _ = self.renderer(
             means3D=means3D, means2D=screenspace_points, shs=shs, colors_precomp=colors_precomp, opacities=opacity,
             scales=scales, rotations=rotations, cov3D_precomp=cov3D_precomp)
@@ -322,10 +322,10 @@ class ScaffoldGS(nn.Module):
     def __init__(self, anchor=None, anchor_feat=None, offset=None, scaling=None, rotation=None, n_offsets: int = 10,
                  feat_dim: int = 32, add_opacity_dist: bool = True, add_cov_dist: bool = True,
                  add_color_dist: bool = True, white_bkgd: bool = False, act_cache: bool = False, opacity=None,
-                 config=None, scene_manager=None, fuse_prefilter: bool = False, use_feat_bank: bool = False,
+                 config=None, scene_manager=None, fuse_prefilter: bool = True, use_feat_bank: bool = False,
                  add_level: bool = False, appearance_dim: int = 0):
         super().__init__()
-        # fuse_prefilter: the anchor-level prefilter (for Octree-GS including the level-of-detail mask, its gather
+        # fuse_prefilter (default; False = the reference's sequence, call by call): the anchor-level prefilter (for Octree-GS including the level-of-detail mask, its gather
         # of the selected anchors and the scatter of the result) runs as one kernel over all anchors, and the
         # number of decoded Gaussians stays on the device: decode and rasterizer are enqueued back to back without
         # a read-back in between (`visibility_filter` reads it when asked for).  Same masks, except that an anchor

@@ -240,6 +240,38 @@ def anchor_filter(settings, anchors: torch.Tensor, scaling: torch.Tensor, rotati
     return visible, mask
 
 
+def gather_rows(mask: torch.Tensor, tensors):
+    """Rows of each tensor in `tensors` (None entries pass through) that the boolean `mask` selects, in order: what
+    `t[mask]` gives for every one of them, in one pass over all of them (gs355_gather_rows) and with one wait for the
+    number of selected rows instead of one per tensor.  Returns the list of gathered tensors."""
+    dev, P = mask.device, mask.shape[0]
+    if not mask.is_cuda or mask.dtype != torch.bool or mask.dim() != 1:
+        raise ValueError("mask must be a one-dimensional bool tensor on the GPU")
+    src = [None if t is None else _dev_f32(t, dev, "tensor") for t in tensors]
+    given = [t for t in src if t is not None]
+    if len(given) > _lib.GATHER_MAX_ARRAYS:
+        raise ValueError("at most %d tensors per call" % _lib.GATHER_MAX_ARRAYS)
+    for t in given:
+        if t.shape[0] != P:
+            raise ValueError("every tensor needs one row per mask entry (%d), got shape %s" % (P, tuple(t.shape)))
+    dst = [torch.empty_like(t) for t in given]
+    arrays = (_lib.GatherArray * max(1, len(given)))()
+    for k, (a, b) in enumerate(zip(given, dst)):
+        arrays[k].src, arrays[k].dst = a.data_ptr() if P else None, b.data_ptr() if P else None
+        arrays[k].row_bytes = 4 * (a.numel() // P if P else 1)
+    need = C.c_size_t(0)
+    lib = _lib.load()
+    _lib.check(lib.gs355_gather_scratch_bytes(P, C.byref(need)))
+    scratch = torch.empty(need.value // 8 + 1, dtype=torch.int64, device=dev)
+    count = torch.empty(1, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    _lib.check(lib.gs355_gather_rows(P, mask.contiguous().data_ptr() if P else None, len(given), arrays,
+                                     count.data_ptr(), scratch.data_ptr(), scratch.numel() * 8, stream))
+    n = int(count.item())  # the one wait: the caller's tensors are exactly sized, as after boolean indexing
+    it = iter(dst)
+    return [None if t is None else next(it)[:n] for t in src]
+
+
 class FrameOutputs:
     def __init__(self, inputs: FrameInputs, want_depth: bool = True, want_alpha: bool = True):
         dev, H, W = inputs.device, inputs.height, inputs.width

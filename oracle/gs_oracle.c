@@ -413,7 +413,11 @@ void orc_blend(const orc_frame *f, const uint32_t *ranges, const uint32_t *value
                         if (fabsf(power) <= 1e-5f * (fabsf(t1) + fabsf(t2) + fabsf(t3))) ++frag;
                         if (power > 0.f) continue;
                         float alpha = fminf(0.99f, co[3] * expf(power));
-                        if (fabsf(alpha - 1.0f / 255.0f) < 1e-4f * (1.0f / 255.0f)) ++frag;
+                        /* rounding distance of alpha: the exponential's own 1e-4, plus what the exponent can
+                         * move by when its three terms are summed in another order or with fused multiply-adds
+                         * (4 units in the last place of the sum of their magnitudes) */
+                        float slack = 1e-4f + 4.0f * 1.1920929e-7f * (fabsf(t1) + fabsf(t2) + fabsf(t3));
+                        if (fabsf(alpha - 1.0f / 255.0f) < slack * (1.0f / 255.0f)) ++frag;
                         if (alpha < 1.0f / 255.0f) continue;
                         float test_T = T * (1.f - alpha);
                         if (fabsf(test_T - 0.0001f) < 1e-4f * 0.0001f) ++frag;

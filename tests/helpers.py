@@ -44,9 +44,7 @@ def settings_for(scene, device, cam=None, sh_degree=None, scale_modifier=1.0):
     )
 
 
-def psnr(a, b):
-    mse = float(np.mean((np.asarray(a, np.float64) - np.asarray(b, np.float64)) ** 2))
-    return float("inf") if mse == 0 else -10.0 * math.log10(mse)
+from oracle.compare import DEPTH_REL, IMG_TOL, PSNR_MIN, plane_errors, psnr  # noqa: E402,F401
 
 
 def u64(t: torch.Tensor) -> np.ndarray:
@@ -57,9 +55,20 @@ def u32(t: torch.Tensor) -> np.ndarray:
     return t.cpu().numpy().view(np.uint32)
 
 
-IMG_TOL = 1e-4  # max-abs bar of image, alpha and depth
-DEPTH_REL = 4e-6  # depth sums reach hundreds of metres: their bar is max(1e-4, 4e-6 * largest depth of the frame)
-PSNR_MIN = 60.0
+# Numbers of every image comparison of the session, for the terminal summary (tests/conftest.py): label ->
+# worst values seen under that label.
+IMAGE_REPORT = {}
+
+
+def _record(label, n_fragile, n_pixels, report):
+    slot = IMAGE_REPORT.setdefault(label or "frame", {"frames": 0, "fragile": 0, "pixels": 0})
+    slot["frames"] += 1
+    slot["fragile"] = max(slot["fragile"], n_fragile)
+    slot["pixels"] = max(slot["pixels"], n_pixels)
+    for name, r in report.items():
+        w = slot.setdefault(name, {"solid": 0.0, "all": 0.0, "over_tol": 0, "psnr": float("inf"), "bar": r["bar"]})
+        w["solid"], w["all"] = max(w["solid"], r["solid"]), max(w["all"], r["all"])
+        w["over_tol"], w["psnr"], w["bar"] = max(w["over_tol"], r["over_tol"]), min(w["psnr"], r["psnr"]), r["bar"]
 
 
 def check_images(got, ref, label="", psnr_min=PSNR_MIN, want_depth=True, want_alpha=True, max_fragile_frac=0.02):
@@ -76,9 +85,9 @@ def check_images(got, ref, label="", psnr_min=PSNR_MIN, want_depth=True, want_al
       * PSNR >= 60 dB over all pixels.
     Prints the fragile-pixel count and the all-pixel max-abs errors."""
     frag = ref["fragile"].astype(np.float64)
-    solid = frag == 0
-    n_fragile = int((~solid).sum())
-    assert n_fragile <= max_fragile_frac * solid.size, "%s too many threshold-adjacent pixels: %d" % (label, n_fragile)
+    n_fragile, n_pixels, errors = plane_errors(got, ref, want_depth, want_alpha)
+    _record(label, n_fragile, n_pixels, errors)
+    assert n_fragile <= max_fragile_frac * n_pixels, "%s too many threshold-adjacent pixels: %d" % (label, n_fragile)
     vis = ref["pre"]["radii"] > 0 if "pre" in ref else None
     if vis is not None and vis.any():
         colour_max = float(np.abs(ref["pre"]["rgb"][vis]).max())
@@ -86,27 +95,17 @@ def check_images(got, ref, label="", psnr_min=PSNR_MIN, want_depth=True, want_al
     else:
         colour_max = float(max(1.0, np.abs(ref["image"]).max()))
         depth_max = float(max(1.0, np.abs(ref["depth"]).max())) if "depth" in ref else 1.0
-    # (name, got, want, max-abs bar on safe pixels, peak signal for the PSNR, largest single flipped contribution)
-    planes = [("image", np.asarray(got["image"]), ref["image"], IMG_TOL, 1.0, colour_max)]
-    if want_depth and got.get("depth") is not None:
-        peak = max(1.0, float(np.abs(ref["depth"]).max()))
-        planes.append(("depth", np.asarray(got["depth"]).reshape(ref["depth"].shape), ref["depth"],
-                       max(IMG_TOL, DEPTH_REL * peak), peak, depth_max))
-    if want_alpha and got.get("alpha") is not None:
-        planes.append(("alpha", np.asarray(got["alpha"]).reshape(ref["alpha"].shape), ref["alpha"], IMG_TOL, 1.0, 1.0))
+    flips = {"image": colour_max, "depth": depth_max, "alpha": 1.0}  # largest single flipped contribution x 255
     report = []
-    for name, g, r, bar, peak, flip in planes:
-        diff = np.abs(g.astype(np.float64) - r.astype(np.float64))
-        solid_err = float(diff[..., solid].max()) if solid.any() else 0.0
-        all_err = float(diff.max()) if diff.size else 0.0
-        report.append("%s solid %.3g all %.3g (bar %.3g)" % (name, solid_err, all_err, bar))
-        assert solid_err <= bar, "%s %s max-abs %g on safe pixels (bar %g)" % (label, name, solid_err, bar)
-        bound = bar + frag * (flip / 255.0) * 1.01
-        worst = float((diff - bound).max()) if diff.size else 0.0
+    for name, r in errors.items():
+        report.append("%s solid %.3g all %.3g (bar %.3g, %d px > 1e-4, PSNR %.1f dB)"
+                      % (name, r["solid"], r["all"], r["bar"], r["over_tol"], min(r["psnr"], 999.0)))
+        assert r["solid"] <= r["bar"], "%s %s max-abs %g on safe pixels (bar %g)" % (label, name, r["solid"], r["bar"])
+        bound = r["bar"] + frag * (flips[name] / 255.0) * 1.01
+        worst = float((r["diff"] - bound).max()) if r["diff"].size else 0.0
         assert worst <= 0.0, "%s %s exceeds the one-flip-per-decision bound by %g" % (label, name, worst)
-        p = psnr(g / peak, r / peak)
-        assert p >= psnr_min, "%s %s PSNR %g" % (label, name, p)
-    print("%s: %d threshold-adjacent pixels of %d; max-abs %s" % (label or "frame", n_fragile, solid.size,
+        assert r["psnr"] >= psnr_min, "%s %s PSNR %g" % (label, name, r["psnr"])
+    print("%s: %d threshold-adjacent pixels of %d; max-abs %s" % (label or "frame", n_fragile, n_pixels,
                                                                 "; ".join(report)), flush=True)
 
 

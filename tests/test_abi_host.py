@@ -334,6 +334,30 @@ def test_one_call_decode_validates_before_any_hip_call():
     assert _err(_lib.GS355_EINVAL, lib.gs355_decode_workspace_bytes, 10, 10, 0, None)
 
 
+def test_gather_rows_validates_before_hip():
+    lib = _lib.load()
+    need = C.c_size_t()
+    assert lib.gs355_gather_scratch_bytes(6_000_000, C.byref(need)) == 0 and 8 * 5860 <= need.value < 1 << 20
+    assert "P must be" in _err(_lib.GS355_EINVAL, lib.gs355_gather_scratch_bytes, -1, C.byref(need))
+    arrays = (_lib.GatherArray * 2)()
+    arrays[0].src, arrays[0].dst, arrays[0].row_bytes = 0x1000, 0x2000, 12
+    arrays[1].src, arrays[1].dst, arrays[1].row_bytes = 0x1000, 0x2000, 192
+    call = lambda *a: _err(_lib.GS355_EINVAL, lib.gs355_gather_rows, *a)  # noqa: E731
+    assert "n_arrays" in call(10, 0x1000, 9, arrays, None, 0x1000, 1 << 20, None)
+    assert "mask is NULL" in call(10, None, 2, arrays, None, 0x1000, 1 << 20, None)
+    assert "scratch is NULL" in call(10, 0x1000, 2, arrays, None, None, 1 << 20, None)
+    arrays[1].row_bytes = 194
+    assert "multiple of 4" in call(10, 0x1000, 2, arrays, None, 0x1000, 1 << 20, None)
+    arrays[1].row_bytes = 8192
+    assert "multiple of 4" in call(10, 0x1000, 2, arrays, None, 0x1000, 1 << 20, None)
+    arrays[1].row_bytes, arrays[1].dst = 192, None
+    assert "src / dst is NULL" in call(10, 0x1000, 2, arrays, None, 0x1000, 1 << 20, None)
+    arrays[1].dst = 0x2002
+    assert "aligned" in call(10, 0x1000, 2, arrays, None, 0x1000, 1 << 20, None)
+    arrays[1].dst = 0x2000
+    assert "too small" in _err(_lib.GS355_ENOSPC, lib.gs355_gather_rows, 10_000, 0x1000, 2, arrays, None, 0x1000, 16, None)
+
+
 def test_header_is_plain_c(tmp_path):
     """include/gs355.h must compile as C99 (the boundary carries no C++ or torch types), and a C caller's view of the
     struct sizes must match what the Python binding assumes."""

@@ -71,6 +71,8 @@ def test_quoted_issued_flops_match_the_profile_they_name():
     c = {k: int(v) for k, v in re.findall(r"(SQ_INSTS_VALU_(?:FMA|MUL|ADD)_F32)\s+(\d+)", block)}
     flops = 64 * (2 * c["SQ_INSTS_VALU_FMA_F32"] + c["SQ_INSTS_VALU_MUL_F32"] + c["SQ_INSTS_VALU_ADD_F32"])
     assert abs(table["blend_issued_flops"] - flops) <= 0.005 * flops
+    busy = float(re.search(r"VALU busy = .*? = ([\d.]+) %", block).group(1)) / 100.0
+    assert abs(table["blend_valu_busy"] - busy) <= 0.01
 
 
 def test_pair_counts_are_measured_not_typed():

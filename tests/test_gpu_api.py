@@ -103,3 +103,25 @@ def test_frames_in_flight_on_two_streams_are_independent(gpu_device):
     for k, (image, radii, depth) in enumerate(outs):
         want = alone[k % 2]
         assert torch.equal(image, want[0]) and torch.equal(radii, want[1]) and torch.equal(depth, want[2])
+
+
+@pytest.mark.parametrize("P,keep", [(0, 0.5), (1, 1.0), (777, 0.0), (5000, 0.3), (300_001, 0.88), (70_000, 1.0)])
+def test_gather_rows_equals_boolean_indexing(gpu_device, P, keep):
+    """gs355_gather_rows (the eval-mode gather of origin_gs/gs_model.py:199-208 as one pass) against torch's
+    boolean indexing, bit for bit: rows of 4, 12, 16, 24 and 192 bytes, a None entry, a strided source."""
+    from landmarksystem_amd import pipeline
+    g = torch.Generator().manual_seed(P)
+    mask = (torch.rand(P, generator=g) < keep).to(gpu_device)
+    wide = torch.randn(P, 6, generator=g).to(gpu_device)
+    tensors = [torch.randn(P, 3, generator=g).to(gpu_device), torch.randn(P, 16, 3, generator=g).to(gpu_device), None,
+               torch.randn(P, 1, generator=g).to(gpu_device), wide[:, :3], torch.randn(P, 4, generator=g).to(gpu_device),
+               wide]
+    got = pipeline.gather_rows(mask, tensors)
+    assert got[2] is None
+    for t, out in zip(tensors, got):
+        if t is not None:
+            want = t[mask]
+            assert out.shape == want.shape and out.is_contiguous()
+            assert torch.equal(out, want)
+    with pytest.raises(ValueError):
+        pipeline.gather_rows(mask, [torch.zeros(P + 1, 3, device=gpu_device)])

@@ -187,7 +187,7 @@ def test_training_step_of_the_vanilla_model(gpu_device):
     points kept for densification; one backward pass fills the parameters' gradients."""
     scene = scenes.tiny_scene(P=600, width=96, height=64, sh_degree=3, seed=23)
     model = models.GaussianModel.from_activated(scene.means3D, scene.scales, scene.rotations, scene.opacities,
-                                                scene.shs).to(gpu_device)
+                                                scene.shs, fuse_prefilter=False).to(gpu_device)
     for p in model.parameters():
         p.requires_grad_(True)
     model.train()

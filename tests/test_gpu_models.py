@@ -17,17 +17,21 @@ from tests.helpers import (check_anchor_model_frame, check_images, oracle_frame,
 pytestmark = pytest.mark.gpu
 
 
-def test_vanilla_model_forward(gpu_device):
+@pytest.mark.parametrize("fuse", [False, True], ids=["reference-sequence", "fused-prefilter"])
+def test_vanilla_model_forward(gpu_device, fuse):
+    """Both forward sequences of the vanilla model: the reference's (prefilter, gather of the visible rows, render:
+    fuse_prefilter=False) and the single pass that is the default."""
     scene = scenes.config2(P=50_000, width=640, height=360)
     model = GaussianModel.from_activated(scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs,
-                                         sh_degree=3, act_cache=True).to(gpu_device).eval()
+                                         sh_degree=3, act_cache=True, fuse_prefilter=fuse).to(gpu_device).eval()
+    assert GaussianModel(dict(sh_degree=3)).fuse_prefilter is True  # the default
     image = model(scene.camera)
     # activations round-trip (log/exp, logit/sigmoid) perturb the inputs by an ulp: feed the oracle the
     # model's own activated tensors
     act = scenes.GaussianScene("act", model.get_xyz.cpu(), model.get_scaling.cpu(), model.get_rotation.cpu(),
                                model.get_opacity.cpu(), model.get_features.cpu(), 3, scene.cameras, scene.bg)
     ref = co.render(oracle_frame(act), oracle_gaussians(act))
-    check_images(dict(image=image.cpu().numpy()), ref, "vanilla model forward")
+    check_images(dict(image=image.cpu().numpy()), ref, "vanilla model forward" + (", fused" if fuse else ""))
     vis = ref["radii"] > 0
     assert torch.equal(model.visibility_filter.cpu(), torch.from_numpy(vis))
     assert model.radii.shape[0] == int(vis.sum())  # eval mode renders the prefiltered subset
@@ -37,11 +41,14 @@ def test_vanilla_model_forward(gpu_device):
     assert torch.equal(image, again)
 
 
-@pytest.mark.parametrize("A,width,height", [(30_000, 640, 360), (500_000, 1920, 1080)])
-def test_scaffold_model_forward(gpu_device, A, width, height):
-    """Scaffold-GS forward, scaled down and at the full size of the 500k-anchor workload."""
+@pytest.mark.parametrize("A,width,height,fuse", [(30_000, 640, 360, False), (30_000, 640, 360, True),
+                                                 (500_000, 1920, 1080, False), (500_000, 1920, 1080, True)])
+def test_scaffold_model_forward(gpu_device, A, width, height, fuse):
+    """Scaffold-GS forward, scaled down and at the full size of the 500k-anchor workload, through the reference's
+    sequence of calls (fuse_prefilter=False) and through the default one-kernel prefilter."""
     scene = scenes.config5(A=A, width=width, height=height)
-    model = ScaffoldGS.from_scene(scene).to(gpu_device).eval()
+    model = ScaffoldGS.from_scene(scene, fuse_prefilter=fuse).to(gpu_device).eval()
+    assert ScaffoldGS.from_scene(scenes.config5(A=10)).fuse_prefilter is True  # the default
     cam = scene.camera
     image = model(cam)
     assert image.shape == (3, height, width)
@@ -51,7 +58,7 @@ def test_scaffold_model_forward(gpu_device, A, width, height):
                                 sh_degree=1), scene.anchor.numpy(), scales=model.get_scaling[:, :3].cpu().numpy(),
                                 rotations=model.get_rotation.cpu().numpy()) > 0
     assert torch.equal(model.voxel_visible_mask.cpu(), torch.from_numpy(vis_ref))
-    dec = check_anchor_model_frame(model, cam, image, "Scaffold-GS %d anchors" % A)
+    dec = check_anchor_model_frame(model, cam, image, "Scaffold-GS %d anchors%s" % (A, ", fused" if fuse else ""))
     assert dec["xyz"].shape[0] > A // 10
 
 
@@ -103,8 +110,8 @@ def test_octree_lod_mask_and_forward(gpu_device):
     level = torch.randint(0, 5, (20_000,), generator=g)
     common = dict(n_offsets=scene.n_offsets)
     model = OctreeGS(scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
-                     voxel_size=0.5, standard_dist=250.0, fork=2, **common)
-    scaffold = ScaffoldGS.from_scene(scene)
+                     voxel_size=0.5, standard_dist=250.0, fork=2, fuse_prefilter=False, **common)
+    scaffold = ScaffoldGS.from_scene(scene, fuse_prefilter=False)
     model.anchor_decoder.load_state_dict(scaffold.anchor_decoder.state_dict())
     model = model.to(gpu_device).eval()
     cam = scene.camera
@@ -131,7 +138,7 @@ def test_octree_lod_mask_and_forward(gpu_device):
 def test_fused_prefilter_gives_the_same_frame(gpu_device):
     scene = scenes.config3(P=200_000, width=960, height=540)
     args = (scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs)
-    plain = GaussianModel.from_activated(*args, sh_degree=3, act_cache=True).to(gpu_device).eval()
+    plain = GaussianModel.from_activated(*args, sh_degree=3, act_cache=True, fuse_prefilter=False).to(gpu_device).eval()
     fused = GaussianModel.from_activated(*args, sh_degree=3, act_cache=True, fuse_prefilter=True).to(gpu_device).eval()
     a, b = plain(scene.camera), fused(scene.camera)
     assert torch.equal(a, b)
@@ -150,9 +157,9 @@ def test_checkpoint_round_trip_renders_the_same_frame(gpu_device, tmp_path):
     from landmarksystem_amd import checkpoints as ck
     scene = scenes.config2(P=30_000, width=480, height=270)
     vanilla = GaussianModel.from_activated(scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs,
-                                           sh_degree=3).to(gpu_device).eval()
+                                           sh_degree=3, fuse_prefilter=False).to(gpu_device).eval()
     ck.save_model(vanilla, tmp_path / "v")
-    loaded = ck.load_gaussian_model(tmp_path / "v", device=gpu_device).eval()
+    loaded = ck.load_gaussian_model(tmp_path / "v", device=gpu_device, fuse_prefilter=False).eval()
     frame = loaded(scene.camera)
     assert torch.equal(vanilla(scene.camera), frame) and float(frame.max()) > 0.0
     ref = vanilla_model_reference(loaded, scene.camera)  # the loaded tensors through the oracle
@@ -217,7 +224,7 @@ def test_fused_anchor_prefilter_matches_the_reference_sequence(gpu_device, dist2
     operations, gathers and visible_filter call."""
     scene = scenes.config5(A=40_000, width=640, height=360)
     cam = scene.camera
-    plain = ScaffoldGS.from_scene(scene).to(gpu_device).eval()
+    plain = ScaffoldGS.from_scene(scene, fuse_prefilter=False).to(gpu_device).eval()
     fused = ScaffoldGS.from_scene(scene, fuse_prefilter=True).to(gpu_device).eval()
     a, b = plain(cam), fused(cam)
     assert torch.equal(plain.voxel_visible_mask, fused.voxel_visible_mask)

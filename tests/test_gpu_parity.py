@@ -433,7 +433,13 @@ def config4_scene():
     return scenes.config4()
 
 
-@pytest.mark.parametrize("pose", [0, 17])
+# poses of the 30-pose trajectory spread over its range of visible fractions (the oracle's visible filter per pose:
+# 22.2 % ... 56.3 %): the smallest (pose 14), the quartiles (20, 0 = the median, 13), the largest (17) and one
+# more on either side of the median (6: 24.6 %, 9: 52.9 %)
+C4_POSES = [14, 6, 20, 0, 13, 9, 17]
+
+
+@pytest.mark.parametrize("pose", C4_POSES)
 def test_full_size_config4_4k_frame_equals_the_oracle(gpu_device, config4_scene, pose):
     """20M Gaussians at 3840x2160 (32,400 tiles; a workspace of about 2 GB) for poses of the trajectory."""
     scene = config4_scene
@@ -578,15 +584,17 @@ def test_non_finite_and_degenerate_inputs(gpu_device):
         np.testing.assert_array_equal(fast[name], g)
 
 
-@pytest.mark.parametrize("modifier", [_lib.STAGE_TILE_SCATTER_ONE_LEVEL, _lib.STAGE_TILE_SCATTER_TWO_LEVEL, 0])
-def test_device_side_count_equals_a_shorter_input(gpu_device, modifier):
+@pytest.mark.parametrize("mask", [_lib.PIPELINE_FAST | _lib.STAGE_TILE_SCATTER_ONE_LEVEL,
+                                  _lib.PIPELINE_FAST | _lib.STAGE_TILE_SCATTER_TWO_LEVEL, _lib.PIPELINE_FAST,
+                                  _lib.STAGE_ALL], ids=["one-level", "two-level", "device-chosen", "classic"])
+def test_device_side_count_equals_a_shorter_input(gpu_device, mask):
     """gs355_gaussians.P_device: arrays sized for a capacity, the number of Gaussians in a device word.  Every stage
-    (both scatter variants) must give what the same call over the first `count` rows gives."""
+    (both scatter variants, and the classic scan / duplicate / radix sort / ranges stages, which leave offsets[] at
+    and beyond the count unwritten) must give what the same call over the first `count` rows gives."""
     scene = scenes.config2(P=120_000, width=800, height=450)
     d = scene.to(gpu_device)
     s = settings_for(scene, gpu_device)
     count = 77_777
-    mask = _lib.PIPELINE_FAST | modifier
 
     def run(n_rows, count_tensor):
         inp = pipeline.FrameInputs(s, d.means3D[:n_rows], opacities=d.opacities[:n_rows], shs=d.shs[:n_rows],
@@ -594,6 +602,8 @@ def test_device_side_count_equals_a_shorter_input(gpu_device, modifier):
         out = pipeline.FrameOutputs(inp)
         out.radii.zero_()
         ws = pipeline.Workspace(gpu_device)
+        ws.ensure(inp.P, 4_000_000, inp.width, inp.height)
+        ws.buffer.fill_(0xA5)  # whatever the stages leave unwritten beyond the count is not zero
         lay = pipeline.run_stages(inp, out, ws, 4_000_000, mask)
         torch.cuda.synchronize()
         n = int(ws.view(lay, "header", inp.P, 0, inp.tiles)[0].item())

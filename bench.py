@@ -575,7 +575,7 @@ def bench_scaffold(args, torch, dev):
 
     scene = scenes.config5(args.gaussians) if args.gaussians else scenes.config5()
     A = scene.anchor.shape[0]
-    model = ScaffoldGS.from_scene(scene, act_cache=True).to(dev).eval()  # the reference's own forward sequence
+    model = ScaffoldGS.from_scene(scene, act_cache=True).to(dev).eval()  # the model as shipped: one-kernel prefilter
     cam = scene.camera.to(dev)
     for _ in range(args.warmup):
         model(cam)
@@ -588,15 +588,16 @@ def bench_scaffold(args, torch, dev):
     fps, ms_per_step = args.steps / elapsed, elapsed * 1e3 / args.steps
     latency = None if args.compact else synchronised_latency(torch, lambda: model(cam), min(args.steps, 60))
 
-    # the same frames with the one-kernel anchor prefilter, and an Octree-GS model over the same anchors (random
-    # levels 0..4) with the reference's level-of-detail sequence and with the fused prefilter
+    # the same frames through the reference's own call sequence (fuse_prefilter=False: prefilter, decoder with the
+    # Gaussian count read back, renderer), and an Octree-GS model over the same anchors (random levels 0..4) with the
+    # reference's level-of-detail sequence and with the fused prefilter
     variants = {}
     level = torch.randint(0, 5, (A,), generator=torch.Generator().manual_seed(5))
     for name, make in () if args.no_model_level else (
-        ("scaffold_fused_prefilter", lambda: ScaffoldGS.from_scene(scene, act_cache=True, fuse_prefilter=True)),
+        ("scaffold_reference_sequence", lambda: ScaffoldGS.from_scene(scene, act_cache=True, fuse_prefilter=False)),
         ("octree_reference_sequence", lambda: OctreeGS(
             scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
-            voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True)),
+            voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True, fuse_prefilter=False)),
         ("octree_fused_prefilter", lambda: OctreeGS(
             scene.anchor, scene.anchor_feat, scene.offset, torch.log(scene.scaling), scene.rotation, level,
             voxel_size=0.5, standard_dist=250.0, n_offsets=scene.n_offsets, act_cache=True, fuse_prefilter=True)),
@@ -632,6 +633,15 @@ def bench_scaffold(args, torch, dev):
         dec_args = dict(camera_center=cam.camera_center, anchor=model.get_anchor, anchor_feat=model.get_anchor_feat,
                         offset=model.get_offset, scaling=model.get_scaling, visible_mask=vis)
         dec_ms, dec = timed(lambda: model.anchor_decoder(**dec_args))
+        # the same call with weights that fp16 cannot represent (an fp32-trained checkpoint): the decoder then carries
+        # them as hi + lo fp16 pairs (more matrix instructions, the low parts in LDS, three wavefronts per workgroup)
+        import copy
+        general = copy.deepcopy(model.anchor_decoder)
+        gen = torch.Generator().manual_seed(7)
+        for prm in general.parameters():
+            prm.mul_(1.0 + 1e-3 * torch.randn(prm.shape, generator=gen).to(dev))
+        dec32_ms, _ = timed(lambda: general(**dec_args))
+        del general
     xyz, color, opacity, scaling, rot = dec[:5]
     a_vis, G = int(vis.sum()), int(xyz.shape[0])
     flops = 13952 * a_vis
@@ -649,7 +659,7 @@ def bench_scaffold(args, torch, dev):
     stages["anchor_prefilter"] = {"ms": round(prefilter_ms, 4), "bytes": 36 * A,
                                   "GBps": round(36 * A / prefilter_ms / 1e6, 1),
                                   "frac_hbm": round(36 * A / prefilter_ms / 1e6 / HBM_PEAK_GBS, 4)}
-    stages["decode"] = {"ms": round(dec_ms, 4), "anchors_per_s": round(a_vis / dec_ms * 1e3), "flops": flops,
+    stages["decode"] = {"ms": round(dec_ms, 4), "ms_fp32_weights": round(dec32_ms, 4), "anchors_per_s": round(a_vis / dec_ms * 1e3), "flops": flops,
                         "TFLOPs": round(flops / dec_ms / 1e9, 3),
                         "frac_mfma_f16": round(flops / dec_ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 6),
                         "bytes": dec_bytes, "GBps": round(dec_bytes / dec_ms / 1e6, 1),

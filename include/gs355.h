@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define GS355_VERSION 2
+#define GS355_VERSION 3
 #define GS355_API __attribute__((visibility("default")))
 #define GS355_TILE 16 /* tile edge in pixels */
 
@@ -328,7 +328,11 @@ typedef struct gs355_decoder {
     const float *bank_b1; /* device f32[3] */
     int32_t fp32_features; /* 0: anchor features are fp16-representable (what fp16 checkpoints hold) and enter the
                               matrix cores as one fp16 operand; 1: general fp32 features, carried as hi + lo fp16
-                              pairs (two more matrix instructions per head).  Weights are rounded to fp16 either way. */
+                              pairs (two more matrix instructions per head). */
+    int32_t fp32_weights;  /* 0: every weight (w0, w1 of the three heads) is fp16-representable and enters the matrix
+                              cores as one fp16 operand; 1: general fp32 weights (what an fp32-trained state_dict.th
+                              holds), carried as hi + lo fp16 pairs like the features.  Declaring fp32 weights as
+                              fp16 rounds them to 11 significant bits (pre-activations then move by ~1e-3 relative). */
 } gs355_decoder;
 
 typedef struct gs355_anchors {

@@ -9,7 +9,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgs355.so")
 
-ABI_VERSION = 2  # GS355_VERSION of include/gs355.h that the structures in this file mirror
+ABI_VERSION = 3  # GS355_VERSION of include/gs355.h that the structures in this file mirror
 
 GS355_OK, GS355_EINVAL, GS355_ENOSPC, GS355_EOVERFLOW, GS355_EHIP = 0, -1, -2, -3, -4
 
@@ -124,6 +124,7 @@ class Decoder(C.Structure):
         ("bank_w1", C.c_void_p),
         ("bank_b1", C.c_void_p),
         ("fp32_features", C.c_int32),
+        ("fp32_weights", C.c_int32),
     ]
 
 

@@ -100,11 +100,14 @@ class FusedAnchorDecoder(nn.Module):
         keep = []
         d = _lib.Decoder()
         d.feat_dim, d.n_offsets = self.feat_dim, self.n_offsets
+        fp16_exact = True  # weights that fp16 cannot hold (fp32-trained checkpoints) go in as hi + lo fp16 pairs
         for j, mlp in enumerate((self.mlp_opacity, self.mlp_cov, self.mlp_color)):
             w0, b0, w1, b1 = (_f32c(t, device) for t in (mlp[0].weight, mlp[0].bias, mlp[2].weight, mlp[2].bias))
             keep += [w0, b0, w1, b1]
+            fp16_exact = fp16_exact and all(bool(torch.equal(w.half().float(), w)) for w in (w0, w1))
             d.in_dim[j] = w0.shape[1]
             d.w0[j], d.b0[j], d.w1[j], d.b1[j] = w0.data_ptr(), b0.data_ptr(), w1.data_ptr(), b1.data_ptr()
+        d.fp32_weights = 0 if fp16_exact else 1
         d.add_level = 1 if self.add_level else 0
         d.bank_in_dim = 0
         if self.use_feat_bank:

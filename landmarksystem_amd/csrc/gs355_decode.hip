@@ -19,10 +19,13 @@
 // as long as both operands agree, so the weights of layer 2 are simply loaded
 // in the order the accumulator registers come in.
 //
-// Precision: weights and anchor features are rounded to fp16 (exact for fp16
-// checkpoints); the four fp32-only inputs (view direction, distance) and the
-// hidden activations enter the matrix cores as hi + lo fp16 pairs, so the
-// result carries fp32-level accuracy with fp32 accumulation.
+// Precision: fp32 accumulation throughout.  Weights and anchor features that
+// fp16 holds exactly (fp16 checkpoints) enter the matrix cores as one fp16
+// operand; general fp32 weights and features, the four fp32-only inputs (view
+// direction, distance) and the hidden activations enter as hi + lo fp16
+// pairs (22 significant bits; the lo x lo products, 2^-22 of a term, are
+// left out), so the result carries fp32-level accuracy either way.  The low
+// parts of the weights live in LDS, their high parts in registers.
 //
 // Work follows the visible anchors: a wavefront takes runs of 128 consecutive
 // anchors, packs the visible ones (in order) into dense tiles of 32 and decodes
@@ -56,6 +59,7 @@ struct DecodeArgs {
     const float* campos;
     const float* level;  // per-anchor level: the fourth fp32-only input instead of the distance (add_level), or NULL
     int split_feat;      // features enter as hi + lo fp16 pairs (fp32 features that fp16 cannot represent)
+    int weights_lo;      // weights enter as hi + lo fp16 pairs (fp32 weights that fp16 cannot represent)
     const float* w0[3];
     const float* b0[3];
     const float* w1[3];
@@ -81,8 +85,9 @@ __device__ __forceinline__ half8_t to_half8(const float v[8])
 // operand: slots 0..3 hold columns ka..ka+3, slots 4..7 columns kb..kb+3 (zero outside the matrix).  Loads are
 // unconditional at clamped (in-range) positions and masked afterwards, so that none of them waits for another:
 // the fragments of a head are fetched with all loads in flight together.
+// `lo`: what the fp16 rounding of each entry left over, itself rounded to fp16.
 __device__ __forceinline__ half8_t weight_fragment(const float* __restrict__ w, int rows, int cols, int row, int ka,
-                                                   int kb, bool enable = true)
+                                                   int kb, bool enable = true, bool lo = false)
 {
     float v[8];
     const int r = min(row, rows - 1);
@@ -90,6 +95,10 @@ __device__ __forceinline__ half8_t weight_fragment(const float* __restrict__ w, 
     for (int j = 0; j < 8; ++j) v[j] = w[(size_t)r * cols + min((j < 4 ? ka : kb - 4) + j, cols - 1)];
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] = (enable && row < rows && (j < 4 ? ka : kb - 4) + j < cols) ? v[j] : 0.0f;
+    if (lo) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] -= (float)(_Float16)v[j];
+    }
     return to_half8(v);
 }
 
@@ -117,25 +126,45 @@ struct HeadWeights {
 
 template <int kTiles>
 __device__ __forceinline__ void load_head(const DecodeArgs& d, int head, int outputs, int row, int half,
-                                          HeadWeights<kTiles>& w)
+                                          HeadWeights<kTiles>& w, bool lo = false)
 {
     const int in = d.in_dim[head];
 #pragma unroll
-    for (int s = 0; s < 2; ++s) w.w0[s] = weight_fragment(d.w0[head], kFeat, in, row, 16 * s + 8 * half, 16 * s + 8 * half + 4);
-    w.w0[2] = weight_fragment(d.w0[head], kFeat, in, row, 32, 32, half == 0);
+    for (int s = 0; s < 2; ++s)
+        w.w0[s] = weight_fragment(d.w0[head], kFeat, in, row, 16 * s + 8 * half, 16 * s + 8 * half + 4, true, lo);
+    w.w0[2] = weight_fragment(d.w0[head], kFeat, in, row, 32, 32, half == 0, lo);
 #pragma unroll
     for (int r = 0; r < kTiles; ++r)
 #pragma unroll
         for (int s = 0; s < 2; ++s)
             w.w1[r][s] = weight_fragment(d.w1[head], outputs, kFeat, 32 * r + row, 16 * s + 4 * half,
-                                         16 * s + 8 + 4 * half);
+                                         16 * s + 8 + 4 * half, true, lo);
+}
+
+// The low parts of a head's weight fragments, kept in LDS: [fragment][lane], fragments in the order w0[0..2],
+// w1[0][0], w1[0][1], w1[1][0], ...  Every wavefront holds the same fragments in its lanes, so the workgroup shares
+// one copy; `store_head_lo` is called by one wavefront per head.
+template <int kTiles>
+__device__ __forceinline__ void store_head_lo(const DecodeArgs& d, int head, int outputs, int row, int half, int lane,
+                                              half8_t (*dst)[64])
+{
+    HeadWeights<kTiles> w;
+    load_head<kTiles>(d, head, outputs, row, half, w, true);
+#pragma unroll
+    for (int s = 0; s < 3; ++s) dst[s][lane] = w.w0[s];
+#pragma unroll
+    for (int r = 0; r < kTiles; ++r)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) dst[3 + 2 * r + s][lane] = w.w1[r][s];
 }
 
 // One head for one tile of 32 anchors: returns up to kTiles accumulators of the
 // second layer (rows = outputs 32r + 8b + 4*half + t, column = this lane's anchor).
-template <int kTiles, bool kSplit>
-__device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const float* bias0, const float* bias1,
-                                         const half8_t X[kSplit ? 5 : 3], int half, floatx16 out[kTiles])
+// `wlo`: the head's low weight fragments in LDS (kWLo), read right before their matrix instruction.
+template <int kTiles, bool kSplit, bool kWLo>
+__device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const half8_t (*wlo)[64], int lane,
+                                         const float* bias0, const float* bias1, const half8_t X[kSplit ? 5 : 3],
+                                         int half, floatx16 out[kTiles])
 {
     // layer 1: hidden = W0 [32 x in] * X^T + b0  (X[3], X[4]: the low parts of features that fp16 cannot hold)
     floatx16 h = bias_rows(bias0, 0, half);
@@ -144,6 +173,10 @@ __device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const flo
     if constexpr (kSplit) {
 #pragma unroll
         for (int s = 0; s < 2; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w0[s], X[3 + s], h, 0, 0, 0);
+    }
+    if constexpr (kWLo) {  // low parts of the weights against the high parts of the inputs
+#pragma unroll
+        for (int s = 0; s < 3; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[s][lane], X[s], h, 0, 0, 0);
     }
     // ReLU, then hi/lo split: registers 8s..8s+7 are the B operand of k-step s
     half8_t hh[2], hl[2];
@@ -167,6 +200,7 @@ __device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const flo
         for (int s = 0; s < 2; ++s) {
             c = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w1[r][s], hh[s], c, 0, 0, 0);
             c = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w1[r][s], hl[s], c, 0, 0, 0);
+            if constexpr (kWLo) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[3 + 2 * r + s][lane], hh[s], c, 0, 0, 0);
         }
         out[r] = c;
     }
@@ -199,8 +233,12 @@ struct TileInputs {
 constexpr int kRun = 128;
 
 // kSplit: the features enter as hi + lo fp16 pairs (general fp32 features; two more matrix instructions per head).
-template <bool kCountOnly, bool kSplit>
-__global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
+// kWLo: so do the weights (general fp32 weights; their low fragments take 19 KB of LDS in the emit pass, which
+// then runs three wavefronts per workgroup so that two workgroups still share a CU).
+constexpr int decode_waves(bool count_only, bool weights_lo) { return (weights_lo && !count_only) ? 3 : 4; }
+
+template <bool kCountOnly, bool kSplit, bool kWLo>
+__global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo))) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
                                                      const uint32_t* __restrict__ offsets, uint32_t capacity,
                                                      float* __restrict__ xyz, float* __restrict__ color,
                                                      float* __restrict__ opacity, float* __restrict__ scaling_out,
@@ -211,21 +249,30 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
     constexpr int kStrideMax = kCountOnly ? 11 : 123;
     constexpr int kListFloats = kCountOnly ? 0 : 160;  // 320 16-bit item numbers after the anchors' rows
     constexpr int kRunFloats = kRun / 4;                // kRun 8-bit positions of the run's visible anchors
-    __shared__ float s_out[4][32 * kStrideMax + kListFloats + kRunFloats];
+    constexpr int kWaves = decode_waves(kCountOnly, kWLo);
+    __shared__ float s_out[kWaves][32 * kStrideMax + kListFloats + kRunFloats];
 
     // biases of the three heads, zero-padded: b0 at [head*32], b1 of opacity / cov / colour at 96 / 128 / 224
     __shared__ float s_bias[256];
+    // low parts of the weight fragments: opacity head 0..4, covariance 5..13, colour 14..18
+    __shared__ half8_t s_wlo[kWLo ? (kCountOnly ? 5 : 19) : 1][64];
 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
     const int n = d.n;
-    {
-        const int t = threadIdx.x;
+    for (int t = threadIdx.x; t < 256; t += 64 * kWaves) {
         float v = 0.0f;
         if (t < 96) v = d.b0[t >> 5][t & 31];
         else if (t < 128) v = (t - 96) < n ? d.b1[0][t - 96] : 0.0f;
         else if (t < 224) v = (t - 128) < 7 * n ? d.b1[1][t - 128] : 0.0f;
         else v = (t - 224) < 3 * n ? d.b1[2][t - 224] : 0.0f;
         s_bias[t] = v;
+    }
+    if constexpr (kWLo) {
+        if (wave == 0) store_head_lo<1>(d, 0, n, col, half, lane, s_wlo);
+        if constexpr (!kCountOnly) {
+            if (wave == 1) store_head_lo<3>(d, 1, 7 * n, col, half, lane, s_wlo + 5);
+            if (wave == 2) store_head_lo<1>(d, 2, 3 * n, col, half, lane, s_wlo + 14);
+        }
     }
     __syncthreads();
     HeadWeights<1> w_op;
@@ -245,7 +292,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
     uint8_t* __restrict__ run_list = reinterpret_cast<uint8_t*>(mine + 32 * kStrideMax + kListFloats);
     const float cx = d.campos[0], cy = d.campos[1], cz = d.campos[2];
 
-    for (int run = blockIdx.x * 4 + wave; run < runs; run += gridDim.x * 4) {
+    for (int run = blockIdx.x * kWaves + wave; run < runs; run += gridDim.x * kWaves) {
       // positions (within the run) of its visible anchors, in order: lane covers anchors lane and 64 + lane
       const int base = run * kRun;
       const int a0 = base + lane, a1 = base + 64 + lane;
@@ -348,7 +395,7 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
         // smallest floats), so tanh itself is only evaluated for the offsets that are kept
         {
             floatx16 op[1];
-            run_head<1, kSplit>(w_op, s_bias, s_bias + 96, X, half, op);
+            run_head<1, kSplit, kWLo>(w_op, s_wlo, lane, s_bias, s_bias + 96, X, half, op);
             store_rows(mine + col * stride, 0, n, 0, half, op[0]);
         }
         if (kCountOnly) {
@@ -365,11 +412,11 @@ __global__ __launch_bounds__(256) void decode_kernel(DecodeArgs d, uint32_t* __r
 
         // ---- covariance and colour heads ----
         floatx16 cv[3];
-        run_head<3, kSplit>(w_cov, s_bias + 32, s_bias + 128, X, half, cv);
+        run_head<3, kSplit, kWLo>(w_cov, s_wlo + (kWLo ? 5 : 0), lane, s_bias + 32, s_bias + 128, X, half, cv);
 #pragma unroll
         for (int r = 0; r < 3; ++r) store_rows(mine + col * stride, n, 7 * n, 32 * r, half, cv[r]);
         floatx16 cl[1];
-        run_head<1, kSplit>(w_col, s_bias + 64, s_bias + 224, X, half, cl);
+        run_head<1, kSplit, kWLo>(w_col, s_wlo + (kWLo ? 14 : 0), lane, s_bias + 64, s_bias + 224, X, half, cl);
         store_rows(mine + col * stride, 8 * n, 3 * n, 0, half, cl[0]);
         {
             float* __restrict__ extra = mine + col * stride + 11 * n;
@@ -633,6 +680,7 @@ static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, bool all
     a.campos = an->campos;
     a.level = dec->add_level ? an->level : nullptr;
     a.split_feat = (dec->fp32_features || dec->bank_in_dim != 0) ? 1 : 0;  // bank-mixed features are general floats
+    a.weights_lo = dec->fp32_weights ? 1 : 0;
     for (int j = 0; j < 3; ++j) {
         a.in_dim[j] = dec->in_dim[j];
         a.w0[j] = dec->w0[j];
@@ -650,17 +698,26 @@ static int fill_args(const gs355_decoder* dec, const gs355_anchors* an, bool all
 
 // Persistent workgroups (4 wavefronts, each walking runs of kRun anchors): at most `cap` of them, about what
 // the chip holds at once, so the weight fragments are fetched once per resident workgroup.
-static dim3 decode_grid(int A, int cap)
+static dim3 decode_grid(int A, int cap, int waves = 4)
 {
     const int runs = (A + kRun - 1) / kRun;
-    int blocks = (runs + 3) / 4;
+    int blocks = (runs + waves - 1) / waves;
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
     return dim3(blocks);
 }
 
-// Launch the count or the emit pass in the variant the features need.
-static void launch_decode(bool count_only, dim3 grid, hipStream_t s, const DecodeArgs& a, uint32_t* counts,
+// Launch the count or the emit pass in the variant the features and the weights need.  `cap`: most workgroups.
+template <bool kCountOnly, bool kSplit, bool kWLo>
+static void launch_variant(int cap, hipStream_t s, const DecodeArgs& a, uint32_t* counts, const uint32_t* offsets,
+                           uint32_t capacity, float* xyz, float* color, float* opacity, float* scaling, float* rot)
+{
+    constexpr int kWaves = decode_waves(kCountOnly, kWLo);
+    hipLaunchKernelGGL((decode_kernel<kCountOnly, kSplit, kWLo>), decode_grid(a.A, cap, kWaves), dim3(64 * kWaves), 0, s, a,
+                       counts, offsets, capacity, xyz, color, opacity, scaling, rot);
+}
+
+static void launch_decode(bool count_only, int cap, hipStream_t s, const DecodeArgs& a, uint32_t* counts,
                           const uint32_t* offsets, uint32_t capacity, const gs355_decoded* out)
 {
     float* xyz = out ? out->xyz : nullptr;
@@ -668,21 +725,18 @@ static void launch_decode(bool count_only, dim3 grid, hipStream_t s, const Decod
     float* opacity = out ? out->opacity : nullptr;
     float* scaling = out ? out->scaling : nullptr;
     float* rot = out ? out->rot : nullptr;
-    if (count_only) {
-        if (a.split_feat)
-            hipLaunchKernelGGL((decode_kernel<true, true>), grid, dim3(256), 0, s, a, counts, offsets, capacity, xyz, color,
-                               opacity, scaling, rot);
-        else
-            hipLaunchKernelGGL((decode_kernel<true, false>), grid, dim3(256), 0, s, a, counts, offsets, capacity, xyz, color,
-                               opacity, scaling, rot);
-    } else {
-        if (a.split_feat)
-            hipLaunchKernelGGL((decode_kernel<false, true>), grid, dim3(256), 0, s, a, counts, offsets, capacity, xyz, color,
-                               opacity, scaling, rot);
-        else
-            hipLaunchKernelGGL((decode_kernel<false, false>), grid, dim3(256), 0, s, a, counts, offsets, capacity, xyz, color,
-                               opacity, scaling, rot);
-    }
+#define GS355_DECODE_CASE(C, S, W)                                                                             \
+    if (count_only == C && (a.split_feat != 0) == S && (a.weights_lo != 0) == W)                               \
+        launch_variant<C, S, W>(cap, s, a, counts, offsets, capacity, xyz, color, opacity, scaling, rot);
+    GS355_DECODE_CASE(true, false, false)
+    GS355_DECODE_CASE(true, false, true)
+    GS355_DECODE_CASE(true, true, false)
+    GS355_DECODE_CASE(true, true, true)
+    GS355_DECODE_CASE(false, false, false)
+    GS355_DECODE_CASE(false, false, true)
+    GS355_DECODE_CASE(false, true, false)
+    GS355_DECODE_CASE(false, true, true)
+#undef GS355_DECODE_CASE
 }
 
 }  // namespace gs355
@@ -743,7 +797,7 @@ int gs355_decode_count(const gs355_decoder* dec, const gs355_anchors* an, uint32
     if (scratch_bytes < need)
         return set_error(GS355_ENOSPC, "decode scratch has %zu bytes, %zu needed", scratch_bytes, need);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    launch_decode(true, decode_grid(a.A, 1024), s, a, counts, nullptr, 0u, nullptr);
+    launch_decode(true, 1024, s, a, counts, nullptr, 0u, nullptr);
     GS355_CHECK_LAUNCH("decode: count");
     return launch_exclusive_scan(counts, offsets, (size_t)a.A, static_cast<uint32_t*>(scratch_buf), s);
 }
@@ -765,7 +819,7 @@ int gs355_decode_count_static(const gs355_decoder* dec, const gs355_anchors* an,
     uint32_t* tmp = nullptr;
     if ((rc = static_scratch(&tmp))) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    launch_decode(true, decode_grid(a.A, 1024), s, a, counts, nullptr, 0u, nullptr);
+    launch_decode(true, 1024, s, a, counts, nullptr, 0u, nullptr);
     GS355_CHECK_LAUNCH("decode: count");
     // the scan writes every block sum before it reads it: nothing in the array has to start at zero
     return launch_exclusive_scan(counts, offsets, (size_t)a.A, tmp, s);
@@ -784,7 +838,7 @@ int gs355_decode_emit(const gs355_decoder* dec, const gs355_anchors* an, const u
     if (!out || !out->xyz || !out->color || !out->opacity || !out->scaling || !out->rot)
         return set_error(GS355_EINVAL, "decoded outputs must all be non-NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    launch_decode(false, decode_grid(a.A, 512), s, a, nullptr, offsets, (uint32_t)capacity, out);
+    launch_decode(false, 512, s, a, nullptr, offsets, (uint32_t)capacity, out);
     GS355_CHECK_LAUNCH("decode: emit");
     return GS355_OK;
 }
@@ -873,7 +927,7 @@ int gs355_decode(const gs355_decoder* dec, const gs355_anchors* an, int64_t capa
             GS355_CHECK_LAUNCH("decode: feature bank");
         }
         a.run_totals = reinterpret_cast<uint2*>(ws + L.run_totals);
-        launch_decode(true, decode_grid(a.A, 1024), s, a, nullptr, nullptr, 0u, nullptr);
+        launch_decode(true, 1024, s, a, nullptr, nullptr, 0u, nullptr);
         GS355_CHECK_LAUNCH("decode: count");
         hipLaunchKernelGGL(run_scan_kernel, dim3(1), dim3(1024), 0, s, a.run_totals, run_base, runs, out->count,
                            out->num_visible);
@@ -885,7 +939,7 @@ int gs355_decode(const gs355_decoder* dec, const gs355_anchors* an, int64_t capa
     a.run_base = run_base;
     a.neural_opacity = out->neural_opacity;
     a.kept_mask = out->mask;
-    launch_decode(false, decode_grid(a.A, 512), s, a, nullptr, nullptr, (uint32_t)capacity, out);
+    launch_decode(false, 512, s, a, nullptr, nullptr, (uint32_t)capacity, out);
     GS355_CHECK_LAUNCH("decode: emit");
     return GS355_OK;
 }

@@ -23,7 +23,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert names == sorted(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.gs355_version() == 2
+    assert lib.gs355_version() == _lib.ABI_VERSION == 3
 
 
 def test_struct_sizes_match_the_header():

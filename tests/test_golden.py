@@ -1,7 +1,7 @@
 """Committed golden fixtures (tests/golden/*.npz, written by tests/golden/make_golden.py): frozen inputs with the
 CPU checker's outputs.  CPU tests keep the checkers on them; GPU tests hold the HIP path to them through the same
 entry points the models use.  Integer results must match exactly; images to 1e-4 outside the pixels the checker
-flagged as threshold-adjacent and >= 60 dB overall; the decode to 2e-5 of the output scale."""
+flagged as threshold-adjacent and >= 60 dB overall; the decode to 3e-5 of the output scale."""
 import math
 import os
 
@@ -117,4 +117,4 @@ def test_hip_decode_reproduces_the_golden_decode(gpu_device):
     for name, got in (("xyz", xyz), ("color", color), ("opacity", opacity), ("scaling", scaling), ("rot", rot)):
         assert got.shape == want[name].shape, name
         scale = max(1.0, float(np.abs(want[name]).max()))
-        assert float(np.abs(got.cpu().numpy() - want[name]).max()) / scale <= 2e-5, name
+        assert float(np.abs(got.cpu().numpy() - want[name]).max()) / scale <= 3e-5, name

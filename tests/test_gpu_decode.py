@@ -10,7 +10,9 @@ from oracle import anchor_oracle as ao
 
 pytestmark = pytest.mark.gpu
 
-TOL = 2e-5  # fp32 accumulation order differs between the matrix cores and torch's CPU GEMM
+# fp32 accumulation order differs between the matrix cores and torch's CPU GEMM, and the hi + lo fp16 operands carry
+# 22 significant bits: random sweeps over every option reached 2.4e-5 on single outputs with large pre-activations
+TOL = 3e-5
 
 
 def build_decoder(sc, device, add_dist=(True, True, True)):
@@ -80,6 +82,37 @@ def test_decode_matches_oracle(gpu_device, A, frac):
     redo = lambda keep=None: ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp,  # noqa: E731
                                        sc.n_offsets, keep_override=keep)
     compare(got, redo(), redo)
+
+
+@pytest.mark.parametrize("A,features_too", [(20_000, False), (20_000, True), (300_000, True)])
+def test_decode_with_weights_fp16_cannot_represent(gpu_device, A, features_too):
+    """An fp32-trained checkpoint: weights (and features) with all 24 significant bits in use.  The decoder detects
+    them and feeds the matrix cores hi + lo fp16 pairs; the result meets the same bar as with fp16-exact weights
+    (rounding the weights to fp16 alone would move the outputs by ~1e-3)."""
+    sc = scenes.config5(A=A)
+    g = torch.Generator().manual_seed(77)
+    mlp = {}
+    for head, (w0, b0, w1, b1) in sc.mlp.items():
+        mlp[head] = (w0 * (1.0 + 1e-3 * torch.randn(w0.shape, generator=g)), 0.1 * torch.randn(b0.shape, generator=g),
+                     w1 * (1.0 + 1e-3 * torch.randn(w1.shape, generator=g)), 0.1 * torch.randn(b1.shape, generator=g))
+        assert not torch.equal(mlp[head][0].half().float(), mlp[head][0])
+    sc.mlp = mlp
+    feat = sc.anchor_feat * (1.0 + 1e-3 * torch.randn(sc.anchor_feat.shape, generator=g)) if features_too else sc.anchor_feat
+    vis = torch.rand(A, generator=g) < 0.6
+    dec = build_decoder(sc, gpu_device)
+    cam = sc.camera.camera_center
+    got = dec(camera_center=cam.to(gpu_device), anchor=sc.anchor.to(gpu_device), anchor_feat=feat.to(gpu_device),
+              offset=sc.offset.to(gpu_device), scaling=sc.scaling.to(gpu_device), visible_mask=vis.to(gpu_device))
+    assert dec._decoder_struct(gpu_device).fp32_weights == 1
+    redo = lambda keep=None: ao.decode(cam, sc.anchor, feat, sc.offset, sc.scaling, vis, sc.mlp,  # noqa: E731
+                                       sc.n_offsets, keep_override=keep)
+    compare(got, redo(), redo)
+    # the one-call decode (count kept on the device) takes the same variant of the kernels
+    dev = dec.decode_on_device(cam.to(gpu_device), sc.anchor.to(gpu_device), feat.to(gpu_device),
+                               sc.offset.to(gpu_device), sc.scaling.to(gpu_device), vis.to(gpu_device))
+    G = int(dev.counts[0])
+    assert G == got[0].shape[0]
+    assert torch.equal(dev.xyz[:G], got[0]) and torch.equal(dev.rot[:G], got[4])
 
 
 def test_decode_heads_without_distance_and_fewer_offsets(gpu_device):

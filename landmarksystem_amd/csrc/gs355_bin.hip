@@ -1038,31 +1038,23 @@ struct LdsSorter {
             }
         }
         __syncthreads();
-        uint32_t csize = 0;
+        uint32_t csize = 0, own = 0;
         if (tid < 256) {  // exclusive scan of the coarse counts (wavefronts 0..3)
-            csize = coarse[tid];
-            uint32_t inc = csize;
+            own = coarse[tid];
+            uint32_t inc = own;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
                 const uint32_t up = __shfl_up(inc, d, 64);
                 if (lane >= d) inc += up;
             }
             if (lane == 63) flags[16 + wave] = inc;
-            csize = inc - csize;  // exclusive within the wavefront
+            csize = inc - own;  // exclusive within the wavefront
         }
         __syncthreads();
-        if (tid < 256) {
+        if (tid < 256) {  // (a thread replaces the one count that only it has read)
             for (int w = 0; w < wave; ++w) csize += flags[16 + w];
-        }
-        __syncthreads();
-        uint32_t my_size = 0;
-        if (tid < 256) {
-            my_size = coarse[tid];  // read the count before it is replaced by the prefix
-        }
-        __syncthreads();
-        if (tid < 256) {
             coarse[tid] = csize;
-            coarse[256 + tid] = my_size;
+            coarse[256 + tid] = own;
         }
         __syncthreads();
         uint32_t bin[kR], slot[kR];
@@ -1128,48 +1120,88 @@ struct LdsSorter {
         return 1;
     }
 
-    __device__ void run(uint32_t tile, const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ buckets,
-                        uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals) const
+    // A bucket on its way from memory: where it lies and this thread's pairs of it (requested, not yet used).
+    struct Fetched {
+        uint32_t tile, lo, n;
+        uint64_t v[kR];
+    };
+
+    __device__ __forceinline__ void fetch_range(Fetched& f, uint32_t tile, const uint32_t* __restrict__ ranges) const
     {
-        const uint32_t lo = ranges[2 * tile], n = ranges[2 * tile + 1] - lo;
+        f.tile = tile;
+        f.lo = ranges[2 * tile];
+        f.n = ranges[2 * tile + 1] - f.lo;
+    }
+
+    // the whole bucket is requested before the first pair is used: one memory latency, not one per round
+    __device__ __forceinline__ void fetch_pairs(Fetched& f, const uint64_t* __restrict__ buckets) const
+    {
+        const bool mine = f.n != 0 && f.n <= (uint32_t)kCap;
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t j = (uint32_t)r * kT + threadIdx.x;
+            f.v[r] = mine && j < f.n ? buckets[f.lo + j] : 0ull;
+        }
+    }
+
+    // Sorts the fetched bucket and writes it out; ends with a barrier.
+    __device__ void sort_fetched(const Fetched& f, uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals) const
+    {
+        const uint32_t lo = f.lo, n = f.n, tile = f.tile;
         if (n == 0 || n > (uint32_t)kCap) return;  // uniform over the workgroup
         if (threadIdx.x == 0) {
             flags[11] = 0;
             flags[12] = 0xFFFFFFFFu;
             flags[13] = 0;
+            flags[14] = 0xFFFFFFFFu;
         }
         __syncthreads();
-        const uint32_t d0 = (uint32_t)(buckets[lo] >> 32);
-        uint32_t diff = 0, dmin = 0xFFFFFFFFu, dmax = 0;
-        for (uint32_t j = threadIdx.x; j < n; j += kT) {
-            const uint64_t v = buckets[lo + j];
-            const uint32_t dj = (uint32_t)(v >> 32);
-            depth[j] = dj;
-            index[j] = (uint32_t)v;
-            diff |= dj ^ d0;
-            dmin = min(dmin, dj);
-            dmax = max(dmax, dj);
+        // depth bits that differ somewhere in the bucket = (OR of all) ^ (AND of all)
+        uint32_t any = 0, all = 0xFFFFFFFFu, dmin = 0xFFFFFFFFu, dmax = 0;
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t j = (uint32_t)r * kT + threadIdx.x;
+            if (j < n) {
+                const uint32_t dj = (uint32_t)(f.v[r] >> 32);
+                depth[j] = dj;
+                index[j] = (uint32_t)f.v[r];
+                any |= dj;
+                all &= dj;
+                dmin = min(dmin, dj);
+                dmax = max(dmax, dj);
+            }
         }
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) {
-            diff |= __shfl_xor(diff, d, 64);
+            any |= __shfl_xor(any, d, 64);
+            all &= __shfl_xor(all, d, 64);
             dmin = min(dmin, (uint32_t)__shfl_xor(dmin, d, 64));
             dmax = max(dmax, (uint32_t)__shfl_xor(dmax, d, 64));
         }
         if ((threadIdx.x & 63) == 0) {
-            if (diff) atomicOr(&flags[11], diff);
+            atomicOr(&flags[11], any);
+            atomicAnd(&flags[14], all);
             atomicMin(&flags[12], dmin);
             atomicMax(&flags[13], dmax);
         }
         __syncthreads();
         int cur = bucket_sort(n, flags[12], flags[13]);
-        if (cur == -2) cur = sort(n, flags[11]);
+        if (cur == -2) cur = sort(n, flags[11] ^ flags[14]);
         for (uint32_t j = threadIdx.x; j < n; j += kT) {
             const uint32_t e = cur < 0 ? j : (uint32_t)perm(cur)[j];
             out_keys[lo + j] = ((uint64_t)tile << 32) | (uint64_t)depth[e];
             out_vals[lo + j] = index[e];
         }
         __syncthreads();
+    }
+
+    __device__ void run(uint32_t tile, const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ buckets,
+                        uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals) const
+    {
+        Fetched f;
+        fetch_range(f, tile, ranges);
+        fetch_pairs(f, buckets);
+        sort_fetched(f, out_keys, out_vals);
     }
 };
 
@@ -1184,11 +1216,9 @@ __global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* 
                                                             const uint32_t* __restrict__ ranges,
                                                             uint64_t* __restrict__ buckets,
                                                             uint64_t* __restrict__ out_keys,
-                                                            uint32_t* __restrict__ out_vals,
-                                                            uint32_t* __restrict__ list_work, uint32_t skip_classes)
+                                                            uint32_t* __restrict__ out_vals, uint32_t skip_classes)
 {
     extern __shared__ uint32_t s_dyn[];
-    if (blockIdx.x == 0 && threadIdx.x < 4) list_work[threadIdx.x] = 0u;  // for the list kernels launched after this one
     if (header->overflow) return;
     static_assert(kT == kThreads, "the global-memory passes are written for kThreads threads");
     static_assert((256 + kWaves * 256 + 8) * sizeof(uint32_t) <= LdsSorter<kT, kR>::kBytes, "scratch of the global passes");
@@ -1211,57 +1241,53 @@ __global__ __launch_bounds__(kT) void tile_sort_each_kernel(const gs355_header* 
     sorter.run(tile, ranges, buckets, out_keys, out_vals);
 }
 
-// Larger size classes: persistent workgroups over the class list made by tile_publish_kernel.  A workgroup starts
-// with the list entry of its own number and then takes the next one nobody has taken (`work`, a counter cleared by
-// tile_sort_each_kernel): buckets of one class differ in size by a factor of two and more, and a fixed assignment
-// leaves most of the chip waiting for the workgroups that drew the large ones.  The request for the next entry is
-// issued before the current bucket is sorted, so its latency is not waited for.
-template <int kT, int kR>
+// Larger size classes: one workgroup per entry of the class list made by tile_publish_kernel.  The number of
+// entries is only known on the device, so a launch has a workgroup per tile and those past the list's end leave at
+// once: the hardware's own dispatch hands out the buckets.  (Persistent workgroups that fetched their work from a
+// counter spent 8-14 us per bucket on dependent requests -- counter, list entry, range, pairs -- whatever the
+// bucket held, requesting the next bucket inside the current sort did not hide them, and even a plain strided loop
+// around the sort costs a sixth of the kernel's time in registers kept alive across it.)  kStrided: a launch
+// smaller than the list, for the class whose workgroups fill a CU each.
+template <int kT, int kR, bool kStrided>
 __device__ __forceinline__ void tile_sort_list_body(const gs355_header* __restrict__ header,
                                                     const uint32_t* __restrict__ ranges,
                                                     const uint32_t* __restrict__ list,
-                                                    const uint32_t* __restrict__ list_count, uint32_t* __restrict__ work,
+                                                    const uint32_t* __restrict__ list_count,
                                                     const uint64_t* __restrict__ buckets,
                                                     uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals,
                                                     uint32_t* lds)
 {
-    __shared__ uint32_t s_next;
     if (header->overflow) return;
     const LdsSorter<kT, kR> sorter(lds);
     const uint32_t count = *list_count;
-    uint32_t k = blockIdx.x;
-    while (k < count) {
-        uint32_t next = 0;
-        if (threadIdx.x == 0) next = atomicAdd(work, 1u) + gridDim.x;
-        sorter.run(list[k], ranges, buckets, out_keys, out_vals);  // (ends with a barrier)
-        if (threadIdx.x == 0) s_next = next;
-        __syncthreads();
-        k = s_next;  // the next write of s_next comes after the barriers of the next run
+    if (kStrided) {
+        for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) sorter.run(list[k], ranges, buckets, out_keys, out_vals);
+    } else if (blockIdx.x < count) {
+        sorter.run(list[blockIdx.x], ranges, buckets, out_keys, out_vals);
     }
 }
 
 // 1024 threads x 5 rounds, held to 64 VGPRs so that two workgroups share a CU
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void tile_sort_list_1024x5_kernel(
     const gs355_header* __restrict__ header, const uint32_t* __restrict__ ranges, const uint32_t* __restrict__ list,
-    const uint32_t* __restrict__ list_count, uint32_t* __restrict__ work, const uint64_t* __restrict__ buckets,
-    uint64_t* __restrict__ out_keys, uint32_t* __restrict__ out_vals)
+    const uint32_t* __restrict__ list_count, const uint64_t* __restrict__ buckets, uint64_t* __restrict__ out_keys,
+    uint32_t* __restrict__ out_vals)
 {
     extern __shared__ uint32_t s_dyn[];
-    tile_sort_list_body<1024, 5>(header, ranges, list, list_count, work, buckets, out_keys, out_vals, s_dyn);
+    tile_sort_list_body<1024, 5, false>(header, ranges, list, list_count, buckets, out_keys, out_vals, s_dyn);
 }
 
-template <int kT, int kR>
+template <int kT, int kR, bool kStrided>
 __global__ __launch_bounds__(kT) void tile_sort_list_kernel(const gs355_header* __restrict__ header,
                                                             const uint32_t* __restrict__ ranges,
                                                             const uint32_t* __restrict__ list,
                                                             const uint32_t* __restrict__ list_count,
-                                                            uint32_t* __restrict__ work,
                                                             const uint64_t* __restrict__ buckets,
                                                             uint64_t* __restrict__ out_keys,
                                                             uint32_t* __restrict__ out_vals)
 {
     extern __shared__ uint32_t s_dyn[];
-    tile_sort_list_body<kT, kR>(header, ranges, list, list_count, work, buckets, out_keys, out_vals, s_dyn);
+    tile_sort_list_body<kT, kR, kStrided>(header, ranges, list, list_count, buckets, out_keys, out_vals, s_dyn);
 }
 
 }  // namespace
@@ -1302,7 +1328,7 @@ static int allow_large_lds()
         (e = raise_lds_limit(scatter_kernel<0, false>, bin_bytes)) != hipSuccess ||
         (e = raise_lds_limit(scatter_kernel<kCoarseShift, true>, bin_bytes)) != hipSuccess ||
         (e = raise_lds_limit(tile_sort_list_1024x5_kernel, LdsSorter<1024, 5>::kBytes)) != hipSuccess ||
-        (e = raise_lds_limit(tile_sort_list_kernel<1024, 10>, LdsSorter<1024, 10>::kBytes)) != hipSuccess)
+        (e = raise_lds_limit(tile_sort_list_kernel<1024, 10, true>, LdsSorter<1024, 10>::kBytes)) != hipSuccess)
         return set_error(GS355_EHIP, "LDS limit of the binning / tile sort kernels: %s", hipGetErrorString(e));
     done[dev].store(1, std::memory_order_release);  // racing threads set the same values
     return GS355_OK;
@@ -1442,25 +1468,26 @@ int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* rang
     int rc;
     if ((rc = allow_large_lds())) return rc;
     const uint32_t* list0 = lists + kListHeader;
-    uint32_t* work = lists + 4;  // next untaken entry of each class list
     hipLaunchKernelGGL((tile_sort_each_kernel<256, 4>), dim3(tiles), dim3(256), S0::kBytes, s, header, ranges, buckets,
-                       out_keys, out_vals, work, skip_classes);
+                       out_keys, out_vals, skip_classes);
     GS355_CHECK_LAUNCH("tile sort: class 0");
-    auto grid = [&](int want) { return dim3(tiles < want ? tiles : want); };
+    // A launch per larger class, a workgroup per tile: those past the end of the class's list leave at once, which
+    // costs nothing measurable (sizing the launch by the list's expected length changed no kernel's time).  The
+    // largest class is the exception: a workgroup of it fills a CU, so its launch is the chip's size and strides.
     // (skip_classes: bit c set = the caller expects list c to be empty; the kernel above has sorted what is on it)
     if (!(skip_classes & 1u)) {
-        hipLaunchKernelGGL((tile_sort_list_kernel<512, 4>), grid(1024), dim3(512), S1::kBytes, s, header, ranges, list0,
-                           lists + 0, work + 0, buckets, out_keys, out_vals);
+        hipLaunchKernelGGL((tile_sort_list_kernel<512, 4, false>), dim3(tiles), dim3(512), S1::kBytes, s, header, ranges,
+                           list0, lists + 0, buckets, out_keys, out_vals);
         GS355_CHECK_LAUNCH("tile sort: class 1");
     }
     if (!(skip_classes & 2u)) {
-        hipLaunchKernelGGL(tile_sort_list_1024x5_kernel, grid(512), dim3(1024), S2::kBytes, s, header, ranges,
-                           list0 + (size_t)tiles, lists + 1, work + 1, buckets, out_keys, out_vals);
+        hipLaunchKernelGGL(tile_sort_list_1024x5_kernel, dim3(tiles), dim3(1024), S2::kBytes, s, header, ranges,
+                           list0 + (size_t)tiles, lists + 1, buckets, out_keys, out_vals);
         GS355_CHECK_LAUNCH("tile sort: class 2");
     }
     if (!(skip_classes & 4u)) {
-        hipLaunchKernelGGL((tile_sort_list_kernel<1024, 10>), grid(256), dim3(1024), S3::kBytes, s, header, ranges,
-                           list0 + 2 * (size_t)tiles, lists + 2, work + 2, buckets, out_keys, out_vals);
+        hipLaunchKernelGGL((tile_sort_list_kernel<1024, 10, true>), dim3(tiles < 256 ? tiles : 256), dim3(1024), S3::kBytes,
+                           s, header, ranges, list0 + 2 * (size_t)tiles, lists + 2, buckets, out_keys, out_vals);
         GS355_CHECK_LAUNCH("tile sort: class 3");
     }
     return GS355_OK;

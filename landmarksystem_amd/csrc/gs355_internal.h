@@ -159,7 +159,7 @@ int launch_tile_scatter(const FrameArgs& f, int32_t P, const uint64_t* rects, co
                         gs355_header* header, const uint32_t* matrix, const uint32_t* group_visible, uint32_t n_cap,
                         uint32_t* tile_base, uint32_t* ranges, uint32_t* lists, uint64_t* buckets, uint64_t* coarse,
                         int levels, hipStream_t s);
-// lists: u32[kListHeader + 4 * tiles]: the four class counts, the class lists' work counters, the four lists
+// lists: u32[kListHeader + 4 * tiles]: the four class counts, four spare words, the four lists
 constexpr int kListHeader = 8;
 int launch_tile_sort(const gs355_header* header, int tiles, const uint32_t* ranges, uint32_t* lists,
                      uint64_t* buckets, uint64_t* out_keys, uint32_t* out_vals, uint32_t skip_classes, hipStream_t s);

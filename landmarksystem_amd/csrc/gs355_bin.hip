@@ -854,7 +854,14 @@ template <int kT, int kR>
 struct LdsSorter {
     static constexpr int kW = kT / 64;
     static constexpr int kCap = kT * kR;
-    static constexpr size_t kBytes = (size_t)kCap * 12 + (size_t)kW * 256 * 4 + 192;
+#ifndef GS_BINS_PER
+#define GS_BINS_PER 4
+#endif
+    static constexpr int kBinsPer = kT >= 512 ? GS_BINS_PER : 2;  // fine bins per thread of the counting pass
+    static constexpr int kB = kBinsPer * kT;                      // fine bins
+    // counters: [kW][256] words for the radix passes, or the fine bins and 512 coarse words of the counting pass
+    static constexpr int kCounterWords = kB + 512 > kW * 256 ? kB + 512 : kW * 256;
+    static constexpr size_t kBytes = (size_t)kCap * 12 + (size_t)kCounterWords * 4 + 192;
 
     uint32_t* depth;     // [kCap]
     uint32_t* index;     // [kCap]
@@ -868,7 +875,7 @@ struct LdsSorter {
         index = lds + kCap;
         perm0 = reinterpret_cast<uint16_t*>(lds + 2 * kCap);
         cnt = reinterpret_cast<uint32_t(*)[256]>(lds + 3 * kCap);
-        flags = lds + 3 * kCap + kW * 256;
+        flags = lds + 3 * kCap + kCounterWords;
     }
 
     __device__ __forceinline__ uint16_t* perm(int which) const { return perm0 + which * kCap; }
@@ -1008,18 +1015,19 @@ struct LdsSorter {
     __device__ int bucket_sort(uint32_t n, uint32_t dmin, uint32_t dmax) const
     {
         const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-        uint32_t* const count = &cnt[0][0];  // [kT] pairs per bin, then the bin's first slot
-        uint32_t* const coarse = count + kT;  // [256] pairs per coarse bin, then their exclusive prefix
+        uint32_t* const count = &cnt[0][0];  // [kB] pairs per bin, then the bin's first slot
+        uint32_t* const coarse = count + kB;  // [256] pairs per coarse bin, then their exclusive prefix
         const uint32_t range = dmax - dmin;
         if (range == 0) return -2;
         // coarse(d) = floor((d - dmin) * 256 / (range + 1)) as the high word of a 32x32 multiply, whose low word is
         // the position inside the coarse bin as a 0.32 fraction; a range below 256 gives every depth its own bin
         const bool direct = range < 256u;
         const uint32_t mult = direct ? 0u : (uint32_t)((256ull << 32) / ((uint64_t)range + 1ull));
-        // position -> bin: floor(pos * kT / n) for n > kT, else the position itself (one pair per bin)
-        const bool spread = n > (uint32_t)kT;
-        const uint32_t to_bin = spread ? (uint32_t)(((uint64_t)kT << 32) / (uint64_t)n) : 0u;
-        count[tid] = 0;
+        // position -> bin: floor(pos * kB / n) for n > kB, else the position itself (one pair per bin)
+        const bool spread = n > (uint32_t)kB;
+        const uint32_t to_bin = spread ? (uint32_t)(((uint64_t)kB << 32) / (uint64_t)n) : 0u;
+#pragma unroll
+        for (int i = 0; i < kBinsPer; ++i) count[i * kT + tid] = 0;
         if (tid < 256) coarse[tid] = 0;
         if (tid == 0) flags[8] = 0;
         __syncthreads();
@@ -1065,13 +1073,21 @@ struct LdsSorter {
             slot[r] = 0;
             if (j < n) {
                 const uint32_t pos = coarse[cbin[r]] + __umulhi(frac[r], coarse[256 + cbin[r]]);  // in [0, n)
-                bin[r] = min(spread ? __umulhi(pos, to_bin) : pos, (uint32_t)kT - 1u);
+                bin[r] = min(spread ? __umulhi(pos, to_bin) : pos, (uint32_t)kB - 1u);
                 slot[r] = atomicAdd(&count[bin[r]], 1u);
             }
         }
         __syncthreads();
-        // exclusive scan of the kT bin counts; remember whether any bin is over-full
-        const uint32_t c = count[tid];
+        // exclusive scan of the kB bin counts (a thread owns kBinsPer consecutive bins); remember whether any bin
+        // is over-full
+        uint32_t mine[kBinsPer], c = 0;
+        bool overfull = false;
+#pragma unroll
+        for (int i = 0; i < kBinsPer; ++i) {
+            mine[i] = count[kBinsPer * tid + i];
+            c += mine[i];
+            overfull = overfull || mine[i] > kMaxBin;
+        }
         uint32_t inc = c;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
@@ -1079,7 +1095,7 @@ struct LdsSorter {
             if (lane >= d) inc += up;
         }
         if (lane == 63) flags[16 + wave] = inc;
-        if (c > kMaxBin) flags[8] = 1;
+        if (overfull) flags[8] = 1;
         __syncthreads();
         if (flags[8] != 0) {
             __syncthreads();
@@ -1087,7 +1103,11 @@ struct LdsSorter {
         }
         uint32_t first = inc - c;
         for (int w = 0; w < wave; ++w) first += flags[16 + w];
-        count[tid] = first;
+#pragma unroll
+        for (int i = 0; i < kBinsPer; ++i) {
+            count[kBinsPer * tid + i] = first;
+            first += mine[i];
+        }
         __syncthreads();
         uint16_t* const P = perm(0);
 #pragma unroll
@@ -1105,7 +1125,7 @@ struct LdsSorter {
             if (j < n) {
                 const uint32_t b = bin[r];
                 const uint32_t lo_slot = count[b];
-                const uint32_t hi_slot = b + 1 < (uint32_t)kT ? count[b + 1] : n;
+                const uint32_t hi_slot = b + 1 < (uint32_t)kB ? count[b + 1] : n;
                 const uint32_t md = depth[j], mi = index[j];
                 uint32_t rank = 0;
                 for (uint32_t q = lo_slot; q < hi_slot; ++q) {

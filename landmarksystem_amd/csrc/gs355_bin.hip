@@ -1160,7 +1160,7 @@ struct LdsSorter {
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
             const uint32_t j = (uint32_t)r * kT + threadIdx.x;
-            f.v[r] = mine && j < f.n ? buckets[f.lo + j] : 0ull;
+            f.v[r] = mine && j < f.n ? __builtin_nontemporal_load(&buckets[f.lo + j]) : 0ull;  // (read once)
         }
     }
 
@@ -1209,7 +1209,9 @@ struct LdsSorter {
         if (cur == -2) cur = sort(n, flags[11] ^ flags[14]);
         for (uint32_t j = threadIdx.x; j < n; j += kT) {
             const uint32_t e = cur < 0 ? j : (uint32_t)perm(cur)[j];
-            out_keys[lo + j] = ((uint64_t)tile << 32) | (uint64_t)depth[e];
+            // (no later stage reads the sorted keys: a streaming store, which leaves the cache to the records the
+            // blend is about to gather)
+            __builtin_nontemporal_store(((uint64_t)tile << 32) | (uint64_t)depth[e], &out_keys[lo + j]);
             out_vals[lo + j] = index[e];
         }
         __syncthreads();

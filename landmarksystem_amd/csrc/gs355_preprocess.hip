@@ -133,7 +133,11 @@ __device__ __forceinline__ void sh_colour_of_entries(float4* __restrict__ mine, 
         const int e = min(q4 / 12, count - 1), m = q4 % 12;
         const float4* __restrict__ block =
             reinterpret_cast<const float4*>(shs + (group_first + owner[first_entry + e]) * 48);
-        v[it] = block[m];
+        {  // (read once per frame: a streaming load, which leaves the cache to the records the blend gathers)
+            typedef float f4v __attribute__((ext_vector_type(4)));
+            const f4v t = __builtin_nontemporal_load(reinterpret_cast<const f4v*>(block) + m);
+            v[it] = make_float4(t.x, t.y, t.z, t.w);
+        }
         dst[it] = e * (kShStride / 4) + m;
     }
 #pragma unroll
@@ -195,10 +199,12 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
     float cov[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, scale[3] = {0.f, 0.f, 0.f}, quat[4] = {0.f, 0.f, 0.f, 0.f};
     float opacity = 0.f;
     bool gated = false;  // anchor outside the level-of-detail mask (anchor prefilter only)
+// (the per-Gaussian inputs are read once per frame: streaming loads)
+#define GEO_LOAD(p) __builtin_nontemporal_load(&(p))
     if (valid) {
-        x = g.means3D[3 * (size_t)i];
-        y = g.means3D[3 * (size_t)i + 1];
-        z = g.means3D[3 * (size_t)i + 2];
+        x = GEO_LOAD(g.means3D[3 * (size_t)i]);
+        y = GEO_LOAD(g.means3D[3 * (size_t)i + 1]);
+        z = GEO_LOAD(g.means3D[3 * (size_t)i + 2]);
         if (kRadiiOnly && fx.use_lod) {
             gated = !lod_keeps(fx.lod, fx.log2_fork, i, x, y, z, f.campos);
             if (fx.lod_mask) fx.lod_mask[i] = gated ? 0 : 1;
@@ -208,11 +214,11 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
             for (int k = 0; k < 6; ++k) cov[k] = g.cov3D_precomp[6 * (size_t)i + k];
         } else {
 #pragma unroll
-            for (int k = 0; k < 3; ++k) scale[k] = g.scales[(kRadiiOnly ? fx.scale_stride : 3) * (size_t)i + k];
+            for (int k = 0; k < 3; ++k) scale[k] = GEO_LOAD(g.scales[(kRadiiOnly ? fx.scale_stride : 3) * (size_t)i + k]);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) quat[k] = g.rotations[4 * (size_t)i + k];
+            for (int k = 0; k < 4; ++k) quat[k] = GEO_LOAD(g.rotations[4 * (size_t)i + k]);
         }
-        if (!kRadiiOnly) opacity = g.opacities[i];
+        if (!kRadiiOnly) opacity = GEO_LOAD(g.opacities[i]);
     }
     if (valid && !gated) do {
         const float vx = ((V[0] * x + V[4] * y) + V[8] * z) + V[12];
@@ -275,13 +281,13 @@ __global__ __launch_bounds__(256) void preprocess_kernel(FrameArgs f, gs355_gaus
         qz = ca * det_inv;
     } while (false);
 
-    if (valid && radii) radii[i] = radius;
+    if (valid && radii) __builtin_nontemporal_store(radius, &radii[i]);  // (no later stage reads radii)
     if (kRadiiOnly) {
         if (valid && fx.visible) fx.visible[i] = radius > 0 ? 1 : 0;
         return;
     }
     if (valid) {
-        tiles_touched[i] = touched;
+        __builtin_nontemporal_store(touched, &tiles_touched[i]);  // (read by the classic scan and the backward pass only)
         rects[i] = rect_packed;
     }
     const bool alive = radius > 0;

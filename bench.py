@@ -635,11 +635,12 @@ def bench_scaffold(args, torch, dev):
         dec_ms, dec = timed(lambda: model.anchor_decoder(**dec_args))
         # the same call with weights that fp16 cannot represent (an fp32-trained checkpoint): the decoder then carries
         # them as hi + lo fp16 pairs (more matrix instructions, the low parts in LDS, three wavefronts per workgroup)
-        import copy
-        general = copy.deepcopy(model.anchor_decoder)
+        src = model.anchor_decoder
+        general = type(src)(src.use_feat_bank, src.add_opacity_dist, src.add_color_dist, src.add_cov_dist, src.view_dim,
+                            src.feat_dim, src.n_offsets).to(dev).eval()
         gen = torch.Generator().manual_seed(7)
-        for prm in general.parameters():
-            prm.mul_(1.0 + 1e-3 * torch.randn(prm.shape, generator=gen).to(dev))
+        for prm, given in zip(general.parameters(), src.parameters()):
+            prm.copy_(given * (1.0 + 1e-3 * torch.randn(prm.shape, generator=gen).to(dev)))
         dec32_ms, _ = timed(lambda: general(**dec_args))
         del general
     xyz, color, opacity, scaling, rot = dec[:5]

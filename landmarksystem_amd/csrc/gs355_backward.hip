@@ -60,31 +60,34 @@ struct PixelGrad {
 // blended its pair; otherwise lane s < 10 of each row returns in `sum` the row's total of accumulator s:
 // the moments of dL/dpower over the pixel offsets (dpow dx, dpow dy, dpow dx^2, dpow dx dy, dpow dy^2),
 // dL/dopacity, dL/d(r, g, b, depth).  T carries the forward blend's state (sign = finished).
-// b.y is log2(opacity) and `inv_opacity` its reciprocal: opacity * exp(power) is evaluated exactly as the forward
-// blend evaluates it (one multiply-add into the hardware exp2), so both passes take the same decisions.
+// b.y is log2(opacity): opacity * exp(power) is evaluated exactly as the forward blend evaluates it (one multiply-add
+// into the hardware exp2, decided on the exponent before the exp2), so both passes take the same decisions.  The
+// opacity's accumulator receives sum(dL/dpower) = opacity * dL/dopacity; the caller divides once per Gaussian.
 __device__ __forceinline__ bool backward_one(float& T, float& prefix, const PixelGrad& pg, float pxf, float pyf,
-                                             const float4 a, const float4 b, const float4 c, float inv_opacity,
-                                             bool enabled, int sub, float& sum)
+                                             const float4 a, const float4 b, const float4 c, bool enabled, int sub,
+                                             float& sum)
 {
     const float dx = a.x - pxf, dy = a.y - pyf;
     const float power = pair_exponent(dx, dy, a.z, a.w, b.x);  // a.z, a.w, b.x = -conic_x / 2, -conic_y, -conic_z / 2
-    const float raw = __builtin_amdgcn_exp2f(__builtin_fmaf(power, 1.4426950408889634f, b.y));  // opacity * exp(power)
+    const float t = __builtin_fmaf(power, 1.4426950408889634f, b.y);
+    const bool accept = enabled && !(power > 0.0f || t < kAlphaCut);  // the forward blend's decision, on the exponent
+    if (__ballot(accept) == 0ull) return false;
+    const float raw = __builtin_amdgcn_exp2f(t);  // opacity * exp(power)
     const float alpha = fminf(0.99f, raw);
-    const bool accept = enabled && !(power > 0.0f || alpha < 1.0f / 255.0f);
     const float test_T = __builtin_fmaf(-alpha, T, T);  // T - alpha T, as the forward blend forms it
     const bool hit = accept && test_T >= 0.0001f;
     if (accept && !hit && T > 0.0f) T = -T;
     if (__ballot(hit) == 0ull) return false;
-    float w = 0.0f, dpow = 0.0f, dop = 0.0f;
+    float w = 0.0f, dpow = 0.0f;
     if (hit) {
         w = alpha * T;
         const float fg = b.z * pg.g0 + b.w * pg.g1 + c.x * pg.g2 + c.y * pg.g3;
         prefix += w * fg;
         const float dalpha = T * fg - (pg.R - prefix) * __builtin_amdgcn_rcpf(1.0f - alpha);
         dpow = raw * dalpha;  // the gradient passes through min(0.99, .) unchanged
-        dop = dpow * inv_opacity;
         T = test_T;
     }
+    const float dop = dpow;  // (times 1 / opacity, once per Gaussian, when the batch's sums are turned into records)
     const float mx = dpow * dx, my = dpow * dy;
     // ten sums over the row's 16 lanes, transposed as they are reduced: after the exchanges inside lane pairs and
     // quads a lane holds one of four (then two) values, the quads' partial sums are rotated together, and lane s
@@ -210,8 +213,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
                 const uint32_t kk = k_next;
                 k_next = mine[i + 1];
                 float sum;
-                if (backward_one(T, prefix, pg, pxf, pyf, s_a[kk], s_b[kk], s_c[kk], s_inv_opacity[kk], i < my_len, sub,
-                                 sum)) {
+                if (backward_one(T, prefix, pg, pxf, pyf, s_a[kk], s_b[kk], s_c[kk], i < my_len, sub, sum)) {
                     // lane s of each row adds accumulator s of the row's Gaussian
                     if (sub < 10 && i < my_len && sum != 0.0f) atomicAdd(&s_grad[kk * kGradFloats + sub], sum);
                 }
@@ -227,7 +229,8 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
             float4* __restrict__ dst = reinterpret_cast<float4*>(key_grads + (size_t)slot * kKeyFloats);
             // d power / d centre = -(conic_x dx + conic_y dy, conic_z dy + conic_y dx), with conic_x = -2 a.z etc.
             dst[0] = make_float4(2.0f * a.z * m[0] + a.w * m[1], 2.0f * hz * m[1] + a.w * m[0], -0.5f * m[2], -m[3]);
-            dst[1] = make_float4(-0.5f * m[4], m[5], m[6], m[7]);
+            // m[5] = sum of opacity * dL/dopacity over the tile's pixels (zero, not 0 * inf, for a Gaussian that never blended)
+            dst[1] = make_float4(-0.5f * m[4], m[5] != 0.0f ? m[5] * s_inv_opacity[tid] : 0.0f, m[6], m[7]);
             dst[2] = make_float4(m[8], m[9], 0.f, 0.f);
         }
     }

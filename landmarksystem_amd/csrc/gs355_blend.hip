@@ -68,12 +68,6 @@ struct PixelState {
     float T, c0, c1, c2, depth;
 };
 
-// The hardware exp2 is monotone, so exp2(t) < 1/255 exactly when t < kAlphaCut, the smallest float whose exp2 reaches
-// 1/255 (found by running v_exp_f32 over every float between -8.2 and -7.8).  The shipped blend decides on t and
-// leaves the exp2 (a quarter-rate instruction) to the pairs that pass; the verification variant decides on the
-// exponential itself, and the tests hold the two to identical images on scenes full of opacities around 1/255.
-constexpr float kAlphaCut = -7.99435329f;  // bits 0xc0ffd1be
-
 // a = px, py, hx, ny;  b = hz, log2(opacity), r, g;  rec_c + entry = b, depth (read only by pixels that accept)
 template <bool kCutOnExponent>
 __device__ __forceinline__ void blend_one(PixelState& p, float pxf, float pyf, const float4 a, const float4 b,

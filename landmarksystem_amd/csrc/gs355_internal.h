@@ -95,6 +95,13 @@ __device__ __forceinline__ float pair_exponent(float dx, float dy, float hx, flo
     return __builtin_fmaf(dx, v, z);
 }
 
+// The hardware exp2 is monotone, so exp2(t) < 1/255 exactly when t < kAlphaCut, the smallest float whose exp2 reaches
+// 1/255 (found by running v_exp_f32 over every float between -8.2 and -7.8).  The blend (forward and backward) decides
+// on t = power * log2(e) + log2(opacity) and leaves the exp2 (a quarter-rate instruction) to the pairs that pass; the
+// forward blend's verification variant decides on the exponential itself, and the tests hold the two to identical
+// images on scenes full of opacities around 1/255.
+constexpr float kAlphaCut = -7.99435329f;  // bits 0xc0ffd1be
+
 // stage launchers (each returns a gs355_status)
 int launch_preprocess(const FrameArgs& f, const gs355_gaussians& g, bool radii_only, float* records,
                       uint32_t* tiles_touched, uint64_t* rects, uint32_t* depth_bits, int32_t* radii, hipStream_t s);

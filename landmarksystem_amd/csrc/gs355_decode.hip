@@ -234,11 +234,11 @@ constexpr int kRun = 128;
 
 // kSplit: the features enter as hi + lo fp16 pairs (general fp32 features; two more matrix instructions per head).
 // kWLo: so do the weights (general fp32 weights; their low fragments take 19 KB of LDS in the emit pass, which
-// then runs three wavefronts per workgroup so that two workgroups still share a CU).
+// then runs three wavefronts per workgroup so that two workgroups still share a CU, held to 256 registers).
 constexpr int decode_waves(bool count_only, bool weights_lo) { return (weights_lo && !count_only) ? 3 : 4; }
 
 template <bool kCountOnly, bool kSplit, bool kWLo>
-__global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo))) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
+__global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kCountOnly ? 2 : 1)) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
                                                      const uint32_t* __restrict__ offsets, uint32_t capacity,
                                                      float* __restrict__ xyz, float* __restrict__ color,
                                                      float* __restrict__ opacity, float* __restrict__ scaling_out,

@@ -14,11 +14,19 @@ Supported: the feature bank (`use_feat_bank`), the level input (`add_level`)
 and the training-mode by-products (`neural_opacity`, `mask`); not the
 appearance embedding (`appearance_dim > 0`: the reference's own branch
 concatenates a 1-D integer tensor to the 2-D input, anchor_decoder.py:204-211,
-and cannot run as written).  Forward only.  All arithmetic runs in the HIP
+and cannot run as written).  Without gradients all arithmetic runs in the HIP
 kernels behind `gs355_decode`: one call enqueues the whole decode and the
 number of Gaussians stays on the device; `forward` waits for that one number
 (the reference's boolean-mask indexing synchronises at the same place) only to
 give its results their exact shapes, `decode_on_device` never waits.
+
+In training mode with gradients enabled and something to differentiate (a
+parameter or an input that requires grad: the training loops of benchmarks/nerf/scaffold_gs and
+octree_gs), `forward` evaluates the module's own statements
+(anchor_decoder.py:147-242) as torch operations on the GPU, so autograd
+reaches the MLPs, the features, the offsets and the scales -- as in the
+reference, whose fused decoder is an inference component and whose training
+runs the torch module.  The rasterizer behind it differentiates in HIP.
 """
 import ctypes as C
 from collections import OrderedDict
@@ -238,9 +246,46 @@ class FusedAnchorDecoder(nn.Module):
         torch.cuda.current_stream(counts.device).synchronize()
         return int(self._host_count[0]), int(self._host_count[1])
 
-    @torch.no_grad()
     def forward(self, camera_center, anchor, anchor_feat, offset, scaling, visible_mask=None, level=None,
                 prog_ratio=None, transition_mask=None, appearance_code=None):
+        if self.dist2level == "progressive" and prog_ratio is not None and transition_mask is not None:
+            raise NotImplementedError("progressive level-of-detail opacity scaling is not part of this decoder")
+        if self.training and torch.is_grad_enabled() and (any(p.requires_grad for p in self.parameters()) or any(
+                torch.is_tensor(t) and t.requires_grad for t in (anchor, anchor_feat, offset, scaling))):
+            return self._forward_differentiable(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, level)
+        with torch.no_grad():
+            return self._forward_kernels(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, level)
+
+    def _forward_differentiable(self, camera_center, anchor, anchor_feat, offset, scaling, visible_mask, level):
+        """The statements of the reference module (anchor_decoder.py:147-242) as torch operations, for autograd:
+        same 7-tuple, the training by-products always present."""
+        level = self._check_level(level, anchor.shape[0])
+        if visible_mask is None:
+            visible_mask = torch.ones(anchor.shape[0], dtype=torch.bool, device=anchor.device)
+        a, feat, off, sc = anchor[visible_mask], anchor_feat[visible_mask], offset[visible_mask], scaling[visible_mask]
+        view = a - camera_center.to(a.device)
+        dist = view.norm(dim=1, keepdim=True)
+        view = view / dist
+        lvl = level.reshape(-1, 1)[visible_mask].to(feat.dtype) if level is not None else None
+        if self.use_feat_bank:
+            w = self.mlp_feature_bank(view if lvl is None else torch.cat([view, lvl], dim=1))  # softmax inside
+            feat = feat[:, ::4].repeat(1, 4) * w[:, 0:1] + feat[:, ::2].repeat(1, 2) * w[:, 1:2] + feat * w[:, 2:3]
+        if lvl is not None:  # (:181-182: both inputs become [feat | view | level])
+            with_dist = without = torch.cat([feat, view, lvl], dim=1)
+        else:
+            with_dist, without = torch.cat([feat, view, dist], dim=1), torch.cat([feat, view], dim=1)
+        n = self.n_offsets
+        neural_opacity = self.mlp_opacity(with_dist if self.add_opacity_dist else without).reshape(-1, 1)
+        mask = (neural_opacity > 0.0).view(-1)
+        color = self.mlp_color(with_dist if self.add_color_dist else without).reshape(-1, 3)[mask]
+        cov = self.mlp_cov(with_dist if self.add_cov_dist else without).reshape(-1, 7)[mask]
+        owner = torch.arange(a.shape[0], device=a.device).repeat_interleave(n)[mask]  # anchor of each kept offset
+        scaling_out = sc[owner, 3:6] * torch.sigmoid(cov[:, 0:3])
+        rot = torch.nn.functional.normalize(cov[:, 3:7])
+        xyz = a[owner] + off.reshape(-1, 3)[mask] * sc[owner, 0:3]
+        return xyz, color, neural_opacity[mask], scaling_out, rot, neural_opacity, mask
+
+    def _forward_kernels(self, camera_center, anchor, anchor_feat, offset, scaling, visible_mask=None, level=None):
         """Returns (xyz[G,3], color[G,3], opacity[G,1], scaling[G,3], rot[G,4], neural_opacity, mask): the neural
         Gaussians of the visible anchors whose decoded opacity is positive, in boolean-mask order; in training mode
         also the opacity of every offset of the visible anchors ([A_vis * n, 1]) and the mask over them, else None.
@@ -248,8 +293,6 @@ class FusedAnchorDecoder(nn.Module):
         The output shapes depend on the data, so the count phase runs first and its two counters are read back
         (the reference's boolean-mask indexing synchronises at the same place); the emit phase then writes into
         tensors of exactly that size."""
-        if self.dist2level == "progressive" and prog_ratio is not None and transition_mask is not None:
-            raise NotImplementedError("progressive level-of-detail opacity scaling is not part of this decoder")
         dev, A, dec, an, tensors = self._marshal(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, level)
         # the two counters go straight into pinned host memory (which the GPU addresses like its own): no copy is
         # enqueued, the host waits for the count phase and reads them

@@ -497,8 +497,40 @@ class ScaffoldGS(nn.Module):
     def _decoder_level(self):
         return None  # Scaffold-GS anchors carry no level
 
-    @torch.no_grad()
     def forward(self, viewpoint_camera, scaling_modifier=1.0, retain_grad=False, render_exclude_filter=None):
+        """scaffold_gs/gs_model.py:162-238 (octree_gs/gs_model.py:228-325).  Under torch.no_grad() or in eval mode:
+        the frame.  In training mode with gradients enabled: `(rendered_image, scaling)` as the reference returns
+        them, differentiable with respect to the anchors' parameters and the decoder's MLPs, with
+        `viewspace_points`, `offset_selection_mask` and `opacity` left on the model for its densification."""
+        if self.training and torch.is_grad_enabled():
+            return self._forward_training(viewpoint_camera, scaling_modifier, retain_grad, render_exclude_filter)
+        with torch.no_grad():
+            return self._forward_frame(viewpoint_camera, scaling_modifier, render_exclude_filter)
+
+    def _forward_training(self, viewpoint_camera, scaling_modifier, retain_grad, render_exclude_filter):
+        viewpoint_camera = viewpoint_camera.to(self._anchor.device)
+        with torch.no_grad():  # (the visibility tests are not differentiated)
+            self._before_prefilter(viewpoint_camera)
+            voxel_visible_mask = self.prefilter_voxel(viewpoint_camera)
+            if render_exclude_filter is not None:
+                voxel_visible_mask = voxel_visible_mask & render_exclude_filter
+        xyz, color, opacity, scaling, rot, neural_opacity, mask = self.anchor_decoder(
+            camera_center=viewpoint_camera.camera_center, anchor=self.get_anchor, anchor_feat=self.get_anchor_feat,
+            offset=self.get_offset, scaling=self.get_scaling, visible_mask=voxel_visible_mask,
+            level=self._decoder_level())
+        screenspace_points = torch.zeros_like(xyz, requires_grad=True) + 0
+        if retain_grad:
+            screenspace_points.retain_grad()
+        self.renderer.raster_settings = _settings(viewpoint_camera, self.background, scaling_modifier, 1)
+        rendered_image, radii, _ = self.renderer(
+            means3D=xyz, means2D=screenspace_points, shs=None, colors_precomp=color, opacities=opacity, scales=scaling,
+            rotations=rot, cov3D_precomp=None)
+        self.viewspace_points = screenspace_points
+        self.visibility_filter, self.voxel_visible_mask = radii > 0, voxel_visible_mask
+        self.offset_selection_mask, self.opacity = mask, neural_opacity
+        return rendered_image, scaling
+
+    def _forward_frame(self, viewpoint_camera, scaling_modifier=1.0, render_exclude_filter=None):
         viewpoint_camera = viewpoint_camera.to(self._anchor.device)
         self._before_prefilter(viewpoint_camera)
         voxel_visible_mask = self.prefilter_voxel(viewpoint_camera)
@@ -565,7 +597,7 @@ class OctreeGS(ScaffoldGS):
             self._anchor_mask = torch.ones(self._level.shape[0], dtype=torch.bool, device=self._level.device)
             return
         anchor_pos = self._anchor + (self.voxel_size / 2) / (float(self.fork) ** self._level)
-        dist = torch.sqrt(torch.sum((anchor_pos - cam_center) ** 2, dim=1)) * resolution_scale
+        dist = torch.sqrt(torch.sum((anchor_pos - cam_center.to(anchor_pos.device)) ** 2, dim=1)) * resolution_scale
         pred_level = torch.log2(self.standard_dist / dist) / math.log2(self.fork) + self._extra_level
         max_level = self._level_span_value()
         if self.dist2level == "floor":

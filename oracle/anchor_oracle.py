@@ -47,22 +47,25 @@ def bank_mix(feat, weights):
 
 
 def decode(camera_center, anchor, anchor_feat, offset, scaling, visible_mask, mlps, n_offsets=10,
-           add_dist=(True, True, True), keep_override=None, level=None, add_level=False, bank=None):
+           add_dist=(True, True, True), keep_override=None, level=None, add_level=False, bank=None,
+           dtype=torch.float32):
     """mlps: {"opacity"|"cov"|"color": (W0[32,in], b0[32], W1[k,32], b1[k])}.
     Returns xyz[G,3], color[G,3], opacity[G,1], scaling[G,3], rot[G,4] and the
     flat keep mask over (visible anchor, offset).  `keep_override` (flat bool
     over (visible anchor, offset)) replaces the mask opacity > 0: tests use it
     to obtain the values of offsets whose opacity is within rounding of zero.
     `level` [A] or [A,1] with `add_level`: every head reads [feat | view | level].
-    `bank` = (W0[32,3 or 4], b0[32], W1[3,32], b1[3]) of mlp_feature_bank."""
+    `bank` = (W0[32,3 or 4], b0[32], W1[3,32], b1[3]) of mlp_feature_bank.
+    `dtype`: torch.float64 evaluates the same statements in double precision (inputs that require grad keep their
+    graph: the reference for the gradients of the training path)."""
     if visible_mask is None:
         visible_mask = torch.ones(anchor.shape[0], dtype=torch.bool)
-    a = anchor[visible_mask].float()
-    feat = anchor_feat[visible_mask].float()
-    off = offset[visible_mask].float()
-    sc = scaling[visible_mask].float()
-    lvl = level.reshape(-1, 1)[visible_mask].float() if (add_level and level is not None) else None
-    view = a - camera_center.float()
+    a = anchor[visible_mask].to(dtype)
+    feat = anchor_feat[visible_mask].to(dtype)
+    off = offset[visible_mask].to(dtype)
+    sc = scaling[visible_mask].to(dtype)
+    lvl = level.reshape(-1, 1)[visible_mask].to(dtype) if (add_level and level is not None) else None
+    view = a - camera_center.to(dtype)
     dist = view.norm(dim=1, keepdim=True)
     view = view / dist
     if bank is not None:

@@ -234,14 +234,15 @@ def test_level_input_follows_the_reference_quirks(gpu_device):
 
 def test_training_mode_returns_every_opacity_and_the_mask(gpu_device):
     """anchor_decoder.py:239-242: in training mode the 7-tuple also carries the opacity of every offset of the
-    visible anchors and the mask that selected the Gaussians."""
+    visible anchors and the mask that selected the Gaussians (here from the kernels: no gradients asked for)."""
     A = 9000
     sc = scenes.config5(A=A)
     dec = build_decoder(sc, gpu_device).train()
     vis = torch.rand(A, generator=torch.Generator().manual_seed(4)) < 0.5
     cam = sc.camera.camera_center
-    out = dec(cam.to(gpu_device), sc.anchor.to(gpu_device), sc.anchor_feat.to(gpu_device), sc.offset.to(gpu_device),
-              sc.scaling.to(gpu_device), vis.to(gpu_device))
+    with torch.no_grad():
+        out = dec(cam.to(gpu_device), sc.anchor.to(gpu_device), sc.anchor_feat.to(gpu_device),
+                  sc.offset.to(gpu_device), sc.scaling.to(gpu_device), vis.to(gpu_device))
     ref = ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp, sc.n_offsets)
     neural_opacity, mask = out[5], out[6]
     a_vis = int(vis.sum())

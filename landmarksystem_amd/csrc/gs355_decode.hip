@@ -73,6 +73,24 @@ struct DecodeArgs {
     uint8_t* kept_mask;      // [A_vis * n] pre-activation > 0, or NULL
 };
 
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+// Eight floats as hi + lo fp16 pairs (hi = the value rounded to fp16, lo = what that rounding left over, rounded
+// to fp16), converted two at a time (one packed conversion per pair and direction).
+__device__ __forceinline__ void split_half8(const float v[8], half8_t& hi, half8_t& lo)
+{
+    half2_t h[4], l[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float2_t x = {v[2 * j], v[2 * j + 1]};
+        h[j] = __builtin_convertvector(x, half2_t);
+        l[j] = __builtin_convertvector(x - __builtin_convertvector(h[j], float2_t), half2_t);
+    }
+    hi = (half8_t){h[0][0], h[0][1], h[1][0], h[1][1], h[2][0], h[2][1], h[3][0], h[3][1]};
+    lo = (half8_t){l[0][0], l[0][1], l[1][0], l[1][1], l[2][0], l[2][1], l[3][0], l[3][1]};
+}
+
 __device__ __forceinline__ half8_t to_half8(const float v[8])
 {
     half8_t h;
@@ -146,10 +164,10 @@ __device__ __forceinline__ void load_head(const DecodeArgs& d, int head, int out
 // one copy; `store_head_lo` is called by one wavefront per head.
 template <int kTiles>
 __device__ __forceinline__ void store_head_lo(const DecodeArgs& d, int head, int outputs, int row, int half, int lane,
-                                              half8_t (*dst)[64])
+                                              half8_t (*dst)[64], bool lo = true)
 {
     HeadWeights<kTiles> w;
-    load_head<kTiles>(d, head, outputs, row, half, w, true);
+    load_head<kTiles>(d, head, outputs, row, half, w, lo);
 #pragma unroll
     for (int s = 0; s < 3; ++s) dst[s][lane] = w.w0[s];
 #pragma unroll
@@ -158,21 +176,47 @@ __device__ __forceinline__ void store_head_lo(const DecodeArgs& d, int head, int
         for (int s = 0; s < 2; ++s) dst[3 + 2 * r + s][lane] = w.w1[r][s];
 }
 
-// One head for one tile of 32 anchors: returns up to kTiles accumulators of the
-// second layer (rows = outputs 32r + 8b + 4*half + t, column = this lane's anchor).
+// Store an accumulator's rows into the anchor's LDS row, head outputs at `base`.  Rows that do not exist
+// (>= outputs; their accumulators hold zeros: masked weights, zero bias) are stored too, all of them at row
+// `outputs` -- the first word after the head, which the stores that follow in program order overwrite (the next
+// head's first output, or the anchor's scaling) -- so that no store is predicated: 16 conditional stores cost five
+// instructions and a branch each.  A row tile that lies inside the head entirely takes constant offsets.
+__device__ __forceinline__ void store_rows(float* __restrict__ dst_anchor, int base, int outputs, int row0, int half,
+                                           const floatx16& c)
+{
+    float* __restrict__ dst = dst_anchor + base;
+    const int lane_row = row0 + 4 * half;
+    if (row0 + 32 <= outputs) {  // uniform
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[lane_row + 8 * (v >> 2) + (v & 3)] = c[v];
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[min(lane_row + 8 * (v >> 2) + (v & 3), outputs)] = c[v];
+    }
+}
+
+// One head for one tile of 32 anchors: the kTiles accumulators of the second layer (rows = outputs
+// 32r + 8b + 4*half + t, column = this lane's anchor) go to the anchor's LDS row as soon as each is complete
+// (one accumulator live at a time).
 // `wlo`: the head's low weight fragments in LDS (kWLo), read right before their matrix instruction.
-template <int kTiles, bool kSplit, bool kWLo>
-__device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const half8_t (*wlo)[64], int lane,
+// kWInLds: the weight fragments themselves are read from `whi` (same order as `wlo`) instead of `w`: the
+// covariance head's nine fragments would otherwise hold 36 registers for the whole kernel.
+template <int kTiles, bool kSplit, bool kWLo, bool kWInLds = false>
+__device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const half8_t (*whi)[64],
+                                         const half8_t (*wlo)[64], int lane,
                                          const float* bias0, const float* bias1, const half8_t X[kSplit ? 5 : 3],
-                                         int half, floatx16 out[kTiles])
+                                         int half, float* __restrict__ dst_anchor, int base, int outputs)
 {
     // layer 1: hidden = W0 [32 x in] * X^T + b0  (X[3], X[4]: the low parts of features that fp16 cannot hold)
     floatx16 h = bias_rows(bias0, 0, half);
+    half8_t w0[3];
 #pragma unroll
-    for (int s = 0; s < 3; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w0[s], X[s], h, 0, 0, 0);
+    for (int s = 0; s < 3; ++s) w0[s] = kWInLds ? whi[s][lane] : w.w0[s];
+#pragma unroll
+    for (int s = 0; s < 3; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(w0[s], X[s], h, 0, 0, 0);
     if constexpr (kSplit) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w0[s], X[3 + s], h, 0, 0, 0);
+        for (int s = 0; s < 2; ++s) h = __builtin_amdgcn_mfma_f32_32x32x16_f16(w0[s], X[3 + s], h, 0, 0, 0);
     }
     if constexpr (kWLo) {  // low parts of the weights against the high parts of the inputs
 #pragma unroll
@@ -182,15 +226,10 @@ __device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const hal
     half8_t hh[2], hl[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-        float r[8], lo[8];
+        float r[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            r[j] = fmaxf(h[8 * s + j], 0.0f);
-            const _Float16 top = (_Float16)r[j];
-            lo[j] = r[j] - (float)top;
-        }
-        hh[s] = to_half8(r);
-        hl[s] = to_half8(lo);
+        for (int j = 0; j < 8; ++j) r[j] = __builtin_amdgcn_fmed3f(h[8 * s + j], 0.0f, __builtin_inff());  // ReLU in one instruction
+        split_half8(r, hh[s], hl[s]);
     }
     // layer 2: out = W1 [outputs x 32] * hidden + b1
 #pragma unroll
@@ -198,23 +237,20 @@ __device__ __forceinline__ void run_head(const HeadWeights<kTiles>& w, const hal
         floatx16 c = bias_rows(bias1, 32 * r, half);
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w1[r][s], hh[s], c, 0, 0, 0);
-            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(w.w1[r][s], hl[s], c, 0, 0, 0);
+            const half8_t w1 = kWInLds ? whi[3 + 2 * r + s][lane] : w.w1[r][s];
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(w1, hh[s], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(w1, hl[s], c, 0, 0, 0);
             if constexpr (kWLo) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[3 + 2 * r + s][lane], hh[s], c, 0, 0, 0);
         }
-        out[r] = c;
+        store_rows(dst_anchor, base, outputs, 32 * r, half, c);
     }
 }
 
-// Store the rows of an accumulator that exist (< outputs) into the tile's LDS block.
-__device__ __forceinline__ void store_rows(float* __restrict__ dst_anchor, int base, int outputs, int row0, int half,
-                                           const floatx16& c)
+// 1 / (1 + exp(-x)) from the hardware exp2 and reciprocal (each within 1 ulp; the product x log2(e) adds
+// |x| 2^-24 to the exponent): relative error below 1e-6 for any x, against the 3e-5 the decode is held to.
+__device__ __forceinline__ float fast_sigmoid(float x)
 {
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int r = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
-        if (r < outputs) dst_anchor[base + r] = c[v];
-    }
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
 }
 
 // Per-lane inputs of one tile of 32 anchors.
@@ -238,7 +274,7 @@ constexpr int kRun = 128;
 constexpr int decode_waves(bool count_only, bool weights_lo) { return (weights_lo && !count_only) ? 3 : 4; }
 
 template <bool kCountOnly, bool kSplit, bool kWLo>
-__global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kCountOnly ? 2 : 1)) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
+__global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (!kCountOnly ? 2 : 1)) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
                                                      const uint32_t* __restrict__ offsets, uint32_t capacity,
                                                      float* __restrict__ xyz, float* __restrict__ color,
                                                      float* __restrict__ opacity, float* __restrict__ scaling_out,
@@ -256,6 +292,8 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
     __shared__ float s_bias[256];
     // low parts of the weight fragments: opacity head 0..4, covariance 5..13, colour 14..18
     __shared__ half8_t s_wlo[kWLo ? (kCountOnly ? 5 : 19) : 1][64];
+    // the covariance head's weight fragments (emit pass): read from here right before their matrix instruction
+    __shared__ half8_t s_wcov[kCountOnly ? 1 : 9][64];
 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
     const int n = d.n;
@@ -274,15 +312,15 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
             if (wave == 2) store_head_lo<1>(d, 2, 3 * n, col, half, lane, s_wlo + 14);
         }
     }
+    if constexpr (!kCountOnly) {
+        if (wave == kWaves - 1) store_head_lo<3>(d, 1, 7 * n, col, half, lane, s_wcov, false);
+    }
     __syncthreads();
     HeadWeights<1> w_op;
     load_head<1>(d, 0, n, col, half, w_op);
-    HeadWeights<3> w_cov;
+    HeadWeights<3> w_cov = {};  // unused: read from s_wcov
     HeadWeights<1> w_col;
-    if (!kCountOnly) {
-        load_head<3>(d, 1, 7 * n, col, half, w_cov);
-        load_head<1>(d, 2, 3 * n, col, half, w_col);
-    }
+    if (!kCountOnly) load_head<1>(d, 2, 3 * n, col, half, w_col);
     const int stride = kCountOnly ? 11 : 11 * n + 13;
     const int items = 32 * n;  // (anchor, offset) pairs of a tile: item = anchor_in_tile * n + offset
     const int inv_n = (65536 + n - 1) / n;  // item / n == (item * inv_n) >> 16 for item < 32 n, n <= 10
@@ -323,9 +361,12 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
         const bool vis = first + col < nvis;  // lanes l and l+32 share entry first + l
         const int a = vis ? base + (int)run_list[first + col] : 0;
         const uint64_t any = __ballot(vis);  // bits l and l + 32 belong to entry l of the tile
-        // Everything the tile needs from global memory is requested here, before the first use.
+        // Everything the tile needs from global memory is requested here, before the first use, and without a
+        // condition: a lane without an anchor (or an item without one) reads anchor 0's data, which nothing uses
+        // (matrix columns are independent, and only items of visible anchors are ever emitted) -- conditional
+        // loads would each become a branch, and the values' first use would wait inside the condition.
         TileInputs<kCountOnly> in;
-        if (vis) {
+        {
             const float4* __restrict__ f4 = reinterpret_cast<const float4*>(d.feat + (size_t)a * kFeat);
 #pragma unroll
             for (int s = 0; s < 2; ++s) {  // features 16s + 8*half .. +7
@@ -338,21 +379,23 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
         }
         if constexpr (!kCountOnly) {
             // half 0: scaling[0..2] (offset scale), half 1: scaling[3..5] (Gaussian scale)
-            if (vis) {
 #pragma unroll
-                for (int k = 0; k < 3; ++k) in.sc3[k] = d.scaling[6 * (size_t)a + 3 * half + k];
-            }
-            if (vis && offsets) in.first_slot = offsets[a];  // entry 0's value is the tile's first output slot
+            for (int k = 0; k < 3; ++k) in.sc3[k] = d.scaling[6 * (size_t)a + 3 * half + k];
+            if (offsets) in.first_slot = offsets[a];  // entry 0's value is the tile's first output slot
             // the learned offsets of the items this lane's position covers (item = entry * n + offset)
+            int item_anchor[5], item_offset[5];
 #pragma unroll
             for (int r = 0; r < 5; ++r) {
-                const int it = r * 64 + lane;
+                const int it = min(r * 64 + lane, items - 1);
                 const int al = (it * inv_n) >> 16;
-                const bool want = it < items && ((any >> al) & 1ull);
-                const int ai = want ? base + (int)run_list[first + al] : 0;
-                const float* __restrict__ of = d.offset + ((size_t)ai * n + (want ? it - al * n : 0)) * 3;
+                item_offset[r] = it - al * n;
+                item_anchor[r] = (int)run_list[min(first + al, nvis - 1)];
+            }
 #pragma unroll
-                for (int k = 0; k < 3; ++k) in.ofv[r][k] = want ? of[k] : 0.0f;
+            for (int r = 0; r < 5; ++r) {
+                const float* __restrict__ of = d.offset + ((size_t)(base + item_anchor[r]) * n + item_offset[r]) * 3;
+#pragma unroll
+                for (int k = 0; k < 3; ++k) in.ofv[r][k] = of[k];
             }
         }
         // B operand: X^T, column = anchor; slots as described at HeadWeights
@@ -364,12 +407,8 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
             for (int s = 0; s < 2; ++s) {
                 x8[0] = in.f[2 * s].x, x8[1] = in.f[2 * s].y, x8[2] = in.f[2 * s].z, x8[3] = in.f[2 * s].w;
                 x8[4] = in.f[2 * s + 1].x, x8[5] = in.f[2 * s + 1].y, x8[6] = in.f[2 * s + 1].z, x8[7] = in.f[2 * s + 1].w;
-                X[s] = to_half8(x8);  // all zero for an invisible anchor
-                if constexpr (kSplit) {  // what the fp16 rounding left over, as a second operand
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) x8[j] -= (float)X[s][j];
-                    X[3 + s] = to_half8(x8);
-                }
+                if constexpr (kSplit) split_half8(x8, X[s], X[3 + s]);  // the second: what the fp16 rounding left over
+                else X[s] = to_half8(x8);                               // all zero for an invisible anchor
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) x8[j] = 0.0f;
@@ -393,11 +432,7 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
         // ---- opacity head ----
         // the mask opacity > 0 is the sign of the pre-activation (tanh is odd, monotone and tanh(x) = x for the
         // smallest floats), so tanh itself is only evaluated for the offsets that are kept
-        {
-            floatx16 op[1];
-            run_head<1, kSplit, kWLo>(w_op, s_wlo, lane, s_bias, s_bias + 96, X, half, op);
-            store_rows(mine + col * stride, 0, n, 0, half, op[0]);
-        }
+        run_head<1, kSplit, kWLo>(w_op, nullptr, s_wlo, lane, s_bias, s_bias + 96, X, half, mine + col * stride, 0, n);
         if (kCountOnly) {
             wave_lds_sync();
             if (half == 0 && vis) {
@@ -411,13 +446,10 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
         }
 
         // ---- covariance and colour heads ----
-        floatx16 cv[3];
-        run_head<3, kSplit, kWLo>(w_cov, s_wlo + (kWLo ? 5 : 0), lane, s_bias + 32, s_bias + 128, X, half, cv);
-#pragma unroll
-        for (int r = 0; r < 3; ++r) store_rows(mine + col * stride, n, 7 * n, 32 * r, half, cv[r]);
-        floatx16 cl[1];
-        run_head<1, kSplit, kWLo>(w_col, s_wlo + (kWLo ? 14 : 0), lane, s_bias + 64, s_bias + 224, X, half, cl);
-        store_rows(mine + col * stride, 8 * n, 3 * n, 0, half, cl[0]);
+        run_head<3, kSplit, kWLo, true>(w_cov, s_wcov, s_wlo + (kWLo ? 5 : 0), lane, s_bias + 32, s_bias + 128, X, half,
+                                        mine + col * stride, n, 7 * n);
+        run_head<1, kSplit, kWLo>(w_col, nullptr, s_wlo + (kWLo ? 14 : 0), lane, s_bias + 64, s_bias + 224, X, half,
+                                  mine + col * stride, 8 * n, 3 * n);
         {
             float* __restrict__ extra = mine + col * stride + 11 * n;
 #pragma unroll
@@ -435,17 +467,21 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
         // activations below are the expensive part, so they run on dense wavefronts of survivors only ----
         uint16_t* __restrict__ list = reinterpret_cast<uint16_t*>(mine + 32 * stride);  // [32 n] item numbers
         uint32_t total = 0;
+        float pre[5];  // the items' opacity pre-activations, all requested before the first is looked at
+        bool exists[5];
+#pragma unroll
+        for (int r = 0; r < 5; ++r) {
+            const int it = min(r * 64 + lane, items - 1);
+            const int al = (it * inv_n) >> 16, m = it - al * n;
+            pre[r] = mine[al * stride + m];
+            exists[r] = r * 64 + lane < items && ((any >> al) & 1ull);
+        }
 #pragma unroll
         for (int r = 0; r < 5; ++r) {
             if (r * 64 >= items) break;  // uniform
-            const int it = r * 64 + lane;
-            bool kept = false;
-            if (it < items) {
-                const int al = (it * inv_n) >> 16, m = it - al * n;
-                kept = ((any >> al) & 1ull) && mine[al * stride + m] > 0.0f;
-            }
+            const bool kept = exists[r] && pre[r] > 0.0f;
             const uint64_t b = __ballot(kept);
-            if (kept) list[total + (uint32_t)__popcll(b & lanes_below)] = (uint16_t)it;
+            if (kept) list[total + (uint32_t)__popcll(b & lanes_below)] = (uint16_t)(r * 64 + lane);
             total += (uint32_t)__popcll(b);
         }
         wave_lds_sync();
@@ -495,16 +531,17 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (kWLo && !kC
             opacity[pos] = tanhf(o[m]);
 #pragma unroll
             for (int k = 0; k < 3; ++k) {
-                color[3 * (size_t)pos + k] = 1.0f / (1.0f + expf(-c3[k]));
-                scaling_out[3 * (size_t)pos + k] = extra[3 + k] * (1.0f / (1.0f + expf(-c7[k])));
+                color[3 * (size_t)pos + k] = fast_sigmoid(c3[k]);
+                scaling_out[3 * (size_t)pos + k] = extra[3 + k] * fast_sigmoid(c7[k]);
                 xyz[3 * (size_t)pos + k] = extra[6 + k] + off3[k] * extra[k];
             }
             const float q0 = c7[3], q1 = c7[4], q2 = c7[5], q3 = c7[6];
-            const float norm = fmaxf(sqrtf(q0 * q0 + q1 * q1 + q2 * q2 + q3 * q3), 1e-12f);
-            rot[4 * (size_t)pos + 0] = q0 / norm;
-            rot[4 * (size_t)pos + 1] = q1 / norm;
-            rot[4 * (size_t)pos + 2] = q2 / norm;
-            rot[4 * (size_t)pos + 3] = q3 / norm;
+            // q / max(|q|, 1e-12) with one reciprocal square root (1 ulp) instead of a root and four divisions
+            const float inv = __builtin_amdgcn_rsqf(fmaxf(q0 * q0 + q1 * q1 + q2 * q2 + q3 * q3, 1e-24f));
+            rot[4 * (size_t)pos + 0] = q0 * inv;
+            rot[4 * (size_t)pos + 1] = q1 * inv;
+            rot[4 * (size_t)pos + 2] = q2 * inv;
+            rot[4 * (size_t)pos + 3] = q3 * inv;
         }
         wave_lds_sync();
       }

@@ -274,7 +274,7 @@ constexpr int kRun = 128;
 constexpr int decode_waves(bool count_only, bool weights_lo) { return (weights_lo && !count_only) ? 3 : 4; }
 
 template <bool kCountOnly, bool kSplit, bool kWLo>
-__global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (!kCountOnly ? 2 : 1)) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
+__global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (!kCountOnly ? 2 : 4)) void decode_kernel(DecodeArgs d, uint32_t* __restrict__ counts,
                                                      const uint32_t* __restrict__ offsets, uint32_t capacity,
                                                      float* __restrict__ xyz, float* __restrict__ color,
                                                      float* __restrict__ opacity, float* __restrict__ scaling_out,
@@ -291,9 +291,14 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (!kCountOnly
     // biases of the three heads, zero-padded: b0 at [head*32], b1 of opacity / cov / colour at 96 / 128 / 224
     __shared__ float s_bias[256];
     // low parts of the weight fragments: opacity head 0..4, covariance 5..13, colour 14..18
-    __shared__ half8_t s_wlo[kWLo ? (kCountOnly ? 5 : 19) : 1][64];
-    // the covariance head's weight fragments (emit pass): read from here right before their matrix instruction
-    __shared__ half8_t s_wcov[kCountOnly ? 1 : 9][64];
+    __shared__ half8_t s_wlo[kWLo ? (kCountOnly ? 5 : 19) : 1][kWLo ? 64 : 1];
+    // the covariance head's weight fragments (0..8) and, where LDS has room for them beside the low parts, the
+    // colour head's (9..13), for the emit pass: read from here right before their matrix instruction instead of
+    // holding 36 + 20 registers for the whole kernel
+    constexpr bool kColourInLds = !kCountOnly && !kWLo;
+    __shared__ half8_t s_whi[kCountOnly ? 1 : (kColourInLds ? 14 : 9)][kCountOnly ? 1 : 64];
+    const half8_t (*const whi)[64] = reinterpret_cast<const half8_t (*)[64]>(s_whi);
+    const half8_t (*const wlo)[64] = reinterpret_cast<const half8_t (*)[64]>(s_wlo);
 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
     const int n = d.n;
@@ -313,14 +318,17 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (!kCountOnly
         }
     }
     if constexpr (!kCountOnly) {
-        if (wave == kWaves - 1) store_head_lo<3>(d, 1, 7 * n, col, half, lane, s_wcov, false);
+        if (wave == kWaves - 1) store_head_lo<3>(d, 1, 7 * n, col, half, lane, s_whi, false);
+        if constexpr (kColourInLds) {
+            if (wave == kWaves - 2) store_head_lo<1>(d, 2, 3 * n, col, half, lane, s_whi + 9, false);
+        }
     }
     __syncthreads();
     HeadWeights<1> w_op;
     load_head<1>(d, 0, n, col, half, w_op);
-    HeadWeights<3> w_cov = {};  // unused: read from s_wcov
-    HeadWeights<1> w_col;
-    if (!kCountOnly) load_head<1>(d, 2, 3 * n, col, half, w_col);
+    const HeadWeights<3> w_cov = {};  // unused: read from s_whi
+    HeadWeights<1> w_col = {};
+    if (!kCountOnly && !kColourInLds) load_head<1>(d, 2, 3 * n, col, half, w_col);
     const int stride = kCountOnly ? 11 : 11 * n + 13;
     const int items = 32 * n;  // (anchor, offset) pairs of a tile: item = anchor_in_tile * n + offset
     const int inv_n = (65536 + n - 1) / n;  // item / n == (item * inv_n) >> 16 for item < 32 n, n <= 10
@@ -357,27 +365,47 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (!kCountOnly
       if (v0) run_list[__popcll(m0 & lanes_below)] = (uint8_t)lane;
       if (v1) run_list[n0 + __popcll(m1 & lanes_below)] = (uint8_t)(64 + lane);
       wave_lds_sync();
+      // Everything a tile needs from global memory is requested before the first use, and without a
+      // condition: a lane without an anchor (or an item without one) reads anchor 0's data, which nothing uses
+      // (matrix columns are independent, and only items of visible anchors are ever emitted) -- conditional
+      // loads would each become a branch, and the values' first use would wait inside the condition.
+      // Features, position and level of the tile's anchors.
+      auto fetch_anchor = [&](int a, TileInputs<kCountOnly>& in) {
+        const float4* __restrict__ f4 = reinterpret_cast<const float4*>(d.feat + (size_t)a * kFeat);
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {  // features 16s + 8*half .. +7
+            in.f[2 * s] = f4[4 * s + 2 * half];
+            in.f[2 * s + 1] = f4[4 * s + 2 * half + 1];
+        }
+#pragma unroll
+        for (int k = 0; k < 3; ++k) in.pos[k] = d.anchor[3 * (size_t)a + k];
+        if (d.level) in.extra = d.level[a];
+      };
+      // The count pass has registers to spare and a run's tiles are otherwise a chain of memory latencies: it
+      // requests the next tile's inputs before it waits for the current tile's.
+      TileInputs<kCountOnly> ahead;
+      if constexpr (kCountOnly) fetch_anchor(col < nvis ? base + (int)run_list[col] : 0, ahead);
       for (int first = 0; first < nvis; first += 32) {  // dense tiles of the run
         const bool vis = first + col < nvis;  // lanes l and l+32 share entry first + l
         const int a = vis ? base + (int)run_list[first + col] : 0;
         const uint64_t any = __ballot(vis);  // bits l and l + 32 belong to entry l of the tile
-        // Everything the tile needs from global memory is requested here, before the first use, and without a
-        // condition: a lane without an anchor (or an item without one) reads anchor 0's data, which nothing uses
-        // (matrix columns are independent, and only items of visible anchors are ever emitted) -- conditional
-        // loads would each become a branch, and the values' first use would wait inside the condition.
         TileInputs<kCountOnly> in;
-        {
-            const float4* __restrict__ f4 = reinterpret_cast<const float4*>(d.feat + (size_t)a * kFeat);
+        if constexpr (kCountOnly) {
+            in = ahead;
+            if (first + 32 < nvis)  // uniform
+                fetch_anchor(first + 32 + col < nvis ? base + (int)run_list[first + 32 + col] : 0, ahead);
+        } else {
+            {  // as fetch_anchor, written out: through the lambda this pass spills three times as many registers
+                const float4* __restrict__ f4 = reinterpret_cast<const float4*>(d.feat + (size_t)a * kFeat);
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {  // features 16s + 8*half .. +7
-                in.f[2 * s] = f4[4 * s + 2 * half];
-                in.f[2 * s + 1] = f4[4 * s + 2 * half + 1];
+                for (int s = 0; s < 2; ++s) {
+                    in.f[2 * s] = f4[4 * s + 2 * half];
+                    in.f[2 * s + 1] = f4[4 * s + 2 * half + 1];
+                }
+#pragma unroll
+                for (int k = 0; k < 3; ++k) in.pos[k] = d.anchor[3 * (size_t)a + k];
+                if (d.level) in.extra = d.level[a];
             }
-#pragma unroll
-            for (int k = 0; k < 3; ++k) in.pos[k] = d.anchor[3 * (size_t)a + k];
-            if (d.level) in.extra = d.level[a];
-        }
-        if constexpr (!kCountOnly) {
             // half 0: scaling[0..2] (offset scale), half 1: scaling[3..5] (Gaussian scale)
 #pragma unroll
             for (int k = 0; k < 3; ++k) in.sc3[k] = d.scaling[6 * (size_t)a + 3 * half + k];
@@ -432,7 +460,7 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (!kCountOnly
         // ---- opacity head ----
         // the mask opacity > 0 is the sign of the pre-activation (tanh is odd, monotone and tanh(x) = x for the
         // smallest floats), so tanh itself is only evaluated for the offsets that are kept
-        run_head<1, kSplit, kWLo>(w_op, nullptr, s_wlo, lane, s_bias, s_bias + 96, X, half, mine + col * stride, 0, n);
+        run_head<1, kSplit, kWLo>(w_op, nullptr, wlo, lane, s_bias, s_bias + 96, X, half, mine + col * stride, 0, n);
         if (kCountOnly) {
             wave_lds_sync();
             if (half == 0 && vis) {
@@ -446,10 +474,10 @@ __global__ __launch_bounds__((64 * decode_waves(kCountOnly, kWLo)), (!kCountOnly
         }
 
         // ---- covariance and colour heads ----
-        run_head<3, kSplit, kWLo, true>(w_cov, s_wcov, s_wlo + (kWLo ? 5 : 0), lane, s_bias + 32, s_bias + 128, X, half,
+        run_head<3, kSplit, kWLo, true>(w_cov, whi, wlo + (kWLo ? 5 : 0), lane, s_bias + 32, s_bias + 128, X, half,
                                         mine + col * stride, n, 7 * n);
-        run_head<1, kSplit, kWLo>(w_col, nullptr, s_wlo + (kWLo ? 14 : 0), lane, s_bias + 64, s_bias + 224, X, half,
-                                  mine + col * stride, 8 * n, 3 * n);
+        run_head<1, kSplit, kWLo, kColourInLds>(w_col, whi + (kColourInLds ? 9 : 0), wlo + (kWLo ? 14 : 0), lane,
+                                                s_bias + 64, s_bias + 224, X, half, mine + col * stride, 8 * n, 3 * n);
         {
             float* __restrict__ extra = mine + col * stride + 11 * n;
 #pragma unroll

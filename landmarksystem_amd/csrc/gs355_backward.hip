@@ -139,7 +139,6 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
     const float pxf = (float)px, pyf = (float)py;
     const float x_lo0 = (float)qx0, x_hi0 = (float)(qx0 + 3), x_lo1 = (float)(qx0 + 4), x_hi1 = (float)(qx0 + 7);
     const float y_lo0 = (float)qy0, y_hi0 = (float)(qy0 + 3), y_lo1 = (float)(qy0 + 4), y_hi1 = (float)(qy0 + 7);
-    const uint64_t lanes_below = (1ull << lane) - 1ull;
 
     PixelGrad pg = {0.f, 0.f, 0.f, 0.f, 0.f};
     if (inside) {
@@ -188,22 +187,20 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(
             // ---- lists: which staged Gaussians reach which 4x4 block (lane = Gaussian), as the forward blend ----
             uint32_t len[4] = {0u, 0u, 0u, 0u};
             for (int chunk = 0; chunk < count; chunk += 64) {
-                const int k = chunk + lane;
-                bool in_x0 = false, in_x1 = false, in_y0 = false, in_y1 = false;
-                if (k < count) {
-                    const float4 a = s_a[k];
-                    const float4 c = s_c[k];
-                    const float bx_lo = a.x - c.z, bx_hi = a.x + c.z, by_lo = a.y - c.w, by_hi = a.y + c.w;
-                    in_x0 = bx_hi >= x_lo0 && bx_lo <= x_hi0;
-                    in_x1 = bx_hi >= x_lo1 && bx_lo <= x_hi1;
-                    in_y0 = by_hi >= y_lo0 && by_lo <= y_hi0;
-                    in_y1 = by_hi >= y_lo1 && by_lo <= y_hi1;
-                }
+                // lane masks straight from the comparisons, combined in scalar registers (as the forward blend)
+                const int k = chunk + lane;  // < kBatch: slots past `count` hold older records, masked by `valid`
+                const uint64_t valid = __ballot(k < count);
+                const float4 a = s_a[k];
+                const float4 c = s_c[k];
+                const float bx_lo = a.x - c.z, bx_hi = a.x + c.z, by_lo = a.y - c.w, by_hi = a.y + c.w;
+                const uint64_t in_x0 = __ballot(bx_hi >= x_lo0) & __ballot(bx_lo <= x_hi0) & valid;
+                const uint64_t in_x1 = __ballot(bx_hi >= x_lo1) & __ballot(bx_lo <= x_hi1) & valid;
+                const uint64_t in_y0 = __ballot(by_hi >= y_lo0) & __ballot(by_lo <= y_hi0);
+                const uint64_t in_y1 = __ballot(by_hi >= y_lo1) & __ballot(by_lo <= y_hi1);
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
-                    const bool reach = ((b & 1) ? in_x1 : in_x0) && ((b >> 1) ? in_y1 : in_y0);
-                    const uint64_t m = __ballot(reach);
-                    if (reach) s_list[wave][b][len[b] + (uint32_t)__popcll(m & lanes_below)] = (uint8_t)k;
+                    const uint64_t m = ((b & 1) ? in_x1 : in_x0) & ((b >> 1) ? in_y1 : in_y0);
+                    if (__builtin_amdgcn_inverse_ballot_w64(m)) s_list[wave][b][len[b] + lanes_below_in(m)] = (uint8_t)k;
                     len[b] += (uint32_t)__popcll(m);
                 }
             }

@@ -142,7 +142,6 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
     // pixel-centre bounds of the quadrant's two block columns and two block rows
     const float x_lo0 = (float)qx0, x_hi0 = (float)(qx0 + 3), x_lo1 = (float)(qx0 + 4), x_hi1 = (float)(qx0 + 7);
     const float y_lo0 = (float)qy0, y_hi0 = (float)(qy0 + 3), y_lo1 = (float)(qy0 + 4), y_hi1 = (float)(qy0 + 7);
-    const uint64_t lanes_below = (1ull << lane) - 1ull;
 
     const uint32_t lo = ranges[2 * tile], hi = ranges[2 * tile + 1];
     PixelState p = {inside ? 1.0f : -1.0f, 0.0f, 0.0f, 0.0f, 0.0f};
@@ -181,26 +180,28 @@ __global__ __launch_bounds__(256) void blend_kernel(FrameArgs f, const gs355_hea
             if (kCull) {
                 // ---- lists: which staged Gaussians reach which 4x4 block (lane = Gaussian) ----
                 uint32_t len[4] = {0u, 0u, 0u, 0u};  // uniform over the wavefront
+                // Every comparison goes straight into a lane mask (a ballot of one compare is the compare's own
+                // result register), the masks are combined in scalar registers, and a lane's rank among a mask's
+                // lanes is the hardware's masked bit count: a per-lane flag carried into a ballot costs two vector
+                // instructions more per ballot, and ranks through `mask & lanes_below` two more per rank.
                 for (int chunk = 0; chunk < count; chunk += 64) {
-                    const int k = chunk + lane;
-                    bool in_x0 = false, in_x1 = false, in_y0 = false, in_y1 = false;
-                    if (k < count) {
-                        const float4 a = s_a[k];
-                        const float4 c = s_c[k];
-                        const float bx_lo = a.x - c.z, bx_hi = a.x + c.z, by_lo = a.y - c.w, by_hi = a.y + c.w;
-                        in_x0 = bx_hi >= x_lo0 && bx_lo <= x_hi0;
-                        in_x1 = bx_hi >= x_lo1 && bx_lo <= x_hi1;
-                        in_y0 = by_hi >= y_lo0 && by_lo <= y_hi0;
-                        in_y1 = by_hi >= y_lo1 && by_lo <= y_hi1;
-                    }
+                    const int k = chunk + lane;  // < kBatch: slots past `count` hold older records, masked by `valid`
+                    const uint64_t valid = __ballot(k < count);
+                    const float4 a = s_a[k];
+                    const float4 c = s_c[k];
+                    const float bx_lo = a.x - c.z, bx_hi = a.x + c.z, by_lo = a.y - c.w, by_hi = a.y + c.w;
+                    const uint64_t in_x0 = __ballot(bx_hi >= x_lo0) & __ballot(bx_lo <= x_hi0) & valid;
+                    const uint64_t in_x1 = __ballot(bx_hi >= x_lo1) & __ballot(bx_lo <= x_hi1) & valid;
+                    const uint64_t in_y0 = __ballot(by_hi >= y_lo0) & __ballot(by_lo <= y_hi0);
+                    const uint64_t in_y1 = __ballot(by_hi >= y_lo1) & __ballot(by_lo <= y_hi1);
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
                         // a block whose 16 pixels have all finished gets no entries (its lane group idles through
                         // the null record while the other blocks of the wavefront are served)
                         if (((live >> (16 * b)) & 0xFFFFull) == 0ull) continue;
-                        const bool hit = ((b & 1) ? in_x1 : in_x0) && ((b >> 1) ? in_y1 : in_y0);
-                        const uint64_t m = __ballot(hit);
-                        if (hit) s_list[wave][b][len[b] + (uint32_t)__popcll(m & lanes_below)] = (ListEntry)(k * 16);
+                        const uint64_t m = ((b & 1) ? in_x1 : in_x0) & ((b >> 1) ? in_y1 : in_y0);
+                        if (__builtin_amdgcn_inverse_ballot_w64(m))
+                            s_list[wave][b][len[b] + lanes_below_in(m)] = (ListEntry)(k * 16);
                         len[b] += (uint32_t)__popcll(m);
                     }
                 }

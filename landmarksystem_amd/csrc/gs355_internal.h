@@ -124,6 +124,12 @@ int launch_render_backward(const FrameArgs& f, const gs355_gaussians& g, const g
                            uint32_t* first_key, uint32_t* scan_tmp, float* key_grads, const gs355_gradients& out,
                            hipStream_t s);
 
+// Number of lanes below this one that `mask` (uniform over the wavefront) holds: the hardware's masked bit count.
+__device__ __forceinline__ uint32_t lanes_below_in(uint64_t mask)
+{
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
 // Orders one wavefront's LDS writes before its later LDS reads (and the reverse).  The hardware executes a
 // wavefront's LDS instructions in order; the fences (wavefront scope: no instructions) and the scheduling
 // barrier keep the compiler from moving the accesses across this point.

@@ -550,6 +550,28 @@ def bench_trajectory(args, torch, dev):
     pairs, pairs_error = (None, None) if args.no_cpu_baseline else guarded(cpu_pair_stats, scene)
     stages, roofline = raster_report(stage_ms, stats, scene.P, inp.tiles, inp.width * inp.height,
                                      12 * scene.shs.shape[1], pairs, None)
+    # the same scene stored along a Morton curve (the checkpoint loaders' spatial_order option): the survivors'
+    # SH blocks are then neighbours in memory instead of isolated reads; same trajectory, reported beside `value`
+    ordered = None
+    if getattr(args, "spatial_leg", not args.no_model_level):
+        from landmarksystem_amd.models import morton_order
+        order = morton_order(d.means3D)
+        kw2 = {k: (v[order].contiguous() if torch.is_tensor(v) else v) for k, v in kwargs.items()}
+        del order
+        with torch.no_grad():
+            for k in range(len(poses)):
+                rast.raster_settings = poses[k]
+                rast(**kw2)
+        fps2, ms2 = frame_loop(torch, rast, kw2, 0, args.steps, settings_list=poses)
+        inp2 = pipeline.FrameInputs(poses[0], kw2["means3D"], opacities=kw2["opacities"], shs=kw2["shs"],
+                                    scales=kw2["scales"], rotations=kw2["rotations"])
+        ms_stage2, _ = stage_breakdown(torch, pipeline, _lib, inp2, n_cap, max(3, args.stage_steps // 2))
+        ordered = {"frames_per_s": round(fps2, 2), "ms_per_frame": round(ms2, 4),
+                   "preprocess_ms_pose0": round(ms_stage2["preprocess"], 4),
+                   "preprocess_ms_pose0_generated_order": round(stage_ms["preprocess"], 4),
+                   "note": "same Gaussians and poses, stored along a 3-D Morton curve; `value` is the generated "
+                           "(random) order"}
+        del kw2, inp2
     cam = scene.camera
     result = base_line("4K frames/sec at 20M Gaussians over 30 aerial poses (1 GPU)", fps, ms_per_step, args,
                        len(poses), "f32", {
@@ -560,6 +582,8 @@ def bench_trajectory(args, torch, dev):
         "stages_of": "pose 0 (%d keys, %d visible)" % (stats["num_keys"], stats["num_visible"]),
         "tiles": inp.tiles, "scene_gen_s": round(gen_s, 1)})
     result.update({"roofline": roofline, "stages": stages})
+    if ordered:
+        result["spatial_order"] = ordered
     if not args.no_cpu_baseline:
         base, err = guarded(cpu_baseline, scene, pairs)
         result["cpu_baseline"] = base if base else {"error": err}
@@ -712,7 +736,7 @@ def compact_entry(line):
     for name in ("preprocess", "keys_sort_ranges", "decode"):
         if name in stages and "frac_hbm" in stages[name]:
             keep.setdefault("frac_hbm_algorithmic", {})[name] = stages[name]["frac_hbm"]
-    for extra in ("parity", "model_variants_frames_per_s"):
+    for extra in ("parity", "model_variants_frames_per_s", "spatial_order"):
         if line.get(extra):
             keep[extra] = line[extra]
     for extra in ("keys_min_mean_max", "visible_fraction_min_max", "visible_anchors", "decoded_gaussians", "keys"):
@@ -732,7 +756,7 @@ def other_configs(args, torch, dev):
         sub = copy.copy(args)
         sub.config, sub.gaussians, sub.spatial_order, sub.two_in_flight, sub.calibration_copy = index, None, False, False, False
         sub.steps, sub.warmup, sub.stage_steps, sub.compact = steps, 10, 10, True
-        sub.no_model_level, sub.no_backward = index != 5, True
+        sub.no_model_level, sub.no_backward, sub.spatial_leg = index != 5, True, index == 4
         sub.no_cpu_baseline = index != 2  # the C checker renders the 1M-Gaussian frame in well under a second
         line, err = guarded(fn, sub, torch, dev)
         out["configs[%d]" % (index - 1)] = compact_entry(line) if line else {"error": err}

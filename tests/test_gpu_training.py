@@ -40,7 +40,7 @@ def test_differentiable_decode_matches_kernels_and_float64_gradients(gpu_device,
     if float(raw.abs().min()) > 1e-5:
         for a, b in zip(got[:5], kernels[:5]):
             assert a.shape == b.shape
-            assert float((a - b).abs().max()) <= TOL * max(1.0, float(b.abs().max()))
+            assert float((a.detach() - b).abs().max()) <= TOL * max(1.0, float(b.abs().max()))
         assert torch.equal(got[6], kernels[6])
     # gradients of a weighted sum of every output against float64 autograd through the oracle's statements
     weights = [torch.randn(t.shape, generator=g) for t in got[:5]]

@@ -115,8 +115,11 @@ def test_decode_with_weights_fp16_cannot_represent(gpu_device, A, features_too):
     assert torch.equal(dev.xyz[:G], got[0]) and torch.equal(dev.rot[:G], got[4])
 
 
-def test_decode_heads_without_distance_and_fewer_offsets(gpu_device):
-    sc = scenes.config5(A=3000, n_offsets=6)
+@pytest.mark.parametrize("n_offsets", [1, 3, 4, 6])
+def test_decode_heads_without_distance_and_fewer_offsets(gpu_device, n_offsets):
+    """Fewer offsets leave the heads' last row tiles partly or wholly beyond their outputs (one offset: 7 covariance
+    outputs in three tiles of 32 rows): the rows that do not exist must not disturb the ones that do."""
+    sc = scenes.config5(A=3000, n_offsets=n_offsets)
     mlp = dict(sc.mlp)
     w0, b0, w1, b1 = mlp["color"]
     mlp["color"] = (w0[:, :35].contiguous(), b0, w1, b1)
@@ -127,8 +130,8 @@ def test_decode_heads_without_distance_and_fewer_offsets(gpu_device):
     cam = sc.camera.camera_center
     got = dec(cam.to(gpu_device), sc.anchor.to(gpu_device), sc.anchor_feat.to(gpu_device), sc.offset.to(gpu_device),
               sc.scaling.to(gpu_device), vis.to(gpu_device))
-    redo = lambda keep=None: ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp, 6,  # noqa: E731
-                                       add_dist=(True, True, False), keep_override=keep)
+    redo = lambda keep=None: ao.decode(cam, sc.anchor, sc.anchor_feat, sc.offset, sc.scaling, vis, sc.mlp,  # noqa: E731
+                                       n_offsets, add_dist=(True, True, False), keep_override=keep)
     compare(got, redo(), redo)
 
 

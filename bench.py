@@ -40,12 +40,12 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 COUNTER_TRAFFIC = {
     "source": "profiles/bench_c3_6M_1080p_hbm_traffic.txt",
     "workload": "configs[2]",
-    "bytes": {"blend": 1844.9e6, "preprocess": 1705.8e6, "keys_sort_ranges": 824.5e6},
+    "bytes": {"blend": 1844.2e6, "preprocess": 1705.8e6, "keys_sort_ranges": 824.4e6},
     # fp32 flops the blend kernel issues per launch (64 lanes x (2 FMA + MUL + ADD) wavefront instructions), from
     # profiles/bench_c3_6M_1080p_valu_counters.txt
     "blend_issued_flops": 10.31e9,
     "blend_issued_flops_source": "profiles/bench_c3_6M_1080p_valu_counters.txt",
-    "blend_valu_busy": 0.976,
+    "blend_valu_busy": 0.957,
 }
 
 # Same for `--config 5`: HBM bytes per launch of the two decode kernels (count + emit)

@@ -462,12 +462,14 @@ def bench_vanilla(args, torch, dev):
         for _ in range(5):
             model(scene.camera)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        n_model = max(20, args.steps // 2)
-        for _ in range(n_model):
-            model(scene.camera)
-        torch.cuda.synchronize()
-        model_fps[name] = round(n_model / (time.perf_counter() - t0), 2)
+        n_model, rates = max(20, args.steps // 2), []
+        for _ in range(3):  # (the reference's sequence waits for the host every frame: median of three timings)
+            t0 = time.perf_counter()
+            for _ in range(n_model):
+                model(scene.camera)
+            torch.cuda.synchronize()
+            rates.append(n_model / (time.perf_counter() - t0))
+        model_fps[name] = round(sorted(rates)[1], 2)
         del model
 
     if args.calibration_copy:
@@ -632,11 +634,14 @@ def bench_scaffold(args, torch, dev):
         for _ in range(5):
             other(cam)
         torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        for _ in range(args.steps):
-            other(cam)
-        torch.cuda.synchronize()
-        variants[name] = round(args.steps / (time.perf_counter() - t1), 2)
+        rates = []  # these paths wait for the host every frame, and the host is a shared machine: median of three
+        for _ in range(3):
+            t1 = time.perf_counter()
+            for _ in range(args.steps):
+                other(cam)
+            torch.cuda.synchronize()
+            rates.append(args.steps / (time.perf_counter() - t1))
+        variants[name] = round(sorted(rates)[1], 2)
         del other
 
     # stages: anchor prefilter and decode alone (HIP events on the launch stream), then the rasterizer stages on the
@@ -666,7 +671,11 @@ def bench_scaffold(args, torch, dev):
         for prm, given in zip(general.parameters(), src.parameters()):
             prm.copy_(given * (1.0 + 1e-3 * torch.randn(prm.shape, generator=gen).to(dev)))
         dec32_ms, _ = timed(lambda: general(**dec_args))
-        del general
+        # and with features off the fp16 grid as well (what a trained checkpoint holds): two more matrix instructions
+        # per head for their low parts
+        feat32 = dec_args["anchor_feat"] * (1.0 + 1e-3 * torch.randn(dec_args["anchor_feat"].shape, generator=gen).to(dev))
+        dec32b_ms, _ = timed(lambda: general(**dict(dec_args, anchor_feat=feat32)))
+        del general, feat32
     xyz, color, opacity, scaling, rot = dec[:5]
     a_vis, G = int(vis.sum()), int(xyz.shape[0])
     flops = 13952 * a_vis
@@ -684,7 +693,8 @@ def bench_scaffold(args, torch, dev):
     stages["anchor_prefilter"] = {"ms": round(prefilter_ms, 4), "bytes": 36 * A,
                                   "GBps": round(36 * A / prefilter_ms / 1e6, 1),
                                   "frac_hbm": round(36 * A / prefilter_ms / 1e6 / HBM_PEAK_GBS, 4)}
-    stages["decode"] = {"ms": round(dec_ms, 4), "ms_fp32_weights": round(dec32_ms, 4), "anchors_per_s": round(a_vis / dec_ms * 1e3), "flops": flops,
+    stages["decode"] = {"ms": round(dec_ms, 4), "ms_fp32_weights": round(dec32_ms, 4),
+                        "ms_fp32_weights_and_features": round(dec32b_ms, 4), "anchors_per_s": round(a_vis / dec_ms * 1e3), "flops": flops,
                         "TFLOPs": round(flops / dec_ms / 1e9, 3),
                         "frac_mfma_f16": round(flops / dec_ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 6),
                         "bytes": dec_bytes, "GBps": round(dec_bytes / dec_ms / 1e6, 1),

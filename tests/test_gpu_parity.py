@@ -453,6 +453,39 @@ def test_full_size_config4_4k_frame_equals_the_oracle(gpu_device, config4_scene,
     assert got["num_keys"] > 10_000_000
 
 
+@pytest.fixture(scope="module")
+def config4_on_device(config4_scene, gpu_device):
+    """The 20M-Gaussian scene resident on the GPU (4.7 GB), uploaded once for the poses below."""
+    sc = config4_scene
+    return scenes.GaussianScene(sc.name, sc.means3D.to(gpu_device), sc.scales.to(gpu_device), sc.rotations.to(gpu_device),
+                                sc.opacities.to(gpu_device), sc.shs.to(gpu_device), sc.sh_degree, sc.cameras, sc.bg)
+
+
+@pytest.mark.parametrize("pose", [p for p in range(30) if p not in C4_POSES])
+def test_full_size_config4_integer_outputs_on_the_other_poses(gpu_device, config4_scene, config4_on_device, pose):
+    """The 23 poses of the trajectory whose images are not compared: radii, key count, every sorted key and value
+    and the ranges against the oracle's preprocess / duplicate / stable sort / ranges (its blend, the slow part, is
+    left out), bit for bit."""
+    scene, dev_scene = config4_scene, config4_on_device
+    print("C4 pose %d (integer outputs)" % pose, flush=True)
+    one = scenes.GaussianScene(scene.name, scene.means3D, scene.scales, scene.rotations, scene.opacities, scene.shs,
+                               scene.sh_degree, [scene.cameras[pose]], scene.bg)
+    one_dev = scenes.GaussianScene(scene.name, dev_scene.means3D, dev_scene.scales, dev_scene.rotations,
+                                   dev_scene.opacities, dev_scene.shs, scene.sh_degree, [scene.cameras[pose]], scene.bg)
+    got = run_fast_path(one_dev, gpu_device)
+    frame = oracle_frame(one)
+    pre = co.preprocess(frame, oracle_gaussians(one))
+    np.testing.assert_array_equal(got["radii"], pre["radii"])
+    offsets, total = co.scan(pre["tiles_touched"])
+    assert got["num_keys"] == total > 10_000_000
+    keys, vals = co.duplicate_keys(pre, offsets, total, frame.grid[0])
+    skeys, svals = co.sort_pairs(keys, vals)
+    np.testing.assert_array_equal(got["sorted_keys"], skeys)
+    np.testing.assert_array_equal(got["sorted_values"], svals)
+    np.testing.assert_array_equal(got["ranges"], co.tile_ranges(skeys, frame.grid[0] * frame.grid[1]))
+    assert np.isfinite(got["image"]).all() and float(got["alpha"].max()) <= 1.0
+
+
 @pytest.mark.parametrize("same,spread,label", [(1800, 0, "one depth only"), (1500, 2500, "one heavy depth among many"),
                                                 (300, 6000, "heavy depth in a class-3 bucket")])
 def test_tile_sort_fallback_on_massive_depth_ties(gpu_device, same, spread, label):

@@ -756,7 +756,7 @@ def compact_entry(line):
 
 
 def other_configs(args, torch, dev):
-    """Compact lines of the other single-GPU workloads BASELINE.json names, measured in the same run: configs[1]
+    """Compact lines of the other single-GPU workloads of the benchmark definition, measured in the same run: configs[1]
     (1M Gaussians, with its parity object), configs[3] (20M Gaussians at 4K over the 30-pose trajectory) and
     configs[4] (Scaffold-GS, 500k anchors)."""
     import copy

@@ -74,6 +74,7 @@ class _TallLinear(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, bias):
+        x = x.contiguous()
         ctx.save_for_backward(x, weight)
         return torch.addmm(bias, x, weight.t())
 

@@ -854,10 +854,9 @@ template <int kT, int kR>
 struct LdsSorter {
     static constexpr int kW = kT / 64;
     static constexpr int kCap = kT * kR;
-#ifndef GS_BINS_PER
-#define GS_BINS_PER 4
-#endif
-    static constexpr int kBinsPer = kT >= 512 ? GS_BINS_PER : 2;  // fine bins per thread of the counting pass
+    // fine bins per thread of the counting pass (measured at 1080p / 6M Gaussians, the two larger classes together:
+    // 1 / 2 / 3 / 4 bins = 0.169 / 0.155 / 0.147 / 0.145 ms)
+    static constexpr int kBinsPer = kT >= 512 ? 4 : 2;
     static constexpr int kB = kBinsPer * kT;                      // fine bins
     // counters: [kW][256] words for the radix passes, or the fine bins and 512 coarse words of the counting pass
     static constexpr int kCounterWords = kB + 512 > kW * 256 ? kB + 512 : kW * 256;

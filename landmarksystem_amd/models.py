@@ -498,11 +498,12 @@ class ScaffoldGS(nn.Module):
         return None  # Scaffold-GS anchors carry no level
 
     def forward(self, viewpoint_camera, scaling_modifier=1.0, retain_grad=False, render_exclude_filter=None):
-        """scaffold_gs/gs_model.py:162-238 (octree_gs/gs_model.py:228-325).  Under torch.no_grad() or in eval mode:
-        the frame.  In training mode with gradients enabled: `(rendered_image, scaling)` as the reference returns
-        them, differentiable with respect to the anchors' parameters and the decoder's MLPs, with
-        `viewspace_points`, `offset_selection_mask` and `opacity` left on the model for its densification."""
-        if self.training and torch.is_grad_enabled():
+        """scaffold_gs/gs_model.py:162-238 (octree_gs/gs_model.py:228-325).  In eval mode: the frame.  In training
+        mode: `(rendered_image, scaling)` as the reference returns them, with `viewspace_points`,
+        `offset_selection_mask` and `opacity` left on the model for its densification; with gradients enabled the
+        pair is differentiable with respect to the anchors' parameters and the decoder's MLPs (under torch.no_grad()
+        the same values come from the kernels)."""
+        if self.training:
             return self._forward_training(viewpoint_camera, scaling_modifier, retain_grad, render_exclude_filter)
         with torch.no_grad():
             return self._forward_frame(viewpoint_camera, scaling_modifier, render_exclude_filter)
@@ -519,7 +520,7 @@ class ScaffoldGS(nn.Module):
             offset=self.get_offset, scaling=self.get_scaling, visible_mask=voxel_visible_mask,
             level=self._decoder_level())
         screenspace_points = torch.zeros_like(xyz, requires_grad=True) + 0
-        if retain_grad:
+        if retain_grad and screenspace_points.requires_grad:  # (not under torch.no_grad())
             screenspace_points.retain_grad()
         self.renderer.raster_settings = _settings(viewpoint_camera, self.background, scaling_modifier, 1)
         rendered_image, radii, _ = self.renderer(

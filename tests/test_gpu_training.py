@@ -102,10 +102,18 @@ def test_scaffold_training_reduces_the_loss(gpu_device):
     assert model.visibility_filter.shape[0] == int(model.offset_selection_mask.sum())
     for p in train:
         assert p.grad is not None and torch.isfinite(p.grad).all()
+    # training mode without gradients: the same pair, from the kernels
+    with torch.no_grad():
+        image2, scaling2 = model(scene.camera)
+    assert not image2.requires_grad and scaling2.shape[1] == 3 and model.opacity.shape[1] == 1
+    with torch.no_grad():
+        image3, _ = model(scene.camera)
+    assert torch.equal(image2, image3)
     # eval mode afterwards is the kernels' frame again (no graph)
     model.eval()
     frame = model(scene.camera)
     assert not frame.requires_grad and frame.shape == target.shape
+    assert float((frame - image2).abs().max()) <= 2e-3  # (same parameters; offsets at the opacity threshold may differ)
 
 
 def test_octree_training_step_with_level_input_and_feature_bank(gpu_device):

@@ -53,7 +53,7 @@ def test_differentiable_decode_matches_kernels_and_float64_gradients(gpu_device,
                     ref_mlp, sc.n_offsets, add_dist=add_dist, keep_override=got[6].cpu(), dtype=torch.float64)
     ref_loss = sum((ref[k] * w.double()).sum() for k, w in zip(("xyz", "color", "opacity", "scaling", "rot"), weights))
     ref_loss.backward()
-    assert abs(float(loss) - float(ref_loss)) <= 1e-4 * abs(float(ref_loss)) + 1e-3
+    assert abs(float(loss.detach()) - float(ref_loss.detach())) <= 1e-4 * abs(float(ref_loss.detach())) + 1e-3
 
     def close(name, a, b):
         scale = float(b.abs().max())

@@ -24,7 +24,9 @@ namespace gs355 {
 
 namespace {
 
-constexpr int kInlineTiles = 32;  // splats touching more tiles than this are expanded by the whole workgroup
+// splats touching more tiles than this are queued and expanded by a wavefront each (8 and 16 measured slower, 64 and
+// 128 the same)
+constexpr int kInlineTiles = 32;
 constexpr int kBinItems = 4;      // Gaussians per thread and round of the binning walk
 
 // ---------------------------------------------------------------------------
@@ -34,7 +36,7 @@ constexpr int kBinItems = 4;      // Gaussians per thread and round of the binni
 //   more tiles (kWide):        one counter per coarse bin of kCoarseTiles consecutive tiles, matrix[c][b]; the
 //                              tiles' own totals are counted later, from the pairs of each bin (fine_count_kernel).
 // A thread walks the tile rectangle of its own Gaussian; rectangles of more than kInlineTiles tiles are queued and
-// walked by all threads together.
+// walked by the wavefronts, one rectangle each at a time.
 template <bool kWide>
 __global__ __launch_bounds__(kBinThreads) void tile_count_kernel(FrameArgs f, int32_t P, int per_group,
                                                                  const uint64_t* __restrict__ rects,
@@ -97,13 +99,15 @@ __global__ __launch_bounds__(kBinThreads) void tile_count_kernel(FrameArgs f, in
             }
         }
         __syncthreads();
+        // large rectangles: one per wavefront at a time, 64 tiles per step (the sixteen wavefronts work on sixteen
+        // rectangles side by side; the whole workgroup on one rectangle left most of its threads idle)
         const uint32_t nq = s_nqueue;
-        for (uint32_t k = 0; k < nq; ++k) {
+        for (uint32_t k = (uint32_t)tid >> 6; k < nq; k += kBinThreads / 64) {
             const uint64_t r = rects[s_queue[k]];
             const int x0 = (int)(r & 0xFFFF), y0 = (int)((r >> 16) & 0xFFFF), x1 = (int)((r >> 32) & 0xFFFF),
                       y1 = (int)(r >> 48);
             const int w = x1 - x0, area = w * (y1 - y0);
-            for (int e = tid; e < area; e += kBinThreads) add((y0 + e / w) * f.grid_x + x0 + e % w);
+            for (int e = tid & 63; e < area; e += 64) add((y0 + e / w) * f.grid_x + x0 + e % w);
         }
         __syncthreads();
     }

@@ -62,13 +62,22 @@ __global__ __launch_bounds__(kBinThreads) void tile_count_kernel(FrameArgs f, in
     uint32_t visible = 0;
     auto add = [&](int t) { atomicAdd(&s_count[kWide ? t >> kCoarseShift : t], 1u); };
 
+    // a thread's Gaussians of a round: their rectangles are requested together, and those of the next round before
+    // this round's are walked (a slice is a dozen rounds or more, each otherwise a memory latency plus its walk)
+    uint64_t ahead[kBinItems];
+#pragma unroll
+    for (int u = 0; u < kBinItems; ++u) ahead[u] = g_begin < g_end ? rects[min(g_begin + u * kBinThreads + tid, g_end - 1)] : 0ull;
     for (int base = g_begin; base < g_end; base += kBinItems * kBinThreads) {
         if (tid == 0) s_nqueue = 0;
         __syncthreads();
-        // a thread's Gaussians of this round: their rectangles are requested together
         uint64_t rr[kBinItems];
 #pragma unroll
-        for (int u = 0; u < kBinItems; ++u) rr[u] = rects[min(base + u * kBinThreads + tid, g_end - 1)];
+        for (int u = 0; u < kBinItems; ++u) rr[u] = ahead[u];
+        if (base + kBinItems * kBinThreads < g_end) {  // uniform
+#pragma unroll
+            for (int u = 0; u < kBinItems; ++u)
+                ahead[u] = rects[min(base + (kBinItems + u) * kBinThreads + tid, g_end - 1)];
+        }
 #pragma unroll
         for (int u = 0; u < kBinItems; ++u) {
             const int i = base + u * kBinThreads + tid;
@@ -1029,11 +1038,7 @@ struct LdsSorter {
         // position -> bin: floor(pos * kB / n) for n > kB, else the position itself (one pair per bin)
         const bool spread = n > (uint32_t)kB;
         const uint32_t to_bin = spread ? (uint32_t)(((uint64_t)kB << 32) / (uint64_t)n) : 0u;
-#pragma unroll
-        for (int i = 0; i < kBinsPer; ++i) count[i * kT + tid] = 0;
-        if (tid < 256) coarse[tid] = 0;
-        if (tid == 0) flags[8] = 0;
-        __syncthreads();
+        // (the counters were cleared by the caller, before the barrier that made dmin and dmax known)
         uint32_t cbin[kR], frac[kR];
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
@@ -1049,9 +1054,8 @@ struct LdsSorter {
             }
         }
         __syncthreads();
-        uint32_t csize = 0, own = 0;
         if (tid < 256) {  // exclusive scan of the coarse counts (wavefronts 0..3)
-            own = coarse[tid];
+            const uint32_t own = coarse[tid];
             uint32_t inc = own;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
@@ -1059,15 +1063,13 @@ struct LdsSorter {
                 if (lane >= d) inc += up;
             }
             if (lane == 63) flags[16 + wave] = inc;
-            csize = inc - own;  // exclusive within the wavefront
-        }
-        __syncthreads();
-        if (tid < 256) {  // (a thread replaces the one count that only it has read)
-            for (int w = 0; w < wave; ++w) csize += flags[16 + w];
-            coarse[tid] = csize;
+            // (a thread replaces the one count that only it has read) exclusive within the wavefront: the
+            // wavefronts' totals are added by whoever reads it, which saves a barrier
+            coarse[tid] = inc - own;
             coarse[256 + tid] = own;
         }
         __syncthreads();
+        const uint32_t before1 = flags[16], before2 = before1 + flags[17], before3 = before2 + flags[18];
         uint32_t bin[kR], slot[kR];
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
@@ -1075,7 +1077,9 @@ struct LdsSorter {
             bin[r] = 0;
             slot[r] = 0;
             if (j < n) {
-                const uint32_t pos = coarse[cbin[r]] + __umulhi(frac[r], coarse[256 + cbin[r]]);  // in [0, n)
+                const uint32_t cb = cbin[r];
+                const uint32_t before = cb >= 192u ? before3 : cb >= 128u ? before2 : cb >= 64u ? before1 : 0u;
+                const uint32_t pos = coarse[cb] + before + __umulhi(frac[r], coarse[256 + cb]);  // in [0, n)
                 bin[r] = min(spread ? __umulhi(pos, to_bin) : pos, (uint32_t)kB - 1u);
                 slot[r] = atomicAdd(&count[bin[r]], 1u);
             }
@@ -1206,6 +1210,13 @@ struct LdsSorter {
             atomicAnd(&flags[14], all);
             atomicMin(&flags[12], dmin);
             atomicMax(&flags[13], dmax);
+        }
+        {  // the counting sort's counters, cleared here so that it needs no barrier of its own for it
+            uint32_t* const count = &cnt[0][0];
+#pragma unroll
+            for (int i = 0; i < kBinsPer; ++i) count[i * kT + threadIdx.x] = 0;
+            if (threadIdx.x < 256) count[kB + threadIdx.x] = 0;
+            if (threadIdx.x == 0) flags[8] = 0;
         }
         __syncthreads();
         int cur = bucket_sort(n, flags[12], flags[13]);
